@@ -1,0 +1,268 @@
+"""ctypes access to the C ABI of ``libeppgcn_hip.so`` with torch tensors as device memory.
+
+This is the thinnest possible host layer: torch only provides allocations and the
+current HIP stream; every computation happens in the library.  Loading fails loudly
+when the library has not been built - there is no fallback implementation.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libeppgcn_hip.so")
+
+EXPORTS = [
+    "eppgcn_last_error", "eppgcn_abi_version", "eppgcn_spmm_forward", "eppgcn_spmm_backward",
+    "eppgcn_ours_backward", "eppgcn_mask_forward", "eppgcn_compact_workspace_bytes",
+    "eppgcn_split_workspace_bytes", "eppgcn_compact_back_edge", "eppgcn_count_nonzero",
+    "eppgcn_map_back_part_size", "eppgcn_threshold_back_part_size", "eppgcn_split_back_part",
+    "eppgcn_build_part", "eppgcn_get_ginfo", "eppgcn_set_timing", "eppgcn_print_time",
+    "eppgcn_clear_time", "eppgcn_get_time_ms", "eppgcn_set_team_size",
+]
+
+_lib = None
+
+
+class EppgcnError(RuntimeError):
+    pass
+
+
+def load():
+    """Loads the shared library (once).  Raises if it is missing: build it with
+    ``python -m eppgcn_amd.build``."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise EppgcnError(f"{LIB_PATH} is missing; run `python -m eppgcn_amd.build` (needs hipcc)")
+    lib = C.CDLL(LIB_PATH)
+    p, i, i64, sz = C.c_void_p, C.c_int, C.c_int64, C.c_size_t
+    lib.eppgcn_last_error.restype = C.c_char_p
+    lib.eppgcn_abi_version.restype = i
+    lib.eppgcn_spmm_forward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p]
+    lib.eppgcn_spmm_backward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p]
+    lib.eppgcn_ours_backward.argtypes = [p, p, p, p, p, p, i, i, i, i, i, i, i, p]
+    lib.eppgcn_mask_forward.argtypes = [p, p, p, p, p, p, p, i, i64, i, i, i, p]
+    lib.eppgcn_compact_workspace_bytes.argtypes = [i64]
+    lib.eppgcn_compact_workspace_bytes.restype = sz
+    lib.eppgcn_split_workspace_bytes.argtypes = [i64]
+    lib.eppgcn_split_workspace_bytes.restype = sz
+    lib.eppgcn_compact_back_edge.argtypes = [p, p, p, p, i64, p, sz, p, C.POINTER(i64), p]
+    lib.eppgcn_count_nonzero.argtypes = [p, i64, p, C.POINTER(i64), p]
+    lib.eppgcn_map_back_part_size.argtypes = [i64, i64, C.POINTER(i)]
+    lib.eppgcn_threshold_back_part_size.argtypes = [i64, i64]
+    lib.eppgcn_split_back_part.argtypes = [p, i, i, p, i64, p, sz, p, C.POINTER(i64), C.POINTER(i64), p]
+    lib.eppgcn_build_part.argtypes = [p, i, i, p, p, i64, p, sz, p, C.POINTER(i64), p]
+    lib.eppgcn_get_ginfo.argtypes = [p, i64, i64, p, C.POINTER(C.c_float), p]
+    lib.eppgcn_set_timing.argtypes = [i]
+    lib.eppgcn_set_timing.restype = None
+    lib.eppgcn_print_time.restype = None
+    lib.eppgcn_clear_time.restype = None
+    lib.eppgcn_get_time_ms.argtypes = [i]
+    lib.eppgcn_get_time_ms.restype = C.c_double
+    lib.eppgcn_set_team_size.argtypes = [i]
+    lib.eppgcn_set_team_size.restype = None
+    for name in ("eppgcn_spmm_forward", "eppgcn_spmm_backward", "eppgcn_ours_backward", "eppgcn_mask_forward",
+                 "eppgcn_compact_back_edge", "eppgcn_count_nonzero", "eppgcn_map_back_part_size",
+                 "eppgcn_threshold_back_part_size", "eppgcn_split_back_part", "eppgcn_build_part",
+                 "eppgcn_get_ginfo"):
+        getattr(lib, name).restype = i
+    _lib = lib
+    return lib
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise EppgcnError(f"libeppgcn_hip error {rc}: {load().eppgcn_last_error().decode()}")
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(t, dtype, name):
+    if not t.is_cuda:
+        raise EppgcnError(f"{name} must be a device tensor")
+    if t.dtype != dtype:
+        raise EppgcnError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise EppgcnError(f"{name} must be contiguous")
+    return t
+
+
+def _mask_bytes(t, name):
+    if t is None or t.numel() == 0:
+        return None
+    if t.dtype not in (torch.bool, torch.uint8):
+        raise EppgcnError(f"{name} must be bool or uint8")
+    if not t.is_cuda or not t.is_contiguous():
+        raise EppgcnError(f"{name} must be a contiguous device tensor")
+    return t
+
+
+# --------------------------------------------------------------------------- aggregation
+def spmm_forward(feats, column_index, degrees, part_ptr, part2node, part_size=32, dim_worker=32,
+                 warp_per_block=8, row_pointers=None, out=None, backward=False):
+    """out[N, D] = neighbour-group aggregation of feats (``backward=True`` uses the unpruned
+    backward entry point; same operator)."""
+    lib = load()
+    _dev(feats, torch.float32, "feats"); _dev(column_index, torch.int32, "column_index")
+    _dev(degrees, torch.float32, "degrees"); _dev(part_ptr, torch.int32, "part_ptr")
+    _dev(part2node, torch.int32, "part2node")
+    n, dim = feats.shape
+    num_parts = part2node.numel()
+    if part_ptr.numel() < num_parts + 1:
+        raise EppgcnError("part_ptr needs num_parts + 1 entries")
+    if degrees.numel() != n:
+        raise EppgcnError("degrees must have one entry per vertex")
+    if out is None:
+        out = torch.empty_like(feats)
+    fn = lib.eppgcn_spmm_backward if backward else lib.eppgcn_spmm_forward
+    _check(fn(_ptr(out), _ptr(feats), _ptr(row_pointers), _ptr(column_index), _ptr(degrees), _ptr(part_ptr),
+              _ptr(part2node), n, dim, num_parts, part_size, dim_worker, warp_per_block, _stream()))
+    return out
+
+
+def ours_backward(d_output, ids, part_pointer, edge_list, degrees, num_parts, part_size=32, layer=1,
+                  blockx=4, blocky=16, out=None):
+    lib = load()
+    _dev(d_output, torch.float32, "d_output"); _dev(ids, torch.int32, "ids")
+    _dev(part_pointer, torch.int32, "part_pointer"); _dev(edge_list, torch.int32, "edge_list")
+    _dev(degrees, torch.float32, "degrees")
+    n, dim = d_output.shape
+    if part_pointer.numel() < num_parts + 1:
+        raise EppgcnError("part_pointer needs num_parts + 1 entries")
+    if out is None:
+        out = torch.empty_like(d_output)
+    _check(lib.eppgcn_ours_backward(_ptr(out), _ptr(d_output), _ptr(ids), _ptr(part_pointer), _ptr(edge_list),
+                                    _ptr(degrees), n, dim, int(num_parts), part_size, layer, blockx, blocky,
+                                    _stream()))
+    return out
+
+
+# --------------------------------------------------------------------------- preparation
+def mask_forward(part2node, part_ptr, column_index, src_mask, ngh_mask, back_edge_mask, node_degs,
+                 is_last_layer: bool, blockx=4, blocky=16):
+    lib = load()
+    _dev(part2node, torch.int32, "part2node"); _dev(part_ptr, torch.int32, "part_ptr")
+    _dev(column_index, torch.int32, "column_index"); _dev(back_edge_mask, torch.int32, "back_edge_mask")
+    _dev(node_degs, torch.int32, "node_degs")
+    src = _mask_bytes(src_mask, "src_mask")
+    ngh = _mask_bytes(ngh_mask, "ngh_mask")
+    if src is None:
+        raise EppgcnError("src_mask must not be empty")
+    _check(lib.eppgcn_mask_forward(_ptr(part2node), _ptr(part_ptr), _ptr(column_index), _ptr(src), _ptr(ngh),
+                                   _ptr(back_edge_mask), _ptr(node_degs), part2node.numel(),
+                                   column_index.numel(), int(bool(is_last_layer)), blockx, blocky, _stream()))
+
+
+def _workspace(nbytes: int, device):
+    return torch.empty((nbytes + 7) // 8, dtype=torch.int64, device=device)
+
+
+def compact_back_edge(edge_mask, column_index):
+    """-> (id int32[E], edge_list int32[E], valid_len int)"""
+    lib = load()
+    _dev(edge_mask, torch.int32, "edge_mask"); _dev(column_index, torch.int32, "column_index")
+    length = edge_mask.numel()
+    if column_index.numel() < length:
+        raise EppgcnError("column_index is shorter than edge_mask")
+    out_id = torch.empty_like(edge_mask)
+    out_edge = torch.empty(length, dtype=torch.int32, device=edge_mask.device)
+    nbytes = lib.eppgcn_compact_workspace_bytes(length)
+    ws = _workspace(nbytes, edge_mask.device)
+    v = C.c_int64(0)
+    _check(lib.eppgcn_compact_back_edge(_ptr(edge_mask), _ptr(column_index), _ptr(out_id), _ptr(out_edge), length,
+                                        _ptr(ws), nbytes, None, C.byref(v), _stream()))
+    return out_id, out_edge, int(v.value)
+
+
+def count_nonzero(node_deg) -> int:
+    lib = load()
+    _dev(node_deg, torch.int32, "node_deg")
+    d = torch.empty(1, dtype=torch.int32, device=node_deg.device)
+    v = C.c_int64(0)
+    _check(lib.eppgcn_count_nonzero(_ptr(node_deg), node_deg.numel(), _ptr(d), C.byref(v), _stream()))
+    return int(v.value)
+
+
+def map_back_part_size(valid_node: int, valid_len: int):
+    """-> (group size >= 1, clamped flag)"""
+    c = C.c_int(0)
+    ps = load().eppgcn_map_back_part_size(int(valid_node), int(valid_len), C.byref(c))
+    return int(ps), bool(c.value)
+
+
+def threshold_back_part_size(valid_node: int, valid_len: int) -> int:
+    return int(load().eppgcn_threshold_back_part_size(int(valid_node), int(valid_len)))
+
+
+def split_back_part(node_deg, num_edges: int, part_size: int):
+    """-> (part_pointer int32[num_edges + 1], num_parts int, valid_len int)"""
+    lib = load()
+    _dev(node_deg, torch.int32, "node_deg")
+    n = node_deg.numel()
+    capacity = int(num_edges) + 1
+    part_pointer = torch.empty(capacity, dtype=torch.int32, device=node_deg.device)
+    nbytes = lib.eppgcn_split_workspace_bytes(n)
+    ws = _workspace(nbytes, node_deg.device)
+    p, v = C.c_int64(0), C.c_int64(0)
+    _check(lib.eppgcn_split_back_part(_ptr(node_deg), n, int(part_size), _ptr(part_pointer), capacity, _ptr(ws),
+                                      nbytes, None, C.byref(p), C.byref(v), _stream()))
+    return part_pointer, int(p.value), int(v.value)
+
+
+def build_part(part_size: int, row_pointers, num_edges: int = None):
+    """Device build of the forward groups -> (part_ptr int32[P+1], part2node int32[P])"""
+    lib = load()
+    _dev(row_pointers, torch.int32, "row_pointers")
+    n = row_pointers.numel() - 1
+    if num_edges is None:
+        num_edges = int(row_pointers[-1].item()) - int(row_pointers[0].item())
+    capacity = num_edges // int(part_size) + n + 1
+    part_ptr = torch.empty(capacity, dtype=torch.int32, device=row_pointers.device)
+    part2node = torch.empty(max(capacity - 1, 1), dtype=torch.int32, device=row_pointers.device)
+    nbytes = lib.eppgcn_split_workspace_bytes(n)
+    ws = _workspace(nbytes, row_pointers.device)
+    p = C.c_int64(0)
+    _check(lib.eppgcn_build_part(_ptr(row_pointers), n, int(part_size), _ptr(part_ptr), _ptr(part2node), capacity,
+                                 _ptr(ws), nbytes, None, C.byref(p), _stream()))
+    np_ = int(p.value)
+    return part_ptr[: np_ + 1], part2node[:np_]
+
+
+def get_ginfo(node_deg, valid_len: int):
+    lib = load()
+    _dev(node_deg, torch.int32, "node_deg")
+    hist = torch.empty(10, dtype=torch.int32, device=node_deg.device)
+    out = (C.c_float * 10)()
+    _check(lib.eppgcn_get_ginfo(_ptr(node_deg), node_deg.numel(), int(valid_len), _ptr(hist), out, _stream()))
+    return torch.tensor(list(out), dtype=torch.float32)
+
+
+# --------------------------------------------------------------------------- timers / tuning
+def set_timing(enabled: bool):
+    load().eppgcn_set_timing(int(bool(enabled)))
+
+
+def print_time():
+    load().eppgcn_print_time()
+
+
+def clear_time():
+    load().eppgcn_clear_time()
+
+
+def get_time_ms(which: int) -> float:
+    return float(load().eppgcn_get_time_ms(which))
+
+
+def set_team_size(lanes: int):
+    load().eppgcn_set_team_size(int(lanes))

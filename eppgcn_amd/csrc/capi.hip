@@ -1,0 +1,326 @@
+// extern "C" entry points of libeppgcn_hip.so: argument checks, timers and the
+// host halves (count read-back, heuristics) of the aggregation path.
+#include "../../include/eppgcn_hip.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+
+#include "common.hpp"
+
+namespace eppgcn {
+
+// ---- implemented in aggregate.hip / prepare.hip
+int aggregate_forward_groups(float*, const float*, const int*, const float*, const int*, const int*, int, int, int,
+                             hipStream_t);
+int aggregate_compacted_groups(float*, const float*, const int*, const int*, const int*, const float*, int, int, int,
+                               hipStream_t);
+void set_agg_force_team(int);
+size_t compact_workspace_bytes(long long);
+size_t split_workspace_bytes(long long);
+int launch_mask_forward(const int*, const int*, const int*, const uint8_t*, uint8_t*, int*, int*, int, long long, int,
+                        hipStream_t);
+int launch_compact_mask(const int*, int*, const int*, int*, long long, void*, hipStream_t);
+int launch_split(bool, const int*, int, int, int*, int*, long long, bool, void*, hipStream_t);
+int launch_count_nonzero(const int*, long long, int*, hipStream_t);
+int launch_ginfo_hist(const int*, long long, int*, hipStream_t);
+
+// ---- errors
+static thread_local std::string g_last_error;
+void set_error(const std::string& msg) { g_last_error = msg; }
+int hip_fail(hipError_t e, const char* what)
+{
+    g_last_error = std::string(what) + ": " + hipGetErrorString(e);
+    return kErrHip;
+}
+
+// ---- timers (milliseconds)
+constexpr int kMaxTimedLayers = 16;
+static bool g_timing = false;
+static double g_for_agg_ms = 0.0, g_back_agg_ms = 0.0, g_mask_ms = 0.0;
+static double g_layer_back_ms[kMaxTimedLayers] = {0};
+
+struct ScopedTimer {
+    hipStream_t stream;
+    double* sink;
+    double* sink2;
+    hipEvent_t start = nullptr, stop = nullptr;
+    ScopedTimer(hipStream_t s, double* a, double* b = nullptr) : stream(s), sink(a), sink2(b)
+    {
+        if (!g_timing) return;
+        if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) { start = nullptr; return; }
+        (void)hipEventRecord(start, stream);
+    }
+    ~ScopedTimer()
+    {
+        if (!start) return;
+        float ms = 0.f;
+        if (hipEventRecord(stop, stream) == hipSuccess && hipEventSynchronize(stop) == hipSuccess &&
+            hipEventElapsedTime(&ms, start, stop) == hipSuccess) {
+            *sink += ms;
+            if (sink2) *sink2 += ms;
+        }
+        (void)hipEventDestroy(start);
+        (void)hipEventDestroy(stop);
+    }
+};
+
+static int read_state(void* workspace, hipStream_t stream, ScanState* host)
+{
+    EPPGCN_HIP(hipMemcpyAsync(host, workspace, sizeof(ScanState), hipMemcpyDeviceToHost, stream));
+    EPPGCN_HIP(hipStreamSynchronize(stream));
+    if (host->error) {
+        set_error("look-back scan stalled: a tile waited past its spin limit; results are invalid");
+        return kErrScanStalled;
+    }
+    return kOk;
+}
+
+static bool aligned(const void* p, size_t a) { return reinterpret_cast<uintptr_t>(p) % a == 0; }
+
+}  // namespace eppgcn
+
+using namespace eppgcn;
+
+extern "C" {
+
+const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
+int eppgcn_abi_version(void) { return 1; }
+
+int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
+                        const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
+                        int dim, int num_parts, int part_size, int dim_worker, int warp_per_block, void* stream)
+{
+    (void)row_pointers;
+    EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
+    EPPGCN_REQUIRE(part_size > 0 && dim_worker > 0 && warp_per_block > 0, "launch hints must be positive");
+    if (num_nodes == 0) return kOk;
+    EPPGCN_REQUIRE(out && in && degrees, "null feature or scale pointer");
+    EPPGCN_REQUIRE(num_parts == 0 || (column_index && part_pointers && part2node), "null index pointer");
+    EPPGCN_REQUIRE(aligned(out, 4) && aligned(in, 4), "feature pointers must be 4-byte aligned");
+    ScopedTimer t(static_cast<hipStream_t>(stream), &g_for_agg_ms);
+    return aggregate_forward_groups(out, in, column_index, degrees, part_pointers, part2node, num_nodes, dim, num_parts,
+                                    static_cast<hipStream_t>(stream));
+}
+
+int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* row_pointers,
+                         const int32_t* column_index, const float* degrees, const int32_t* part_pointers,
+                         const int32_t* part2node, int num_nodes, int dim, int num_parts, int part_size, int dim_worker,
+                         int warp_per_block, void* stream)
+{
+    (void)row_pointers;
+    EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
+    EPPGCN_REQUIRE(part_size > 0 && dim_worker > 0 && warp_per_block > 0, "launch hints must be positive");
+    if (num_nodes == 0) return kOk;
+    EPPGCN_REQUIRE(d_input && d_output && degrees, "null feature or scale pointer");
+    EPPGCN_REQUIRE(num_parts == 0 || (column_index && part_pointers && part2node), "null index pointer");
+    EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
+    ScopedTimer t(static_cast<hipStream_t>(stream), &g_back_agg_ms);
+    return aggregate_forward_groups(d_input, d_output, column_index, degrees, part_pointers, part2node, num_nodes, dim,
+                                    num_parts, static_cast<hipStream_t>(stream));
+}
+
+int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
+                         const int32_t* edge_list, const float* degrees, int num_nodes, int dim, int num_parts,
+                         int part_size, int layer, int blockx, int blocky, void* stream)
+{
+    (void)part_size;   // the reference's kernel ignores it too (EPPGCN_kernel.cu:636)
+    EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
+    EPPGCN_REQUIRE(blockx > 0 && blocky > 0, "launch hints must be positive");
+    EPPGCN_REQUIRE(layer >= 1, "layer is 1-based");
+    if (num_nodes == 0) return kOk;
+    EPPGCN_REQUIRE(d_input && d_output && degrees, "null feature or scale pointer");
+    EPPGCN_REQUIRE(num_parts == 0 || (ids && part_pointer && edge_list), "null index pointer");
+    EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
+    ScopedTimer t(static_cast<hipStream_t>(stream), &g_back_agg_ms,
+                  layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr);
+    return aggregate_compacted_groups(d_input, d_output, ids, part_pointer, edge_list, degrees, num_nodes, dim,
+                                      num_parts, static_cast<hipStream_t>(stream));
+}
+
+int eppgcn_mask_forward(const int32_t* part2node, const int32_t* part_pointers, const int32_t* column_index,
+                        const uint8_t* src_mask, uint8_t* ngh_mask, int32_t* back_edge_mask, int32_t* node_degs,
+                        int num_parts, int64_t num_edges, int is_last_layer, int blockx, int blocky, void* stream)
+{
+    EPPGCN_REQUIRE(num_parts >= 0 && num_edges >= 0, "negative size");
+    EPPGCN_REQUIRE(blockx > 0 && blocky > 0, "launch hints must be positive");
+    if (num_parts == 0) return kOk;
+    EPPGCN_REQUIRE(part2node && part_pointers && column_index && src_mask && back_edge_mask && node_degs,
+                   "null pointer");
+    EPPGCN_REQUIRE(is_last_layer || ngh_mask, "ngh_mask may only be NULL on the last layer");
+    ScopedTimer t(static_cast<hipStream_t>(stream), &g_mask_ms);
+    return launch_mask_forward(part2node, part_pointers, column_index, src_mask, ngh_mask, back_edge_mask, node_degs,
+                               num_parts, num_edges, is_last_layer ? 1 : 0, static_cast<hipStream_t>(stream));
+}
+
+size_t eppgcn_compact_workspace_bytes(int64_t length) { return compact_workspace_bytes(length < 0 ? 0 : length); }
+size_t eppgcn_split_workspace_bytes(int64_t num_nodes) { return split_workspace_bytes(num_nodes < 0 ? 0 : num_nodes); }
+
+int eppgcn_compact_back_edge(const int32_t* edge_mask, const int32_t* column_index, int32_t* out_id, int32_t* out_edge,
+                             int64_t length, void* workspace, size_t workspace_bytes, int32_t* d_valid_len,
+                             int64_t* h_valid_len, void* stream)
+{
+    EPPGCN_REQUIRE(length >= 0 && length < (1ll << 31), "length must fit int32");
+    EPPGCN_REQUIRE(workspace && aligned(workspace, 8), "workspace must be 8-byte aligned");
+    EPPGCN_REQUIRE(workspace_bytes >= compact_workspace_bytes(length), "workspace too small");
+    EPPGCN_REQUIRE(length == 0 || (edge_mask && column_index && out_id && out_edge), "null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (int rc = launch_compact_mask(edge_mask, out_id, column_index, out_edge, length, workspace, s)) return rc;
+    ScanState* st = static_cast<ScanState*>(workspace);
+    if (d_valid_len)
+        EPPGCN_HIP(hipMemcpyAsync(d_valid_len, st->counts, sizeof(int), hipMemcpyDeviceToDevice, s));
+    if (h_valid_len) {
+        ScanState host;
+        if (int rc = read_state(workspace, s, &host)) return rc;
+        *h_valid_len = host.counts[0];
+    }
+    return kOk;
+}
+
+int eppgcn_count_nonzero(const int32_t* node_deg, int64_t length, int32_t* d_count, int64_t* h_count, void* stream)
+{
+    EPPGCN_REQUIRE(length >= 0 && length < (1ll << 31), "length must fit int32");
+    EPPGCN_REQUIRE(d_count && (length == 0 || node_deg), "null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (int rc = launch_count_nonzero(node_deg, length, d_count, s)) return rc;
+    if (h_count) {
+        int v = 0;
+        EPPGCN_HIP(hipMemcpyAsync(&v, d_count, sizeof(int), hipMemcpyDeviceToHost, s));
+        EPPGCN_HIP(hipStreamSynchronize(s));
+        *h_count = v;
+    }
+    return kOk;
+}
+
+int eppgcn_map_back_part_size(int64_t valid_node, int64_t valid_len, int* clamped)
+{
+    if (clamped) *clamped = 0;
+    if (valid_node <= 0) {
+        if (clamped) *clamped = 1;
+        return 1;
+    }
+    const double valid_degree = 1.0 * static_cast<double>(valid_len) / static_cast<double>(valid_node);
+    const double beta0 = 0.65538, beta1 = 1.67431e-5, beta2 = -2.24342e-6, beta3 = 0.63641;
+    const double raw = std::round(beta0 + beta1 * static_cast<double>(valid_node) +
+                                  beta2 * static_cast<double>(valid_len) + beta3 * valid_degree);
+    if (raw < 1.0) {
+        if (clamped) *clamped = 1;
+        return 1;
+    }
+    return static_cast<int>(raw);
+}
+
+int eppgcn_threshold_back_part_size(int64_t valid_node, int64_t valid_len)
+{
+    if (valid_node <= 0) return 4;
+    const int64_t valid_degree = valid_len / valid_node;
+    if (valid_degree < 4) return 4;
+    if (valid_degree < 16) return 8;
+    if (valid_degree < 64) return 16;
+    if (valid_degree < 256) return 32;
+    if (valid_degree < 512) return 64;
+    return 0;
+}
+
+static int finish_split(void* workspace, hipStream_t s, int32_t* d_counts, int64_t* h_a, int64_t* h_b)
+{
+    ScanState* st = static_cast<ScanState*>(workspace);
+    if (d_counts) EPPGCN_HIP(hipMemcpyAsync(d_counts, st->counts, 2 * sizeof(int), hipMemcpyDeviceToDevice, s));
+    if (h_a || h_b) {
+        ScanState host;
+        if (int rc = read_state(workspace, s, &host)) return rc;
+        if (h_a) *h_a = host.counts[0];
+        if (h_b) *h_b = host.counts[1];
+        if (host.overflow) {
+            set_error("group pointers do not fit the given capacity (need " + std::to_string(host.counts[0] + 1) +
+                      " entries)");
+            return kErrCapacity;
+        }
+    }
+    return kOk;
+}
+
+int eppgcn_split_back_part(const int32_t* node_deg, int num_nodes, int part_size, int32_t* part_pointer,
+                           int64_t capacity, void* workspace, size_t workspace_bytes, int32_t* d_counts,
+                           int64_t* h_num_parts, int64_t* h_valid_len, void* stream)
+{
+    EPPGCN_REQUIRE(num_nodes >= 0 && part_size >= 1, "num_nodes >= 0 and part_size >= 1 required");
+    EPPGCN_REQUIRE(capacity >= 1 && part_pointer, "part_pointer needs at least one entry");
+    EPPGCN_REQUIRE(workspace && aligned(workspace, 8), "workspace must be 8-byte aligned");
+    EPPGCN_REQUIRE(workspace_bytes >= split_workspace_bytes(num_nodes), "workspace too small");
+    EPPGCN_REQUIRE(num_nodes == 0 || node_deg, "null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (int rc = launch_split(false, node_deg, num_nodes, part_size, part_pointer, nullptr, capacity, true, workspace, s))
+        return rc;
+    return finish_split(workspace, s, d_counts, h_num_parts, h_valid_len);
+}
+
+int eppgcn_build_part(const int32_t* row_pointers, int num_nodes, int part_size, int32_t* part_pointers,
+                      int32_t* part2node, int64_t capacity, void* workspace, size_t workspace_bytes, int32_t* d_counts,
+                      int64_t* h_num_parts, void* stream)
+{
+    EPPGCN_REQUIRE(num_nodes >= 0 && part_size >= 1, "num_nodes >= 0 and part_size >= 1 required");
+    EPPGCN_REQUIRE(capacity >= 1 && part_pointers && (capacity == 1 || part2node), "output buffers required");
+    EPPGCN_REQUIRE(workspace && aligned(workspace, 8), "workspace must be 8-byte aligned");
+    EPPGCN_REQUIRE(workspace_bytes >= split_workspace_bytes(num_nodes), "workspace too small");
+    EPPGCN_REQUIRE(row_pointers, "null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (int rc = launch_split(true, row_pointers, num_nodes, part_size, part_pointers, part2node, capacity, false,
+                              workspace, s))
+        return rc;
+    return finish_split(workspace, s, d_counts, h_num_parts, nullptr);
+}
+
+int eppgcn_get_ginfo(const int32_t* node_deg, int64_t num_nodes, int64_t valid_len, int32_t* d_hist, float* h_out,
+                     void* stream)
+{
+    EPPGCN_REQUIRE(num_nodes >= 0 && num_nodes < (1ll << 31), "num_nodes must fit int32");
+    EPPGCN_REQUIRE(d_hist && h_out && (num_nodes == 0 || node_deg), "null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (int rc = launch_ginfo_hist(node_deg, num_nodes, d_hist, s)) return rc;
+    int hist[10];
+    EPPGCN_HIP(hipMemcpyAsync(hist, d_hist, sizeof(hist), hipMemcpyDeviceToHost, s));
+    EPPGCN_HIP(hipStreamSynchronize(s));
+    // same expressions as the reference: float counts, double divisions, float32 results
+    const int valid_node = hist[0];
+    h_out[0] = static_cast<float>(valid_node * 1.0 / 10000);
+    h_out[1] = static_cast<float>(valid_len * 1.0 / 10000);
+    h_out[2] = static_cast<float>(1.0 * valid_len / valid_node);
+    for (int i = 3; i < 10; ++i) h_out[i] = static_cast<float>(static_cast<float>(hist[i]) * 1.0 / valid_node);
+    return kOk;
+}
+
+void eppgcn_set_timing(int enabled) { g_timing = enabled != 0; }
+
+void eppgcn_print_time(void)
+{
+    // same lines as the reference's print_time (EPPGCN_kernel.cu:96-106), in seconds
+    std::printf("for_agg_time: %.6f\n", g_for_agg_ms / 1000);
+    std::printf("back_agg_time: %.6f\n", g_back_agg_ms / 1000);
+    for (int i = 0; i < kMaxTimedLayers && g_layer_back_ms[i] != 0.0; ++i)
+        std::printf("l%d_back_agg_time: %.6f\n", i + 1, g_layer_back_ms[i] / 1000);
+    std::printf("mask_time: %.6f\n", g_mask_ms / 1000);
+    std::fflush(stdout);
+}
+
+void eppgcn_clear_time(void)
+{
+    // the marking time survives a clear, as in the reference (EPPGCN_kernel.cu:108-116): marking
+    // runs once during warm-up and is still reported after the timed epochs
+    g_for_agg_ms = 0.0;
+    g_back_agg_ms = 0.0;
+    for (double& v : g_layer_back_ms) v = 0.0;
+}
+
+double eppgcn_get_time_ms(int which)
+{
+    if (which == 0) return g_for_agg_ms;
+    if (which == 1) return g_back_agg_ms;
+    if (which == 2) return g_mask_ms;
+    if (which > 100 && which <= 100 + kMaxTimedLayers) return g_layer_back_ms[which - 101];
+    return -1.0;
+}
+
+void eppgcn_set_team_size(int lanes) { set_agg_force_team(lanes); }
+
+}  // extern "C"

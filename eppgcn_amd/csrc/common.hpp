@@ -1,0 +1,200 @@
+// Shared device helpers for the gfx950 (CDNA4, wave64) kernels of the GCN
+// aggregation path: cross-lane primitives, the decoupled look-back tile
+// protocol, and host-side error plumbing.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+namespace eppgcn {
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------- host errors
+// Every C entry point returns 0 on success or a negative code and leaves a
+// message readable through eppgcn_last_error().
+enum : int {
+    kOk = 0,
+    kErrInvalidArgument = -1,
+    kErrHip = -2,
+    kErrScanStalled = -3,   // a look-back wait exceeded its spin limit
+    kErrCapacity = -4,      // an output buffer was too small for the result
+};
+
+void set_error(const std::string& msg);
+int hip_fail(hipError_t e, const char* what);
+
+#define EPPGCN_HIP(expr)                                        \
+    do {                                                        \
+        hipError_t _e = (expr);                                 \
+        if (_e != hipSuccess) return ::eppgcn::hip_fail(_e, #expr); \
+    } while (0)
+
+#define EPPGCN_REQUIRE(cond, msg)                               \
+    do {                                                        \
+        if (!(cond)) {                                          \
+            ::eppgcn::set_error(std::string(__func__) + ": " + (msg)); \
+            return ::eppgcn::kErrInvalidArgument;               \
+        }                                                       \
+    } while (0)
+
+// ---------------------------------------------------------------- lane helpers
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+// Number of set ballot bits strictly below this lane (rank of the lane among the
+// lanes whose predicate held).
+__device__ __forceinline__ int ballot_rank(uint64_t ballot)
+{
+    return __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(ballot >> 32),
+                                     __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(ballot), 0u));
+}
+
+// DPP controls (GFX9 encoding): row_ror:n rotates within a row of 16 lanes.
+constexpr int kDppRowRor4 = 0x124;
+constexpr int kDppRowRor8 = 0x128;
+constexpr int kDppQuadXor1 = 0xB1;   // quad_perm [1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;   // quad_perm [2,3,0,1]
+
+template <int kCtrl>
+__device__ __forceinline__ float dpp_f32(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xF, 0xF, false));
+}
+
+// value of lane (l ^ 16) inside each half of 32 lanes: ds_swizzle bit-mask mode,
+// and_mask = 0x1F, or_mask = 0, xor_mask = 0x10.
+__device__ __forceinline__ float swizzle_xor16(float v)
+{
+    return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));
+}
+
+// Sum of v over the lanes that hold the same position inside their team, for
+// teams of kTeam consecutive lanes: afterwards every lane holds the total of the
+// 64/kTeam lanes congruent to it modulo kTeam.  Offsets below 16 stay inside a
+// DPP row (rotations), 16 uses ds_swizzle, 32 a bpermute: no LDS memory and no
+// global atomics are involved.
+template <int kTeam>
+__device__ __forceinline__ float cross_team_sum(float v)
+{
+    if constexpr (kTeam <= 1) v += dpp_f32<kDppQuadXor1>(v);
+    if constexpr (kTeam <= 2) v += dpp_f32<kDppQuadXor2>(v);
+    if constexpr (kTeam <= 4) v += dpp_f32<kDppRowRor4>(v);
+    if constexpr (kTeam <= 8) v += dpp_f32<kDppRowRor8>(v);
+    if constexpr (kTeam <= 16) v += swizzle_xor16(v);
+    if constexpr (kTeam <= 32) v += __shfl_xor(v, 32, kWave);
+    return v;
+}
+
+__device__ __forceinline__ int wave_inclusive_scan(int v)
+{
+    const int lane = lane_id();
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        int t = __shfl_up(v, off, kWave);
+        if (lane >= off) v += t;
+    }
+    return v;
+}
+
+__device__ __forceinline__ uint64_t wave_inclusive_scan_u64(uint64_t v)
+{
+    const int lane = lane_id();
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        uint64_t t = static_cast<uint64_t>(__shfl_up(static_cast<long long>(v), off, kWave));
+        if (lane >= off) v += t;
+    }
+    return v;
+}
+
+__device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+        v += static_cast<uint64_t>(__shfl_xor(static_cast<long long>(v), off, kWave));
+    return v;
+}
+
+// ---------------------------------------------------------------- look-back tiles
+// One 64-bit descriptor per tile: status in the two top bits, payload below.
+// Status and payload travel in one relaxed agent-scope atomic, so a reader that
+// sees the status also sees the payload.  Payloads are sums of non-negative
+// fields that never carry into each other, so packed payloads add directly.
+constexpr uint64_t kTileEmpty = 0;
+constexpr uint64_t kTileAggregate = 1ull << 62;
+constexpr uint64_t kTilePrefix = 2ull << 62;
+constexpr uint64_t kTilePayloadMask = (1ull << 62) - 1;
+constexpr unsigned kSpinLimit = 1u << 22;   // polls before a wait is declared stalled
+
+struct ScanState {
+    int counter;        // next tile id to hand out
+    int error;          // set to 1 when a look-back wait hit kSpinLimit
+    int counts[2];      // results the last tile publishes (meaning depends on the kernel)
+    int overflow;       // set to 1 when an output would not fit its capacity
+    int pad[3];
+};
+static_assert(sizeof(ScanState) == 32, "descriptor array starts 32 bytes into the workspace");
+
+__device__ __forceinline__ void tile_store(uint64_t* desc, int tile, uint64_t v)
+{
+    __hip_atomic_store(desc + tile, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ uint64_t tile_load(uint64_t* desc, int tile)
+{
+    return __hip_atomic_load(desc + tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Block-wide dynamic tile id.  Ids are handed out in start order, so when tile t
+// runs every tile below t is already running or finished: waiting on them cannot
+// deadlock on hardware that keeps resident workgroups running.
+__device__ __forceinline__ int acquire_tile(ScanState* st, int* s_tile)
+{
+    if (threadIdx.x == 0) *s_tile = atomicAdd(&st->counter, 1);
+    __syncthreads();
+    return *s_tile;
+}
+
+// Executed by one full wave.  Publishes this tile's aggregate, walks back over
+// the predecessors 64 at a time until a tile with a known inclusive prefix is
+// found, publishes this tile's inclusive prefix and returns its exclusive prefix
+// to every lane.  Every wait is bounded: after kSpinLimit polls the error flag is
+// raised and the walk continues with what it has, so the kernel always drains.
+__device__ __forceinline__ uint64_t tile_lookback(uint64_t* desc, ScanState* st, int tile, uint64_t aggregate)
+{
+    const int lane = lane_id();
+    if (tile == 0) {
+        if (lane == 0) tile_store(desc, 0, kTilePrefix | aggregate);
+        return 0;
+    }
+    if (lane == 0) tile_store(desc, tile, kTileAggregate | aggregate);
+    uint64_t exclusive = 0;
+    int base = tile - 1;
+    bool stalled = false;
+    while (true) {
+        const int t = base - lane;
+        uint64_t d = kTilePrefix;               // tiles before the first count as "prefix 0"
+        unsigned spins = 0;
+        while (true) {
+            if (t >= 0) d = tile_load(desc, t);
+            const bool ready = (d >> 62) != 0;
+            if (__all(ready)) break;
+            if (++spins >= kSpinLimit) { stalled = true; break; }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        const uint64_t has_prefix = __ballot((d >> 62) == 2);
+        const int first = has_prefix ? __builtin_ctzll(has_prefix) : kWave;
+        exclusive += wave_sum_u64(lane <= first ? (d & kTilePayloadMask) : 0ull);
+        if (first < kWave || stalled) break;
+        base -= kWave;
+    }
+    if (lane == 0) {
+        if (stalled) atomicExch(&st->error, 1);
+        tile_store(desc, tile, kTilePrefix | ((exclusive + aggregate) & kTilePayloadMask));
+    }
+    return exclusive;
+}
+
+}  // namespace eppgcn

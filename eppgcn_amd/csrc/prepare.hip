@@ -1,0 +1,414 @@
+// Execution-path preparation for gfx950 (wave64): path marking from the train
+// mask, single-pass stream compaction of the kept edges, splitting of the kept
+// edges into backward neighbour groups, forward neighbour groups from the CSR
+// row pointers, and the small counting kernels the group-size heuristics need.
+//
+// Replaces mask_forward_cuda_kernel (EPPGCN/GCNConv/EPPGCN_kernel.cu:351-388), the three
+// live cuCompactor namespaces and the thrust scans (EPPGCN/GCNConv/cuCompactor.cu:42-48,
+// :328-465, :467-621, :623-680) and the CPU loop of build_part
+// (EPPGCN/GCNConv/EPPGCN.cpp:186-227).
+//
+// Both scans are single-pass "decoupled look-back" scans: a tile publishes its
+// aggregate, then its wave 0 walks back over the predecessors' descriptors, 64
+// per step, until it meets a tile whose inclusive prefix is known.  Lane ranks
+// inside a wave come from a 64-bit ballot and mbcnt; no block-wide bit-sliced
+// counting and no second pass over the input.
+#include "common.hpp"
+
+namespace eppgcn {
+
+// ================================================================ scan state init
+__global__ void scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < num_tiles) desc[i] = kTileEmpty;
+    if (i == 0) {
+        st->counter = 0;
+        st->error = 0;
+        st->counts[0] = 0;
+        st->counts[1] = 0;
+        st->overflow = 0;
+    }
+}
+
+// ================================================================ path marking
+// A team of TS lanes owns one forward group and strides over its slots.
+template <int TS>
+__global__ __launch_bounds__(256) void mask_forward_kernel(
+    const int* __restrict__ part2node, const int* __restrict__ part_ptr, const int* __restrict__ col,
+    const uint8_t* __restrict__ src_mask, uint8_t* __restrict__ ngh_mask, int* __restrict__ back_edge_mask,
+    int* __restrict__ node_degs, int num_parts, int is_last)
+{
+    constexpr int TPW = kWave / TS;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int team = lane / TS;
+    const int tl = lane % TS;
+    const long long wave_global = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
+    const long long p = wave_global * TPW + team;
+    int beg = 0, end = 0, row = 0;
+    bool row_in_src = false;
+    if (p < num_parts) {
+        beg = part_ptr[p];
+        end = part_ptr[p + 1];
+        row = part2node[p];
+        row_in_src = !is_last && end > beg && src_mask[row] != 0;
+    }
+    if (row_in_src && tl == 0) ngh_mask[row] = 1;
+    int kept = 0;
+    // all lanes of the wave iterate together so that the ballot below is wave-uniform
+    const int span = end - beg;
+    int max_span = span;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) max_span = max(max_span, __shfl_xor(max_span, off, kWave));
+    for (int i = tl; i - tl < max_span; i += TS) {
+        const bool in_range = i < span;
+        bool keep = false;
+        if (in_range) {
+            const int e = beg + i;
+            const int end_id = col[e];
+            keep = src_mask[end_id] != 0;
+            if (keep) back_edge_mask[e] = row;
+            if (row_in_src) ngh_mask[end_id] = 1;
+        }
+        const uint64_t ballot = __ballot(keep);
+        const uint64_t team_bits = (TS == 64) ? ballot : ((ballot >> (team * TS)) & ((1ull << (TS % 64)) - 1ull));
+        kept += __popcll(team_bits);
+    }
+    if (tl == 0 && kept > 0) atomicAdd(node_degs + row, kept);
+}
+
+// ================================================================ compaction
+constexpr int kCompactBlock = 256;
+constexpr int kCompactItems = 16;
+constexpr int kCompactTile = kCompactBlock * kCompactItems;
+static_assert(kCompactItems * (kCompactBlock / kWave) == kWave, "one wave scans the per-(slab, wave) counts");
+
+__global__ __launch_bounds__(kCompactBlock) void compact_mask_kernel(
+    const int* __restrict__ in_id, const int* __restrict__ in_edge, int* __restrict__ out_id,
+    int* __restrict__ out_edge, int length, int num_tiles, ScanState* st, uint64_t* desc)
+{
+    __shared__ int s_tile;
+    __shared__ int s_count[kWave];
+    __shared__ int s_prefix;
+    const int tile = acquire_tile(st, &s_tile);
+    if (tile >= num_tiles) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const long long base = static_cast<long long>(tile) * kCompactTile;
+
+    int v[kCompactItems];
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k) {
+        const long long idx = base + k * kCompactBlock + threadIdx.x;
+        v[k] = idx < length ? in_id[idx] : -1;
+    }
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k) {
+        const uint64_t ballot = __ballot(v[k] != -1);
+        if (lane == 0) s_count[k * (kCompactBlock / kWave) + wave] = __popcll(ballot);
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const int c = s_count[lane];
+        const int incl = wave_inclusive_scan(c);
+        const int total = __shfl(incl, kWave - 1, kWave);
+        s_count[lane] = incl - c;
+        const uint64_t excl = tile_lookback(desc, st, tile, static_cast<uint64_t>(total));
+        if (lane == 0) {
+            s_prefix = static_cast<int>(excl);
+            if (tile == num_tiles - 1) st->counts[0] = static_cast<int>(excl) + total;
+        }
+    }
+    __syncthreads();
+    const int prefix = s_prefix;
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k) {
+        const bool pred = v[k] != -1;
+        const uint64_t ballot = __ballot(pred);
+        if (pred) {
+            const long long idx = base + k * kCompactBlock + threadIdx.x;
+            const int dst = prefix + s_count[k * (kCompactBlock / kWave) + wave] + ballot_rank(ballot);
+            out_id[dst] = v[k];
+            out_edge[dst] = in_edge[idx];
+        }
+    }
+}
+
+// Zero both outputs from the compacted length (read on the device) to the end.
+__global__ void zero_tail2_kernel(int* __restrict__ a, int* __restrict__ b, const int* __restrict__ d_start, int length)
+{
+    const long long start = *d_start;
+    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+    for (long long i = start + static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < length; i += stride) {
+        a[i] = 0;
+        b[i] = 0;
+    }
+}
+
+__global__ void zero_tail1_kernel(int* __restrict__ a, const int* __restrict__ d_start, int offset, long long length)
+{
+    const long long start = static_cast<long long>(*d_start) + offset;
+    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+    for (long long i = start + static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < length; i += stride)
+        a[i] = 0;
+}
+
+// ================================================================ counting
+__global__ __launch_bounds__(256) void count_nonzero_kernel(const int* __restrict__ in, int length, int* __restrict__ d_count)
+{
+    int local = 0;
+    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+    for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < length; i += stride)
+        local += in[i] != 0;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off, kWave);
+    if ((threadIdx.x & (kWave - 1)) == 0 && local) atomicAdd(d_count, local);
+}
+
+// Degree histogram of get_ginfo (EPPGCN/GCNConv/EPPGCN.cpp:356-377): hist[0] = #(deg != 0),
+// hist[3..9] = the seven buckets, the last one also taking deg <= 0 and deg >= 160.
+__global__ __launch_bounds__(256) void ginfo_hist_kernel(const int* __restrict__ node_deg, int length, int* __restrict__ hist)
+{
+    int local[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+    for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < length; i += stride) {
+        const int deg = node_deg[i];
+        local[0] += deg != 0;
+        int b = 7;
+        if (deg >= 1 && deg < 5) b = 1;
+        else if (deg >= 5 && deg < 10) b = 2;
+        else if (deg >= 10 && deg < 20) b = 3;
+        else if (deg >= 20 && deg < 40) b = 4;
+        else if (deg >= 40 && deg < 80) b = 5;
+        else if (deg >= 80 && deg < 160) b = 6;
+#pragma unroll
+        for (int k = 1; k < 8; ++k) local[k] += b == k;
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        int s = local[k];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, kWave);
+        if ((threadIdx.x & (kWave - 1)) == 0 && s) atomicAdd(hist + (k == 0 ? 0 : k + 2), s);
+    }
+}
+
+// ================================================================ group splitting
+// Vertex i with g_i slots (g_i = kept degree, or CSR degree) yields q_i = ceil(g_i/ps)
+// groups; group j of vertex i starts at G_i + j*ps where G_i is the exclusive sum
+// of g.  One look-back scan carries (sum q, sum g) packed as q*2^31 + g.  The
+// tile's groups are then written by all threads together: output slot o finds its
+// vertex by binary search over the tile's q offsets in LDS, so a hub vertex with
+// a hundred thousand groups costs its tile a longer loop, not one thread a longer
+// life.
+constexpr int kSplitBlock = 256;
+constexpr int kSplitItems = 8;
+constexpr int kSplitTile = kSplitBlock * kSplitItems;
+
+template <bool kFromRowPtr>
+__global__ __launch_bounds__(kSplitBlock) void split_groups_kernel(
+    const int* __restrict__ src, int num_nodes, int part_size, int* __restrict__ part_ptr_out,
+    int* __restrict__ part2node_out, long long capacity, int num_tiles, ScanState* st, uint64_t* desc)
+{
+    __shared__ int s_tile;
+    __shared__ int s_q[kSplitTile + 1];
+    __shared__ int s_g[kSplitTile];
+    __shared__ uint64_t s_wave[kSplitBlock / kWave];
+    __shared__ uint64_t s_tile_excl;
+    const int tile = acquire_tile(st, &s_tile);
+    if (tile >= num_tiles) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const long long base = static_cast<long long>(tile) * kSplitTile;
+
+    int g[kSplitItems], q[kSplitItems];
+    int tq = 0, tg = 0;
+#pragma unroll
+    for (int j = 0; j < kSplitItems; ++j) {
+        const long long i = base + threadIdx.x * kSplitItems + j;
+        int gi = 0;
+        if (i < num_nodes) gi = kFromRowPtr ? src[i + 1] - src[i] : src[i];
+        gi = gi > 0 ? gi : 0;
+        g[j] = gi;
+        q[j] = (gi + part_size - 1) / part_size;
+        tq += q[j];
+        tg += gi;
+    }
+    const uint64_t mine = (static_cast<uint64_t>(tq) << 31) | static_cast<uint64_t>(tg);
+    const uint64_t incl = wave_inclusive_scan_u64(mine);
+    if (lane == kWave - 1) s_wave[wave] = incl;
+    __syncthreads();
+    uint64_t wave_excl = 0, tile_total = 0;
+#pragma unroll
+    for (int w = 0; w < kSplitBlock / kWave; ++w) {
+        if (w < wave) wave_excl += s_wave[w];
+        tile_total += s_wave[w];
+    }
+    if (wave == 0) {
+        const uint64_t excl = tile_lookback(desc, st, tile, tile_total);
+        if (lane == 0) s_tile_excl = excl;
+    }
+    // tile-relative q offsets and absolute g offsets of this thread's vertices
+    uint64_t run = wave_excl + incl - mine;
+    const int g_first = kFromRowPtr ? src[0] : 0;
+    __syncthreads();
+    const uint64_t tile_excl = s_tile_excl;
+    const int q_base = static_cast<int>(tile_excl >> 31);
+    const int g_base = static_cast<int>(tile_excl & 0x7fffffffull) + g_first;
+#pragma unroll
+    for (int j = 0; j < kSplitItems; ++j) {
+        const int slot = threadIdx.x * kSplitItems + j;
+        s_q[slot] = static_cast<int>(run >> 31);
+        s_g[slot] = g_base + static_cast<int>(run & 0x7fffffffull);
+        run += (static_cast<uint64_t>(q[j]) << 31) | static_cast<uint64_t>(g[j]);
+    }
+    const int tile_q = static_cast<int>(tile_total >> 31);
+    if (threadIdx.x == 0) s_q[kSplitTile] = tile_q;
+    __syncthreads();
+
+    for (int o = threadIdx.x; o < tile_q; o += kSplitBlock) {
+        // last slot with s_q[slot] <= o
+        int lo = 0, hi = kSplitTile;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (s_q[mid] <= o) lo = mid; else hi = mid - 1;
+        }
+        const int j = o - s_q[lo];
+        const long long dst = static_cast<long long>(q_base) + o;
+        if (dst < capacity) {
+            part_ptr_out[dst] = s_g[lo] + j * part_size;
+            if (part2node_out && dst + 1 < capacity) part2node_out[dst] = static_cast<int>(base) + lo;
+        }
+    }
+    if (tile == num_tiles - 1 && threadIdx.x == 0) {
+        const uint64_t total = tile_excl + tile_total;
+        const int total_q = static_cast<int>(total >> 31);
+        const int total_g = static_cast<int>(total & 0x7fffffffull);
+        st->counts[0] = total_q;
+        st->counts[1] = total_g;
+        if (total_q < capacity) part_ptr_out[total_q] = total_g + g_first;
+        if (static_cast<long long>(total_q) + 1 > capacity) st->overflow = 1;
+    }
+}
+
+// ================================================================ host launchers
+size_t scan_workspace_bytes(long long length, int tile)
+{
+    const long long tiles = (length + tile - 1) / tile;
+    return sizeof(ScanState) + sizeof(uint64_t) * static_cast<size_t>(tiles > 0 ? tiles : 1);
+}
+
+size_t compact_workspace_bytes(long long length) { return scan_workspace_bytes(length, kCompactTile); }
+size_t split_workspace_bytes(long long num_nodes) { return scan_workspace_bytes(num_nodes, kSplitTile); }
+
+static int init_scan(void* workspace, int num_tiles, hipStream_t stream)
+{
+    ScanState* st = static_cast<ScanState*>(workspace);
+    uint64_t* desc = reinterpret_cast<uint64_t*>(st + 1);
+    const int n = num_tiles > 0 ? num_tiles : 1;
+    hipLaunchKernelGGL(scan_init_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, st, desc, num_tiles);
+    EPPGCN_HIP(hipGetLastError());
+    return kOk;
+}
+
+int launch_mask_forward(const int* part2node, const int* part_ptr, const int* col, const uint8_t* src_mask,
+                        uint8_t* ngh_mask, int* back_edge_mask, int* node_degs, int num_parts,
+                        long long num_edges, int is_last, hipStream_t stream)
+{
+    if (num_parts == 0) return kOk;
+    const double avg = static_cast<double>(num_edges) / num_parts;
+    int ts = 4;
+    while (ts < 64 && ts < avg) ts <<= 1;
+    const long long groups_per_block = (kWave / ts) * 4;
+    const unsigned grid = static_cast<unsigned>((num_parts + groups_per_block - 1) / groups_per_block);
+#define EPPGCN_MASK(TS_)                                                                                 \
+    hipLaunchKernelGGL((mask_forward_kernel<TS_>), dim3(grid), dim3(256), 0, stream, part2node, part_ptr, \
+                       col, src_mask, ngh_mask, back_edge_mask, node_degs, num_parts, is_last)
+    switch (ts) {
+        case 4: EPPGCN_MASK(4); break;
+        case 8: EPPGCN_MASK(8); break;
+        case 16: EPPGCN_MASK(16); break;
+        case 32: EPPGCN_MASK(32); break;
+        default: EPPGCN_MASK(64); break;
+    }
+#undef EPPGCN_MASK
+    EPPGCN_HIP(hipGetLastError());
+    return kOk;
+}
+
+// Results land in the ScanState at the head of the workspace: counts[0] = kept length.
+int launch_compact_mask(const int* in_id, int* out_id, const int* in_edge, int* out_edge, long long length,
+                        void* workspace, hipStream_t stream)
+{
+    ScanState* st = static_cast<ScanState*>(workspace);
+    uint64_t* desc = reinterpret_cast<uint64_t*>(st + 1);
+    const int num_tiles = static_cast<int>((length + kCompactTile - 1) / kCompactTile);
+    if (int rc = init_scan(workspace, num_tiles, stream)) return rc;
+    if (num_tiles > 0) {
+        hipLaunchKernelGGL(compact_mask_kernel, dim3(num_tiles), dim3(kCompactBlock), 0, stream, in_id, in_edge,
+                           out_id, out_edge, static_cast<int>(length), num_tiles, st, desc);
+        EPPGCN_HIP(hipGetLastError());
+        long long blocks = (length + 1023) / 1024;
+        if (blocks > 2048) blocks = 2048;
+        hipLaunchKernelGGL(zero_tail2_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, out_id,
+                           out_edge, st->counts, static_cast<int>(length));
+        EPPGCN_HIP(hipGetLastError());
+    }
+    return kOk;
+}
+
+// counts[0] = number of groups, counts[1] = number of slots covered.
+int launch_split(bool from_row_ptr, const int* src, int num_nodes, int part_size, int* part_ptr_out,
+                 int* part2node_out, long long capacity, bool zero_tail, void* workspace, hipStream_t stream)
+{
+    ScanState* st = static_cast<ScanState*>(workspace);
+    uint64_t* desc = reinterpret_cast<uint64_t*>(st + 1);
+    const int num_tiles = (num_nodes + kSplitTile - 1) / kSplitTile;
+    if (int rc = init_scan(workspace, num_tiles, stream)) return rc;
+    if (num_tiles == 0) {
+        if (capacity > 0) EPPGCN_HIP(hipMemsetAsync(part_ptr_out, 0, sizeof(int) * (zero_tail ? capacity : 1), stream));
+        return kOk;
+    }
+    if (from_row_ptr)
+        hipLaunchKernelGGL((split_groups_kernel<true>), dim3(num_tiles), dim3(kSplitBlock), 0, stream, src, num_nodes,
+                           part_size, part_ptr_out, part2node_out, capacity, num_tiles, st, desc);
+    else
+        hipLaunchKernelGGL((split_groups_kernel<false>), dim3(num_tiles), dim3(kSplitBlock), 0, stream, src, num_nodes,
+                           part_size, part_ptr_out, part2node_out, capacity, num_tiles, st, desc);
+    EPPGCN_HIP(hipGetLastError());
+    if (zero_tail) {
+        long long blocks = (capacity + 1023) / 1024;
+        if (blocks > 2048) blocks = 2048;
+        if (blocks < 1) blocks = 1;
+        hipLaunchKernelGGL(zero_tail1_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, part_ptr_out,
+                           st->counts, 1, capacity);
+        EPPGCN_HIP(hipGetLastError());
+    }
+    return kOk;
+}
+
+int launch_count_nonzero(const int* in, long long length, int* d_count, hipStream_t stream)
+{
+    EPPGCN_HIP(hipMemsetAsync(d_count, 0, sizeof(int), stream));
+    if (length == 0) return kOk;
+    long long blocks = (length + 1023) / 1024;
+    if (blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL(count_nonzero_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, in,
+                       static_cast<int>(length), d_count);
+    EPPGCN_HIP(hipGetLastError());
+    return kOk;
+}
+
+int launch_ginfo_hist(const int* node_deg, long long length, int* d_hist10, hipStream_t stream)
+{
+    EPPGCN_HIP(hipMemsetAsync(d_hist10, 0, sizeof(int) * 10, stream));
+    if (length == 0) return kOk;
+    long long blocks = (length + 1023) / 1024;
+    if (blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL(ginfo_hist_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, node_deg,
+                       static_cast<int>(length), d_hist10);
+    EPPGCN_HIP(hipGetLastError());
+    return kOk;
+}
+
+}  // namespace eppgcn

@@ -1,0 +1,178 @@
+/*
+ * C ABI of the MI355X (gfx950) GCN aggregation path: libeppgcn_hip.so.
+ *
+ * Tensor-free: device pointers, sizes and a HIP stream (passed as void*, a
+ * hipStream_t; NULL = the default stream).  These are the entry points a binding
+ * of the reference's `GNNAdvisor` extension module needs; each declaration names
+ * the reference interface it stands in for (paths relative to the reference
+ * checkout, EPPGCN/GCNConv/).  The dense X*W products of the reference's
+ * launchers stay with the caller (torch.mm); the library covers aggregation,
+ * path marking, compaction and group construction.
+ *
+ * Conventions
+ *   - Every function returns 0 on success or a negative code (EPPGCN_ERR_*);
+ *     eppgcn_last_error() then returns a message.  Nothing aborts the process.
+ *   - All pointers are DEVICE pointers unless the name starts with h_.
+ *     Index data is int32, features fp32 row-major contiguous, masks one byte
+ *     per vertex (torch.bool layout).
+ *   - Calls are asynchronous on `stream` unless a host result (h_*) is
+ *     requested; a function that fills an h_* argument synchronises the stream
+ *     first, as the reference's compactors do.
+ *   - Scan-based functions need a workspace of at least the number of bytes the
+ *     matching *_workspace_bytes() call returns, 8-byte aligned.  The library
+ *     itself allocates no device memory.
+ */
+#ifndef EPPGCN_HIP_H_
+#define EPPGCN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EPPGCN_OK 0
+#define EPPGCN_ERR_INVALID_ARGUMENT (-1)
+#define EPPGCN_ERR_HIP (-2)
+#define EPPGCN_ERR_SCAN_STALLED (-3)
+#define EPPGCN_ERR_CAPACITY (-4)
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char* eppgcn_last_error(void);
+/* ABI version of this header. */
+int eppgcn_abi_version(void);
+
+/* ---------------------------------------------------------------------------
+ * Aggregation.
+ * ------------------------------------------------------------------------- */
+
+/* Forward neighbour-group aggregation:
+ *   out[r,:] = sum_{e in groups of r} fl32(degrees[r]*degrees[col[e]]) * in[col[e],:]
+ * `out` ([num_nodes, dim]) is fully overwritten (rows without groups become 0).
+ * Stands in for spmm_forward_cuda minus its torch::mm (EPPGCN_kernel.cu:123-202;
+ * kernel :204-295; bound as GNNA.forward, EPPGCN.cpp:79-102,390).  row_pointers
+ * may be NULL (the reference's kernel never reads it).  part_size, dim_worker and
+ * warp_per_block are the caller's launch hints for 32-lane warps; the wave64
+ * mapping is chosen from `dim`, the hints only have to be positive. */
+int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers,
+                        const int32_t* column_index, const float* degrees,
+                        const int32_t* part_pointers, const int32_t* part2node,
+                        int num_nodes, int dim, int num_parts,
+                        int part_size, int dim_worker, int warp_per_block, void* stream);
+
+/* Unpruned backward aggregation: the same operator applied to d_output (valid
+ * because the normalised adjacency is symmetric).  Stands in for
+ * spmm_backward_cuda minus its two torch::mm (EPPGCN_kernel.cu:395-469; kernel
+ * :471-545; bound as GNNA.backward, EPPGCN.cpp:104-130,391). */
+int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* row_pointers,
+                         const int32_t* column_index, const float* degrees,
+                         const int32_t* part_pointers, const int32_t* part2node,
+                         int num_nodes, int dim, int num_parts,
+                         int part_size, int dim_worker, int warp_per_block, void* stream);
+
+/* Pruned backward aggregation over the compacted execution path:
+ *   d_input[id_p,:] += sum_{k in group p} fl32(degrees[id_p]*degrees[edge_list[k]]) * d_output[edge_list[k],:]
+ * with id_p = ids[part_pointer[p]]; d_input is fully overwritten (zero elsewhere).
+ * part_pointer holds num_parts+1 entries.  Stands in for ours_backward_cuda minus
+ * its two torch::mm (EPPGCN_kernel.cu:547-624; kernel :626-670; bound as
+ * GNNA.ours_backward, EPPGCN.cpp:157-184,393).  `layer` (1-based) only selects the
+ * per-layer timer; blockx/blocky are the caller's hints and must be positive. */
+int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids,
+                         const int32_t* part_pointer, const int32_t* edge_list, const float* degrees,
+                         int num_nodes, int dim, int num_parts, int part_size, int layer,
+                         int blockx, int blocky, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Execution-path preparation.
+ * ------------------------------------------------------------------------- */
+
+/* Marks one layer's backward path from the forward groups (in place):
+ *   slot e of row r with src_mask[col[e]]      -> back_edge_mask[e] = r, node_degs[r] += 1
+ *   !is_last_layer and src_mask[r]             -> ngh_mask[r] = ngh_mask[col[e]] = 1
+ * back_edge_mask must be pre-filled with -1 and node_degs with 0 by the caller
+ * (EPPGCN/dataset.py:149-156); ngh_mask may be NULL when is_last_layer.  Stands in
+ * for mask_forward_cuda (EPPGCN_kernel.cu:297-349; kernel :351-388; bound as
+ * GNNA.mask_forward, EPPGCN.cpp:132-155,392; is_last_layer = (layer == num_layers)). */
+int eppgcn_mask_forward(const int32_t* part2node, const int32_t* part_pointers,
+                        const int32_t* column_index, const uint8_t* src_mask, uint8_t* ngh_mask,
+                        int32_t* back_edge_mask, int32_t* node_degs, int num_parts,
+                        int64_t num_edges, int is_last_layer, int blockx, int blocky, void* stream);
+
+/* Workspace sizes for the scan-based functions below. */
+size_t eppgcn_compact_workspace_bytes(int64_t length);
+size_t eppgcn_split_workspace_bytes(int64_t num_nodes);
+
+/* Stable two-array compaction of the slots with edge_mask[e] != -1:
+ *   out_id[k] = edge_mask[e_k], out_edge[k] = column_index[e_k], k < V; both
+ * outputs (length entries each) are zero from V on.  V is left in device memory at
+ * d_valid_len (may be NULL) and, when h_valid_len is not NULL, copied to the host
+ * after synchronising.  Stands in for compact_mask (cuCompactor.cu:682-686 over
+ * :328-465) as compact_back_edge uses it (EPPGCN.cpp:282-296,399). */
+int eppgcn_compact_back_edge(const int32_t* edge_mask, const int32_t* column_index,
+                             int32_t* out_id, int32_t* out_edge, int64_t length,
+                             void* workspace, size_t workspace_bytes,
+                             int32_t* d_valid_len, int64_t* h_valid_len, void* stream);
+
+/* Number of entries != 0 (valid_node of the group-size heuristics).  Stands in for
+ * compact_count (cuCompactor.cu:694-696 over :623-680).  d_count: one device int. */
+int eppgcn_count_nonzero(const int32_t* node_deg, int64_t length, int32_t* d_count,
+                         int64_t* h_count, void* stream);
+
+/* Backward group size from the fitted regression, in double arithmetic with C
+ * round() (EPPGCN.cpp:303-310, get_map_back_part_size).  Pure host function.
+ * The raw value can be <= 0 on large sparse paths; *clamped (may be NULL) is set
+ * when the returned value was raised to 1. */
+int eppgcn_map_back_part_size(int64_t valid_node, int64_t valid_len, int* clamped);
+/* Legacy threshold rule of build_back_part (EPPGCN.cpp:246-258); returns 0 when the
+ * ratio is >= 512, as the reference leaves it. */
+int eppgcn_threshold_back_part_size(int64_t valid_node, int64_t valid_len);
+
+/* Splits the kept edges of every vertex into groups of part_size and writes the
+ * group pointers: part_pointer[0..P] with part_pointer[P] = V, zero after that up
+ * to `capacity` entries.  d_counts (may be NULL) receives {P, V} on the device;
+ * h_num_parts / h_valid_len are filled after synchronising when not NULL.
+ * Fails with EPPGCN_ERR_CAPACITY (host results requested) if P + 1 > capacity.
+ * Stands in for compact_part + exclusive_scan (cuCompactor.cu:688-692 over
+ * :467-621, and :42-48) as split_back_part composes them (EPPGCN.cpp:327-346,401). */
+int eppgcn_split_back_part(const int32_t* node_deg, int num_nodes, int part_size,
+                           int32_t* part_pointer, int64_t capacity,
+                           void* workspace, size_t workspace_bytes, int32_t* d_counts,
+                           int64_t* h_num_parts, int64_t* h_valid_len, void* stream);
+
+/* Forward neighbour groups from the CSR row pointers (device): part_pointers[0..P]
+ * (terminator = row_pointers[num_nodes]) and part2node[0..P-1]; `capacity` is the
+ * number of entries part_pointers can hold (part2node: capacity - 1); an upper
+ * bound is num_edges / part_size + num_nodes + 1.  Stands in for build_part
+ * (EPPGCN.cpp:186-227,397), which the reference runs on the CPU. */
+int eppgcn_build_part(const int32_t* row_pointers, int num_nodes, int part_size,
+                      int32_t* part_pointers, int32_t* part2node, int64_t capacity,
+                      void* workspace, size_t workspace_bytes, int32_t* d_counts,
+                      int64_t* h_num_parts, void* stream);
+
+/* Degree-distribution features of get_ginfo (EPPGCN.cpp:348-386,402): h_out[10]
+ * on the host; d_hist: ten device ints of scratch.  Synchronises. */
+int eppgcn_get_ginfo(const int32_t* node_deg, int64_t num_nodes, int64_t valid_len,
+                     int32_t* d_hist, float* h_out, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Timers (print_time / clear_time, EPPGCN_kernel.cu:89-116; EPPGCN.cpp:394-395).
+ * Timing is off by default so that calls stay asynchronous; when enabled every
+ * aggregation / marking call brackets its kernels with events and synchronises.
+ * Not thread-safe, like the reference's file-scope accumulators.
+ * ------------------------------------------------------------------------- */
+void eppgcn_set_timing(int enabled);
+void eppgcn_print_time(void);
+void eppgcn_clear_time(void);
+/* which: 0 forward aggregation, 1 backward aggregation (all layers), 2 path marking,
+ * 100+k backward aggregation of layer k (1-based, k <= 16).  Milliseconds. */
+double eppgcn_get_time_ms(int which);
+
+/* Forces the number of lanes per neighbour group in the aggregation kernels
+ * (power of two in 4..64; 0 = choose from the feature width).  For tuning runs. */
+void eppgcn_set_team_size(int lanes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EPPGCN_HIP_H_ */

@@ -1,0 +1,357 @@
+"""GPU parity: every entry point of the C ABI (through ctypes) against the CPU checker.
+
+Bars: integer outputs (group pointers, path marking, compacted lists, counts) bit-exact;
+aggregation outputs within rel. tol. 1e-5 of the float64 sum, the tolerance being taken
+relative to sum_j |w_ij x_j| per output element (summation-order differences only)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from oracle import closed_forms as cf
+from tests.helpers import hub_csr, random_symmetric_csr, scale_inv_sqrt, scale_sqrt
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def api():
+    from eppgcn_amd import capi
+    capi.load()
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return capi
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda()
+
+
+def assert_close(got, want64, bound, what=""):
+    err = np.abs(got.astype(np.float64) - want64)
+    lim = RTOL * bound + 1e-30
+    worst = float(np.max(err / lim)) if err.size else 0.0
+    assert worst <= 1.0, f"{what}: max err/limit = {worst:.3f}"
+
+
+GRAPHS = {
+    "single": lambda: random_symmetric_csr(1, 0, 0),
+    "tiny": lambda: random_symmetric_csr(7, 9, 2),
+    "small": lambda: random_symmetric_csr(130, 260, 5),
+    "isolated": lambda: random_symmetric_csr(3000, 9000, 11, isolated=0.3),
+    "hub": lambda: hub_csr(5000, 4000, 7),
+    "medium": lambda: random_symmetric_csr(20000, 150000, 13),
+}
+
+
+# ----------------------------------------------------------------------------- build_part
+@pytest.mark.parametrize("name", list(GRAPHS))
+@pytest.mark.parametrize("ps", [1, 3, 8, 32, 5000])
+def test_build_part_bit_exact(api, name, ps):
+    indptr, col = GRAPHS[name]()
+    want_pp, want_p2n = co.build_part(ps, indptr)
+    pp, p2n = api.build_part(ps, dev(indptr), col.size)
+    assert np.array_equal(pp.cpu().numpy(), want_pp)
+    assert np.array_equal(p2n.cpu().numpy(), want_p2n)
+
+
+# ----------------------------------------------------------------------------- mask_forward
+@pytest.mark.parametrize("name", ["tiny", "small", "isolated", "hub", "medium"])
+@pytest.mark.parametrize("ratio", [0.0, 0.1, 0.5, 1.0])
+@pytest.mark.parametrize("ps", [1, 5, 32, 200])
+def test_mask_forward_bit_exact(api, name, ratio, ps):
+    indptr, col = GRAPHS[name]()
+    n, e = indptr.size - 1, col.size
+    rng = np.random.default_rng(int(ratio * 100) + ps)
+    src = rng.random(n) < ratio
+    pre_ngh = rng.random(n) < 0.02
+    pre_degs = rng.integers(0, 3, n).astype(np.int32)
+    pp, p2n = co.build_part(ps, indptr)
+    for is_last in (False, True):
+        want = cf.mask_forward(indptr, col, src, pre_ngh, np.full(e, -1, np.int32), pre_degs, is_last)
+        ngh = dev(pre_ngh)
+        bem = torch.full((e,), -1, dtype=torch.int32, device="cuda")
+        degs = dev(pre_degs)
+        api.mask_forward(dev(p2n), dev(pp), dev(col), dev(src), None if is_last else ngh, bem, degs, is_last)
+        assert np.array_equal(bem.cpu().numpy(), want[1])
+        assert np.array_equal(degs.cpu().numpy(), want[2])
+        assert np.array_equal(ngh.cpu().numpy(), want[0] if not is_last else pre_ngh)
+
+
+# ----------------------------------------------------------------------------- compaction
+@pytest.mark.parametrize("length", [0, 1, 63, 64, 65, 4095, 4096, 4097, 100000, 1 << 20, (1 << 22) + 12345])
+@pytest.mark.parametrize("density", [0.0, 0.1, 0.5, 1.0])
+def test_compact_back_edge_bit_exact(api, length, density):
+    rng = np.random.default_rng(length % 9973 + int(density * 10))
+    em = np.where(rng.random(length) < density, rng.integers(0, 1 << 20, length), -1).astype(np.int32)
+    col = rng.integers(0, 1 << 20, length).astype(np.int32)
+    want_id, want_edge, want_v = cf.compact_mask(em, col)
+    oid, oedge, v = api.compact_back_edge(dev(em), dev(col))
+    assert v == want_v
+    assert np.array_equal(oid.cpu().numpy(), want_id)
+    assert np.array_equal(oedge.cpu().numpy(), want_edge)
+
+
+def test_compact_is_deterministic_across_runs(api):
+    rng = np.random.default_rng(5)
+    length = 3_000_000
+    em = np.where(rng.random(length) < 0.3, rng.integers(0, 1000, length), -1).astype(np.int32)
+    col = rng.integers(0, 1000, length).astype(np.int32)
+    dem, dcol = dev(em), dev(col)
+    first = api.compact_back_edge(dem, dcol)
+    for _ in range(5):
+        again = api.compact_back_edge(dem, dcol)
+        assert again[2] == first[2]
+        assert torch.equal(again[0], first[0]) and torch.equal(again[1], first[1])
+
+
+# ----------------------------------------------------------------------------- split / counts
+@pytest.mark.parametrize("n", [1, 5, 2047, 2048, 2049, 100000, 1 << 20])
+@pytest.mark.parametrize("ps", [1, 2, 8, 32, 64])
+def test_split_back_part_bit_exact(api, n, ps):
+    rng = np.random.default_rng(n % 1000 + ps)
+    degs = (rng.integers(0, 40, n) * (rng.random(n) < 0.6)).astype(np.int32)
+    if n > 10:
+        degs[n // 3] = 70000          # far more than 1023 groups for one vertex
+    e = int(degs.sum()) + 17
+    want_pp, want_p = cf.split_back_part(degs, e, ps)
+    pp, p, v = api.split_back_part(dev(degs), e, ps)
+    assert p == want_p and v == int(degs.sum())
+    assert np.array_equal(pp.cpu().numpy(), want_pp)
+    assert api.count_nonzero(dev(degs)) == cf.compact_count(degs)
+
+
+def test_split_all_zero_and_capacity_error(api):
+    degs = np.zeros(5000, np.int32)
+    pp, p, v = api.split_back_part(dev(degs), 100, 8)
+    assert p == 0 and v == 0 and not pp.cpu().numpy().any()
+    degs[:] = 3
+    with pytest.raises(api.EppgcnError):
+        api.split_back_part(dev(degs), 100, 1)     # 15000 groups cannot fit 101 entries
+
+
+def test_heuristics_and_ginfo(api):
+    for vn, vl in [(1000, 5000), (100000, 1000000), (419000, 13_400_000), (7, 7)]:
+        ps, clamped = api.map_back_part_size(vn, vl)
+        raw = cf.map_back_part_size(vn, vl)
+        assert ps == max(raw, 1) and clamped == (raw < 1)
+        assert api.threshold_back_part_size(vn, vl) == cf.threshold_back_part_size(vn, vl)
+    assert api.map_back_part_size(1_000_000, 100_000_000) == (1, True)   # raw value is negative
+    rng = np.random.default_rng(1)
+    degs = (rng.integers(0, 300, 100000) * (rng.random(100000) < 0.7)).astype(np.int32)
+    got = api.get_ginfo(dev(degs), 12345).numpy()
+    assert np.allclose(got, cf.get_ginfo(degs, 12345), rtol=1e-6)
+
+
+# ----------------------------------------------------------------------------- aggregation
+def _forward_case(api, indptr, col, s, x, ps, what):
+    n = indptr.size - 1
+    pp, p2n = co.build_part(ps, indptr)
+    got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp), dev(p2n), part_size=ps).cpu().numpy()
+    want = co.spmm_f64(x, indptr, col, s)
+    bound = cf.abs_sum_bound(indptr, col, s, x)
+    assert_close(got, want, bound, what)
+    return got
+
+
+@pytest.mark.parametrize("name", list(GRAPHS))
+@pytest.mark.parametrize("dim", [16, 22])
+@pytest.mark.parametrize("ps", [1, 4, 32, 700])
+def test_forward_aggregation_headline_widths(api, name, dim, ps):
+    indptr, col = GRAPHS[name]()
+    n = indptr.size - 1
+    rng = np.random.default_rng(dim + ps)
+    x = rng.standard_normal((n, dim)).astype(np.float32)
+    for scale_fn in (scale_inv_sqrt, scale_sqrt):
+        s = scale_fn(indptr)
+        got = _forward_case(api, indptr, col, s, x, ps, f"{name} D={dim} ps={ps}")
+        # the fp32 restatement of the reference's rounding model agrees to the same tolerance
+        pp, p2n = co.build_part(ps, indptr)
+        ref32 = co.spmm_groups(x, col, s, pp, p2n, n)
+        assert_close(got, ref32.astype(np.float64), 2 * cf.abs_sum_bound(indptr, col, s, x), "vs fp32 restatement")
+
+
+@pytest.mark.parametrize("dim", [1, 2, 3, 4, 6, 8, 12, 31, 32, 64, 96, 100, 128, 250, 256, 300, 512, 1030, 1100])
+def test_forward_aggregation_every_width_class(api, dim):
+    indptr, col = hub_csr(1500, 1200, 3)
+    n = indptr.size - 1
+    x = np.random.default_rng(dim).standard_normal((n, dim)).astype(np.float32)
+    s = scale_inv_sqrt(indptr)
+    for ps in (7, 64):
+        _forward_case(api, indptr, col, s, x, ps, f"D={dim} ps={ps}")
+
+
+@pytest.mark.parametrize("team", [4, 8, 16, 32, 64])
+@pytest.mark.parametrize("dim", [16, 22, 64])
+def test_forward_aggregation_forced_team_sizes(api, team, dim):
+    indptr, col = hub_csr(4000, 3000, 9)
+    n = indptr.size - 1
+    x = np.random.default_rng(team + dim).standard_normal((n, dim)).astype(np.float32)
+    s = scale_inv_sqrt(indptr)
+    try:
+        api.set_team_size(team)
+        for ps in (3, 32):
+            _forward_case(api, indptr, col, s, x, ps, f"team={team} D={dim} ps={ps}")
+    finally:
+        api.set_team_size(0)
+
+
+def test_forward_unit_scale_integer_features_bit_exact(api):
+    """With s == 1 and small integer features every partial sum is exact in fp32, so any
+    grouping, lane mapping or atomic order must give exactly the neighbour sum."""
+    indptr, col = hub_csr(6000, 5000, 4)
+    n = indptr.size - 1
+    x = np.random.default_rng(0).integers(-8, 9, (n, 22)).astype(np.float32)
+    s = np.ones(n, np.float32)
+    want = np.zeros((n, 22), np.float64)
+    np.add.at(want, cf.row_index(indptr), x[col].astype(np.float64))
+    for ps in (1, 5, 32, 100):
+        pp, p2n = co.build_part(ps, indptr)
+        got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp), dev(p2n), part_size=ps).cpu().numpy()
+        assert np.array_equal(got.astype(np.float64), want)
+        back = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp), dev(p2n), part_size=ps, backward=True)
+        assert np.array_equal(back.cpu().numpy(), got)
+
+
+def test_forward_zero_groups_and_argument_errors(api):
+    x = torch.randn(10, 16, device="cuda")
+    empty = torch.zeros(0, dtype=torch.int32, device="cuda")
+    pp = torch.zeros(1, dtype=torch.int32, device="cuda")
+    out = api.spmm_forward(x, empty, torch.ones(10, device="cuda"), pp, empty)
+    assert not out.any()
+    with pytest.raises(api.EppgcnError):
+        api.spmm_forward(x.double(), empty, torch.ones(10, device="cuda"), pp, empty)
+    with pytest.raises(api.EppgcnError):
+        api.spmm_forward(x, empty, torch.ones(10, device="cuda"), pp, empty, part_size=0)
+    with pytest.raises(api.EppgcnError):
+        api.spmm_forward(x.cpu(), empty, torch.ones(10, device="cuda"), pp, empty)
+
+
+# ----------------------------------------------------------------------------- pruned backward
+def _gpu_path(api, indptr, col, src, ps_fwd, ps_back):
+    """mask -> compact -> split on the GPU, checked bit-exact against the closed form."""
+    n, e = indptr.size - 1, col.size
+    pp, p2n = co.build_part(ps_fwd, indptr)
+    bem = torch.full((e,), -1, dtype=torch.int32, device="cuda")
+    degs = torch.zeros(n, dtype=torch.int32, device="cuda")
+    api.mask_forward(dev(p2n), dev(pp), dev(col), dev(src), None, bem, degs, True)
+    oid, oedge, v = api.compact_back_edge(bem, dev(col))
+    bpp, p, v2 = api.split_back_part(degs, e, ps_back)
+    w_id, w_edge, w_pp, w_v, w_p, w_degs = cf.pruned_path(indptr, col, src, ps_back)
+    assert v == v2 == w_v and p == w_p
+    assert np.array_equal(oid.cpu().numpy(), w_id) and np.array_equal(oedge.cpu().numpy(), w_edge)
+    assert np.array_equal(bpp.cpu().numpy(), w_pp) and np.array_equal(degs.cpu().numpy(), w_degs)
+    return oid, oedge, bpp, p
+
+
+@pytest.mark.parametrize("name", ["tiny", "small", "isolated", "hub", "medium"])
+@pytest.mark.parametrize("dim", [16, 22, 64])
+@pytest.mark.parametrize("ratio", [0.0, 0.01, 0.1, 0.5, 1.0])
+def test_pruned_backward_vs_checker_and_unpruned(api, name, dim, ratio):
+    indptr, col = GRAPHS[name]()
+    n = indptr.size - 1
+    rng = np.random.default_rng(dim + int(ratio * 100))
+    src = rng.random(n) < ratio
+    s = scale_inv_sqrt(indptr)
+    dy = (rng.standard_normal((n, dim)) * src[:, None]).astype(np.float32)
+    want = co.spmm_f64(dy, indptr, col, s)
+    bound = cf.abs_sum_bound(indptr, col, s, dy)
+    for ps_back in (1, 8, 64):
+        oid, oedge, bpp, p = _gpu_path(api, indptr, col, src, 5, ps_back)
+        got = api.ours_backward(dev(dy), oid, bpp, oedge, dev(s), p, part_size=ps_back).cpu().numpy()
+        assert_close(got, want, bound, f"{name} D={dim} r={ratio} ps={ps_back}")
+        ref32 = co.ours_backward(dy, oid.cpu().numpy(), bpp.cpu().numpy(), oedge.cpu().numpy(), s, p)
+        assert_close(got, ref32.astype(np.float64), 2 * bound, "vs fp32 restatement")
+        # pruning really ignores gradient rows outside the mask
+        noisy = (dy + (~src)[:, None] * 50.0).astype(np.float32)
+        got2 = api.ours_backward(dev(noisy), oid, bpp, oedge, dev(s), p, part_size=ps_back).cpu().numpy()
+        assert_close(got2, want, bound, "noise outside the mask")
+
+
+def test_two_layer_mask_chain_on_gpu(api):
+    """The wiring of the reference's driver for 2 layers (EPPGCN/gcn_main.py:130-139)."""
+    indptr, col = GRAPHS["medium"]()
+    n, e = indptr.size - 1, col.size
+    rng = np.random.default_rng(2)
+    train = rng.random(n) < 0.1
+    pp, p2n = co.build_part(8, indptr)
+    dpp, dp2n, dcol = dev(pp), dev(p2n), dev(col)
+    ngh0 = torch.zeros(n, dtype=torch.bool, device="cuda")
+    em = [torch.full((e,), -1, dtype=torch.int32, device="cuda") for _ in range(2)]
+    nd = [torch.zeros(n, dtype=torch.int32, device="cuda") for _ in range(2)]
+    api.mask_forward(dp2n, dpp, dcol, dev(train), ngh0, em[1], nd[1], False)          # conv 0's forward
+    api.mask_forward(dp2n, dpp, dcol, ngh0, torch.zeros(0, dtype=torch.bool, device="cuda"), em[0], nd[0], True)
+    row = cf.row_index(indptr)
+    closure = train.copy()
+    closure[col[train[row]]] = True
+    assert np.array_equal(ngh0.cpu().numpy(), closure)
+    assert np.array_equal(em[1].cpu().numpy() != -1, train[col])
+    assert np.array_equal(em[0].cpu().numpy() != -1, closure[col])
+
+
+# ----------------------------------------------------------------------------- full-size properties
+@pytest.fixture(scope="module")
+def rmat20():
+    from eppgcn_amd import graphs
+    return graphs.make_graph("cfg3_rmat20", device="cuda")
+
+
+def test_rmat20_exact_integer_sums_and_path_invariants(api, rmat20):
+    """Size-independent properties at a benchmark size (R-MAT scale 20): exact integer neighbour
+    sums against torch index_add in int64; compacted-path invariants; pruned == unpruned."""
+    from eppgcn_amd import graphs
+    g = rmat20
+    n, e = g.num_nodes, g.num_edges
+    ps = int(g.avg_degree)
+    pp, p2n = api.build_part(ps, g.row_pointers, e)
+    assert int(pp[-1]) == e and int((pp[1:] - pp[:-1]).max()) <= ps and int((pp[1:] - pp[:-1]).min()) >= 1
+    row = g.row_index()
+    xi = (graphs.uniform32(5, torch.arange(n * 16, device="cuda")) % 17 - 8).reshape(n, 16)
+    ones = torch.ones(n, device="cuda")
+    got = api.spmm_forward(xi.float(), g.column_index, ones, pp, p2n, part_size=ps)
+    want = torch.zeros(n, 16, dtype=torch.int64, device="cuda").index_add_(0, row, xi[g.column_index.long()])
+    assert torch.equal(got.long(), want)
+
+    train = graphs.bernoulli_mask(n, 0.1, 2, "cuda")
+    bem = torch.full((e,), -1, dtype=torch.int32, device="cuda")
+    degs = torch.zeros(n, dtype=torch.int32, device="cuda")
+    api.mask_forward(p2n, pp, g.column_index, train, None, bem, degs, True)
+    keep = train[g.column_index.long()]
+    assert torch.equal(bem != -1, keep)
+    oid, oedge, v = api.compact_back_edge(bem, g.column_index)
+    assert v == int(keep.sum())
+    assert torch.equal(oid[:v].long(), row[keep]) and torch.equal(oedge[:v], g.column_index[keep])
+    assert not oid[v:].any() and not oedge[v:].any()
+    assert torch.equal(torch.bincount(oid[:v].long(), minlength=n).int(), degs)
+    for ps_b in (8, 32):
+        bpp, p, v2 = api.split_back_part(degs, e, ps_b)
+        assert v2 == v and int(bpp[p]) == v
+        sizes = bpp[1: p + 1] - bpp[:p]
+        assert int(sizes.min()) >= 1 and int(sizes.max()) <= ps_b
+        assert torch.equal(oid[bpp[:p].long()], oid[(bpp[1: p + 1] - 1).long()])   # a group never spans two rows
+        dy = xi.float() * train[:, None]
+        pruned = api.ours_backward(dy, oid, bpp, oedge, ones, p, part_size=ps_b)
+        unpruned = api.spmm_forward(dy, g.column_index, ones, pp, p2n, part_size=ps, backward=True)
+        assert torch.equal(pruned, unpruned)
+
+
+def test_rmat20_linearity_and_tolerance(api, rmat20):
+    from eppgcn_amd import graphs
+    g = rmat20
+    n, e = g.num_nodes, g.num_edges
+    ps = int(g.avg_degree)
+    pp, p2n = api.build_part(ps, g.row_pointers, e)
+    for dim in (16, 22):
+        x = graphs.normal32(1, (n, dim), "cuda")
+        got = api.spmm_forward(x, g.column_index, g.degrees, pp, p2n, part_size=ps)
+        row = g.row_index()
+        w = (g.degrees[row] * g.degrees[g.column_index.long()]).double()
+        want = torch.zeros(n, dim, dtype=torch.float64, device="cuda").index_add_(
+            0, row, w[:, None] * x[g.column_index.long()].double())
+        bound = torch.zeros(n, dim, dtype=torch.float64, device="cuda").index_add_(
+            0, row, w.abs()[:, None] * x[g.column_index.long()].double().abs())
+        worst = ((got.double() - want).abs() / (RTOL * bound + 1e-30)).max().item()
+        assert worst <= 1.0, f"D={dim}: max err/limit {worst:.3f}"
