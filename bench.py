@@ -1,0 +1,212 @@
+#!/usr/bin/env python3
+"""Benchmark of the GCN aggregation path on one MI355X.
+
+A step is one epoch's worth of aggregation for the 2-layer GCN of the reference's driver
+(hidden 16, 22 classes): forward aggregation at width 16 and 22, pruned backward aggregation
+at width 22 (last layer) and 16 (first layer), launched back to back through the C ABI with
+every input resident in HBM.  The dense X*W products are not part of the metric.
+
+Prints ONE JSON line:  metric = BASELINE.json's, value = algorithmic GB/s of the epoch's
+aggregation, ms_per_step = aggregation ms per epoch, plus `roofline` for the dominant kernel
+(HIP-event time of the kernel alone) and `cpu_baseline` (the CPU checker's OpenMP restatement
+timed on the host cores on one epoch of the same workload).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0
+METRIC = "fwd+bwd aggregation ms/epoch and achieved HBM GB/s (% peak), 1 MI355X"
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="cfg4_rmat22",
+                    choices=["cfg1_uniform", "cfg2_chunglu", "cfg3_rmat20", "cfg4_rmat22"])
+    ap.add_argument("--train_ratio", type=float, default=0.1)
+    ap.add_argument("--backsize_mode", default="constant", choices=["constant", "map", "threshold"])
+    ap.add_argument("--backsize", type=int, default=32)
+    ap.add_argument("--part_size", type=int, default=0, help="forward group size (0 = int(avg degree))")
+    ap.add_argument("--team", type=int, default=0, help="force lanes per group (0 = automatic)")
+    ap.add_argument("--no_cpu_baseline", action="store_true")
+    ap.add_argument("--no_train", action="store_true", help="skip the 100-epoch training timing")
+    ap.add_argument("--train_epochs", type=int, default=100)
+    ap.add_argument("--verbose", action="store_true")
+    return ap.parse_args()
+
+
+def log(args, *a):
+    if args.verbose:
+        print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus must be 1 (no multi-GPU path exists).",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from eppgcn_amd import capi, graphs, workload
+
+    capi.load()                      # fails loudly when the HIP library is missing
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs the MI355X (no CPU fallback exists)")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    t0 = time.perf_counter()
+    g = graphs.make_graph(args.config, device=dev)
+    torch.cuda.synchronize()
+    log(args, "graph", g.stats(), f"{time.perf_counter() - t0:.1f}s")
+    t0 = time.perf_counter()
+    wl = workload.prepare(g, 2, args.train_ratio, 2, args.part_size or None, args.backsize_mode, args.backsize)
+    torch.cuda.synchronize()
+    prep_s = time.perf_counter() - t0
+    n, e = g.num_nodes, g.num_edges
+    dims = (16, 22)                  # aggregation widths of layer 0 and layer 1 (hidden, classes)
+
+    # synthetic inputs of the real shapes: projected features, and gradients that are
+    # zero outside the rows the corresponding mask allows (what autograd would deliver)
+    x16 = graphs.normal32(1, (n, 16), dev, 0)
+    x22 = graphs.normal32(1, (n, 22), dev, 1)
+    dy22 = graphs.normal32(1, (n, 22), dev, 2) * wl.train_mask[:, None]
+    dy16 = graphs.normal32(1, (n, 16), dev, 3) * wl.ngh_masks[0][:, None]
+    out16, out22 = torch.empty_like(x16), torch.empty_like(x22)
+    p_last, p_first = wl.paths[1], wl.paths[0]
+    if args.team:
+        capi.set_team_size(args.team)
+
+    def fwd16():
+        capi.spmm_forward(x16, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 32, 8,
+                          g.row_pointers, out16)
+
+    def fwd22():
+        capi.spmm_forward(x22, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 16, 8,
+                          g.row_pointers, out22)
+
+    def bwd22():
+        capi.ours_backward(dy22, p_last.ids, p_last.part_pointer, p_last.edge_list, g.degrees, p_last.num_parts,
+                           p_last.part_size, 2, 4, 16, out22)
+
+    def bwd16():
+        capi.ours_backward(dy16, p_first.ids, p_first.part_pointer, p_first.edge_list, g.degrees,
+                           p_first.num_parts, p_first.part_size, 1, 4, 16, out16)
+
+    kernels = [
+        ("fwd_agg_d16", fwd16, workload.bytes_forward(n, e, 16)),
+        ("fwd_agg_d22", fwd22, workload.bytes_forward(n, e, 22)),
+        ("bwd_agg_d22_last", bwd22, workload.bytes_pruned_backward(n, p_last.valid_len, p_last.num_parts, 22)),
+        ("bwd_agg_d16_first", bwd16, workload.bytes_pruned_backward(n, p_first.valid_len, p_first.num_parts, 16)),
+    ]
+    bytes_epoch = sum(k[2] for k in kernels)
+
+    def step():
+        for _, fn, _ in kernels:
+            fn()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = bytes_epoch / (ms_per_step * 1e-3) / 1e9
+
+    # per-kernel time: the library's own HIP events on the launch stream, around the
+    # aggregation kernel alone (the output clear is outside the bracket)
+    capi.set_timing(True)
+    per_kernel = {}
+    reps = max(3, min(args.steps, 10))
+    for name, fn, nbytes in kernels:
+        which = 0 if name.startswith("fwd") else 1
+        capi.clear_time()
+        for _ in range(reps):
+            fn()
+        ms = capi.get_time_ms(which) / reps
+        per_kernel[name] = {"ms": round(ms, 4), "alg_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1),
+                            "pct_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS * 100, 2)}
+    capi.set_timing(False)
+    capi.clear_time()
+    dominant = max(per_kernel, key=lambda k: per_kernel[k]["ms"])
+    dk = per_kernel[dominant]
+    roofline = {"bound": "hbm", "kernel": dominant, "achieved": dk["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(dk["GBps"] / PEAK_HBM_GBS, 4), "traffic": None,
+                "kernel_ms": dk["ms"], "alg_bytes_per_launch": dk["alg_bytes"]}
+
+    result = {
+        "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": args.config, "N": n, "E": e, "train_ratio": args.train_ratio,
+                   "agg_widths": list(dims), "forward_group_size": wl.part_size,
+                   "forward_groups": wl.num_parts, "backsize_mode": args.backsize_mode,
+                   "backward_group_size": [p.part_size for p in wl.paths],
+                   "kept_edges": [p.valid_len for p in wl.paths],
+                   "backward_groups": [p.num_parts for p in wl.paths], "max_degree": g.stats()["max_degree"]},
+        "agg_ms_per_epoch": round(ms_per_step, 4), "alg_bytes_per_epoch": bytes_epoch,
+        "pct_of_peak_hbm": round(value / PEAK_HBM_GBS * 100, 2),
+        "per_kernel": per_kernel, "path_preparation_s": round(prep_s, 3),
+        "roofline": roofline,
+    }
+
+    if not args.no_train:
+        try:
+            from eppgcn_amd import train
+            result["train"] = train.time_gpu_training(g, wl, epochs=args.train_epochs, warmup=10)
+        except Exception as exc:  # the training leg must never hide the kernel figures
+            result["train"] = {"error": repr(exc)}
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args, g, wl, x16, x22, dy22, dy16, bytes_epoch)
+        if not args.no_train and "error" not in result.get("train", {"error": 1}):
+            try:
+                from eppgcn_amd import train
+                result["cpu_torch_sparse"] = train.time_cpu_sparse_training(g, wl.train_mask, epochs=args.train_epochs)
+            except Exception as exc:
+                result["cpu_torch_sparse"] = {"error": repr(exc)}
+    print(json.dumps(result), flush=True)
+
+
+def cpu_baseline(args, g, wl, x16, x22, dy22, dy16, bytes_epoch):
+    """The CPU checker's OpenMP restatement of the same four aggregations, one epoch, on the
+    host cores.  A reported baseline, not a target."""
+    from oracle import c_oracle as co
+    co.load()
+    col = g.column_index.cpu().numpy()
+    s = g.degrees.cpu().numpy()
+    pp, p2n = wl.part_ptr.cpu().numpy(), wl.part2node.cpu().numpy()
+    n = g.num_nodes
+    host = {k: v.cpu().numpy() for k, v in (("x16", x16), ("x22", x22), ("dy22", dy22), ("dy16", dy16))}
+    paths = [(p.ids.cpu().numpy(), p.part_pointer.cpu().numpy(), p.edge_list.cpu().numpy(), p.num_parts)
+             for p in wl.paths]
+    t0 = time.perf_counter()
+    co.spmm_groups(host["x16"], col, s, pp, p2n, n, threads=True)
+    co.spmm_groups(host["x22"], col, s, pp, p2n, n, threads=True)
+    ids, bpp, el, npb = paths[1]
+    co.ours_backward(host["dy22"], ids, bpp, el, s, npb, threads=True)
+    ids, bpp, el, npb = paths[0]
+    co.ours_backward(host["dy16"], ids, bpp, el, s, npb, threads=True)
+    dt = time.perf_counter() - t0
+    return {"value": round(bytes_epoch / dt / 1e9, 2), "unit": "GB/s", "cores": co.num_threads(), "kind": "port",
+            "ms_per_epoch": round(dt * 1e3, 1),
+            "sample": f"one epoch (4 aggregations) of {args.config}, OpenMP C restatement, "
+                      f"{co.num_threads()} threads of {os.cpu_count()} host cpus"}
+
+
+if __name__ == "__main__":
+    main()

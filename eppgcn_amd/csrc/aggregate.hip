@@ -288,10 +288,11 @@ static hipError_t launch_slab(float* out, const float* in, const int* col, const
 
 template <class Groups>
 static int aggregate_dispatch(float* out, const float* in, const int* col, const float* scale, Groups g,
-                              int num_nodes, int dim, int num_parts, hipStream_t stream)
+                              int num_nodes, int dim, int num_parts, hipStream_t stream, double* sink, double* sink2)
 {
     EPPGCN_HIP(hipMemsetAsync(out, 0, static_cast<size_t>(num_nodes) * dim * sizeof(float), stream));
     if (num_parts == 0) return kOk;
+    KernelTimer timer(stream, sink, sink2);   // brackets the aggregation kernel(s) only, not the clear
     const uintptr_t bits = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(in);
     int vw = 1;
     if (dim % 4 == 0 && bits % 16 == 0) vw = 4;
@@ -310,18 +311,18 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
 
 int aggregate_forward_groups(float* out, const float* in, const int* col, const float* scale,
                              const int* part_ptr, const int* part2node, int num_nodes, int dim,
-                             int num_parts, hipStream_t stream)
+                             int num_parts, hipStream_t stream, double* sink, double* sink2)
 {
     return aggregate_dispatch(out, in, col, scale, ForwardGroups{part_ptr, part2node}, num_nodes, dim,
-                              num_parts, stream);
+                              num_parts, stream, sink, sink2);
 }
 
 int aggregate_compacted_groups(float* out, const float* in, const int* ids, const int* part_ptr,
                                const int* edge_list, const float* scale, int num_nodes, int dim,
-                               int num_parts, hipStream_t stream)
+                               int num_parts, hipStream_t stream, double* sink, double* sink2)
 {
     return aggregate_dispatch(out, in, edge_list, scale, CompactedGroups{part_ptr, ids}, num_nodes, dim,
-                              num_parts, stream);
+                              num_parts, stream, sink, sink2);
 }
 
 }  // namespace eppgcn

@@ -12,9 +12,9 @@ namespace eppgcn {
 
 // ---- implemented in aggregate.hip / prepare.hip
 int aggregate_forward_groups(float*, const float*, const int*, const float*, const int*, const int*, int, int, int,
-                             hipStream_t);
+                             hipStream_t, double*, double*);
 int aggregate_compacted_groups(float*, const float*, const int*, const int*, const int*, const float*, int, int, int,
-                               hipStream_t);
+                               hipStream_t, double*, double*);
 void set_agg_force_team(int);
 size_t compact_workspace_bytes(long long);
 size_t split_workspace_bytes(long long);
@@ -40,30 +40,7 @@ static bool g_timing = false;
 static double g_for_agg_ms = 0.0, g_back_agg_ms = 0.0, g_mask_ms = 0.0;
 static double g_layer_back_ms[kMaxTimedLayers] = {0};
 
-struct ScopedTimer {
-    hipStream_t stream;
-    double* sink;
-    double* sink2;
-    hipEvent_t start = nullptr, stop = nullptr;
-    ScopedTimer(hipStream_t s, double* a, double* b = nullptr) : stream(s), sink(a), sink2(b)
-    {
-        if (!g_timing) return;
-        if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) { start = nullptr; return; }
-        (void)hipEventRecord(start, stream);
-    }
-    ~ScopedTimer()
-    {
-        if (!start) return;
-        float ms = 0.f;
-        if (hipEventRecord(stop, stream) == hipSuccess && hipEventSynchronize(stop) == hipSuccess &&
-            hipEventElapsedTime(&ms, start, stop) == hipSuccess) {
-            *sink += ms;
-            if (sink2) *sink2 += ms;
-        }
-        (void)hipEventDestroy(start);
-        (void)hipEventDestroy(stop);
-    }
-};
+bool timing_enabled() { return g_timing; }
 
 static int read_state(void* workspace, hipStream_t stream, ScanState* host)
 {
@@ -98,9 +75,8 @@ int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers
     EPPGCN_REQUIRE(out && in && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (column_index && part_pointers && part2node), "null index pointer");
     EPPGCN_REQUIRE(aligned(out, 4) && aligned(in, 4), "feature pointers must be 4-byte aligned");
-    ScopedTimer t(static_cast<hipStream_t>(stream), &g_for_agg_ms);
     return aggregate_forward_groups(out, in, column_index, degrees, part_pointers, part2node, num_nodes, dim, num_parts,
-                                    static_cast<hipStream_t>(stream));
+                                    static_cast<hipStream_t>(stream), &g_for_agg_ms, nullptr);
 }
 
 int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* row_pointers,
@@ -115,9 +91,8 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
     EPPGCN_REQUIRE(d_input && d_output && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (column_index && part_pointers && part2node), "null index pointer");
     EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
-    ScopedTimer t(static_cast<hipStream_t>(stream), &g_back_agg_ms);
     return aggregate_forward_groups(d_input, d_output, column_index, degrees, part_pointers, part2node, num_nodes, dim,
-                                    num_parts, static_cast<hipStream_t>(stream));
+                                    num_parts, static_cast<hipStream_t>(stream), &g_back_agg_ms, nullptr);
 }
 
 int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
@@ -132,10 +107,9 @@ int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* i
     EPPGCN_REQUIRE(d_input && d_output && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (ids && part_pointer && edge_list), "null index pointer");
     EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
-    ScopedTimer t(static_cast<hipStream_t>(stream), &g_back_agg_ms,
-                  layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr);
     return aggregate_compacted_groups(d_input, d_output, ids, part_pointer, edge_list, degrees, num_nodes, dim,
-                                      num_parts, static_cast<hipStream_t>(stream));
+                                      num_parts, static_cast<hipStream_t>(stream), &g_back_agg_ms,
+                                      layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr);
 }
 
 int eppgcn_mask_forward(const int32_t* part2node, const int32_t* part_pointers, const int32_t* column_index,
@@ -148,7 +122,7 @@ int eppgcn_mask_forward(const int32_t* part2node, const int32_t* part_pointers, 
     EPPGCN_REQUIRE(part2node && part_pointers && column_index && src_mask && back_edge_mask && node_degs,
                    "null pointer");
     EPPGCN_REQUIRE(is_last_layer || ngh_mask, "ngh_mask may only be NULL on the last layer");
-    ScopedTimer t(static_cast<hipStream_t>(stream), &g_mask_ms);
+    KernelTimer t(static_cast<hipStream_t>(stream), &g_mask_ms);
     return launch_mask_forward(part2node, part_pointers, column_index, src_mask, ngh_mask, back_edge_mask, node_degs,
                                num_parts, num_edges, is_last_layer ? 1 : 0, static_cast<hipStream_t>(stream));
 }

@@ -40,6 +40,39 @@ int hip_fail(hipError_t e, const char* what);
         }                                                       \
     } while (0)
 
+// ---------------------------------------------------------------- kernel timers
+// Optional event timing of the kernels of one call (off by default: calls stay
+// asynchronous).  When enabled the destructor synchronises on the stop event and
+// adds the elapsed milliseconds to the sinks.
+bool timing_enabled();
+struct KernelTimer {
+    hipStream_t stream;
+    double* sink;
+    double* sink2;
+    hipEvent_t start = nullptr, stop = nullptr;
+    KernelTimer(hipStream_t s, double* a, double* b = nullptr) : stream(s), sink(a), sink2(b)
+    {
+        if (!a || !timing_enabled()) return;
+        if (hipEventCreate(&start) != hipSuccess) { start = nullptr; return; }
+        if (hipEventCreate(&stop) != hipSuccess) { (void)hipEventDestroy(start); start = nullptr; return; }
+        (void)hipEventRecord(start, stream);
+    }
+    ~KernelTimer()
+    {
+        if (!start) return;
+        float ms = 0.f;
+        if (hipEventRecord(stop, stream) == hipSuccess && hipEventSynchronize(stop) == hipSuccess &&
+            hipEventElapsedTime(&ms, start, stop) == hipSuccess) {
+            *sink += ms;
+            if (sink2) *sink2 += ms;
+        }
+        (void)hipEventDestroy(start);
+        (void)hipEventDestroy(stop);
+    }
+    KernelTimer(const KernelTimer&) = delete;
+    KernelTimer& operator=(const KernelTimer&) = delete;
+};
+
 // ---------------------------------------------------------------- lane helpers
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 

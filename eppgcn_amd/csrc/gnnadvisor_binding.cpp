@@ -1,0 +1,285 @@
+// Python extension module `GNNAdvisor` for PyTorch-ROCm: the twelve functions the
+// reference's Python calls (EPPGCN/GCNConv/EPPGCN.cpp:388-403), same positional
+// signatures, implemented over the C ABI of libeppgcn_hip.so.  torch supplies the
+// tensors, the dense X*W products and the current HIP stream; everything else
+// happens in the HIP library.  Host C++ only: no device code in this file.
+//
+// Differences from the reference binding, all deliberate:
+//   - errors raise (RuntimeError in Python) instead of printf + exit(-1);
+//   - work is issued on torch's current stream and is asynchronous unless a host
+//     value is returned;
+//   - build_part computes on the device and returns int32 tensors (the reference
+//     loops on the CPU and returns float32, which corrupts offsets above 2^24);
+//   - compact_back_edge's info tensor is float64 so that int(info[0].item()) is
+//     exact for any edge count;
+//   - split_back_part's part_pointer has num_edges + 1 entries, so the terminator
+//     is always in bounds;
+//   - get_map_back_part_size never returns less than 1.
+#include <torch/extension.h>
+
+#include <c10/hip/HIPStream.h>
+
+#include <vector>
+
+#include "eppgcn_hip.h"
+
+namespace {
+
+using torch::Tensor;
+
+void check(int rc, const char* what)
+{
+    TORCH_CHECK(rc == 0, what, " failed (", rc, "): ", eppgcn_last_error());
+}
+
+#define CHECK_DEVICE(x) TORCH_CHECK((x).is_cuda(), #x " must be a GPU tensor")
+#define CHECK_CONTIGUOUS(x) TORCH_CHECK((x).is_contiguous(), #x " must be contiguous")
+#define CHECK_INPUT(x) \
+    CHECK_DEVICE(x);   \
+    CHECK_CONTIGUOUS(x)
+#define CHECK_I32(x) \
+    CHECK_INPUT(x);  \
+    TORCH_CHECK((x).scalar_type() == torch::kInt32, #x " must be int32")
+#define CHECK_F32(x) \
+    CHECK_INPUT(x);  \
+    TORCH_CHECK((x).scalar_type() == torch::kFloat32, #x " must be float32")
+#define CHECK_MASK(x) \
+    CHECK_INPUT(x);   \
+    TORCH_CHECK((x).scalar_type() == torch::kBool || (x).scalar_type() == torch::kUInt8, #x " must be bool")
+
+void* stream_of(const Tensor& t)
+{
+    return static_cast<void*>(c10::hip::getCurrentHIPStream(t.get_device()).stream());
+}
+
+const int32_t* i32(const Tensor& t) { return t.numel() ? t.data_ptr<int32_t>() : nullptr; }
+const float* f32(const Tensor& t) { return t.numel() ? t.data_ptr<float>() : nullptr; }
+
+Tensor workspace(size_t bytes, const Tensor& like)
+{
+    return torch::empty({static_cast<int64_t>((bytes + 7) / 8)}, like.options().dtype(torch::kInt64));
+}
+
+// ---------------------------------------------------------------- forward / backward
+std::vector<Tensor> forward(Tensor input, Tensor weight, Tensor row_pointers, Tensor column_index, Tensor degrees,
+                            Tensor part_pointers, Tensor part2Node, int partSize, int dimWorker, int warpPerBlock)
+{
+    CHECK_F32(input); CHECK_F32(weight); CHECK_I32(row_pointers); CHECK_I32(column_index);
+    CHECK_F32(degrees); CHECK_I32(part_pointers); CHECK_I32(part2Node);
+    TORCH_CHECK(input.dim() == 2 && weight.dim() == 2 && input.size(1) == weight.size(0), "shape mismatch");
+    TORCH_CHECK(degrees.numel() == input.size(0), "degrees must have one entry per vertex");
+    TORCH_CHECK(part_pointers.numel() >= part2Node.numel() + 1, "part_pointers needs num_parts + 1 entries");
+    auto tmp = torch::mm(input, weight);
+    auto output = torch::empty_like(tmp);
+    check(eppgcn_spmm_forward(output.data_ptr<float>(), tmp.data_ptr<float>(), i32(row_pointers), i32(column_index),
+                              f32(degrees), i32(part_pointers), i32(part2Node), static_cast<int>(tmp.size(0)),
+                              static_cast<int>(tmp.size(1)), static_cast<int>(part2Node.numel()), partSize, dimWorker,
+                              warpPerBlock, stream_of(input)),
+          "forward");
+    return {output};
+}
+
+std::vector<Tensor> backward(Tensor d_output, Tensor X, Tensor W, Tensor row_pointers, Tensor column_index,
+                             Tensor degrees, Tensor part_pointers, Tensor part2Node, int partSize, int dimWorker,
+                             int warpPerBlock)
+{
+    CHECK_F32(d_output); CHECK_F32(X); CHECK_F32(W); CHECK_I32(row_pointers); CHECK_I32(column_index);
+    CHECK_F32(degrees); CHECK_I32(part_pointers); CHECK_I32(part2Node);
+    TORCH_CHECK(d_output.dim() == 2 && degrees.numel() == d_output.size(0), "shape mismatch");
+    TORCH_CHECK(part_pointers.numel() >= part2Node.numel() + 1, "part_pointers needs num_parts + 1 entries");
+    auto d_input_prime = torch::empty_like(d_output);
+    check(eppgcn_spmm_backward(d_input_prime.data_ptr<float>(), d_output.data_ptr<float>(), i32(row_pointers),
+                               i32(column_index), f32(degrees), i32(part_pointers), i32(part2Node),
+                               static_cast<int>(d_output.size(0)), static_cast<int>(d_output.size(1)),
+                               static_cast<int>(part2Node.numel()), partSize, dimWorker, warpPerBlock,
+                               stream_of(d_output)),
+          "backward");
+    auto d_input = torch::mm(d_input_prime, W.transpose(0, 1));
+    auto d_weight = torch::mm(X.transpose(0, 1), d_input_prime);
+    return {d_input, d_weight};
+}
+
+void mask_forward(Tensor id, Tensor partPointer, Tensor edgeList, Tensor src_mask, Tensor ngh_mask,
+                  Tensor backEdgeMask, Tensor node_degs, int num_layers, int layer, int blockx, int blocky)
+{
+    CHECK_I32(id); CHECK_I32(partPointer); CHECK_I32(edgeList); CHECK_MASK(src_mask); CHECK_MASK(ngh_mask);
+    CHECK_I32(backEdgeMask); CHECK_I32(node_degs);
+    const bool is_last = layer == num_layers;
+    TORCH_CHECK(partPointer.numel() >= id.numel() + 1, "partPointer needs num_parts + 1 entries");
+    TORCH_CHECK(backEdgeMask.numel() >= edgeList.numel(), "backEdgeMask is shorter than the edge list");
+    TORCH_CHECK(src_mask.numel() == node_degs.numel(), "src_mask and node_degs must have one entry per vertex");
+    TORCH_CHECK(is_last || ngh_mask.numel() == node_degs.numel(), "ngh_mask must have one entry per vertex");
+    check(eppgcn_mask_forward(i32(id), i32(partPointer), i32(edgeList),
+                              static_cast<const uint8_t*>(src_mask.data_ptr()),
+                              ngh_mask.numel() ? static_cast<uint8_t*>(ngh_mask.data_ptr()) : nullptr,
+                              backEdgeMask.data_ptr<int32_t>(), node_degs.data_ptr<int32_t>(),
+                              static_cast<int>(id.numel()), edgeList.numel(), is_last ? 1 : 0, blockx, blocky,
+                              stream_of(id)),
+          "mask_forward");
+}
+
+std::vector<Tensor> ours_backward(Tensor d_output, Tensor X, Tensor W, Tensor id, Tensor partPointer, Tensor edgeList,
+                                  Tensor degrees, int partSize, int numParts, int layer, int blockx, int blocky)
+{
+    CHECK_F32(d_output); CHECK_F32(X); CHECK_F32(W); CHECK_I32(id); CHECK_I32(partPointer); CHECK_I32(edgeList);
+    CHECK_F32(degrees);
+    TORCH_CHECK(d_output.dim() == 2 && degrees.numel() == d_output.size(0), "shape mismatch");
+    TORCH_CHECK(numParts >= 0 && partPointer.numel() >= static_cast<int64_t>(numParts) + 1,
+                "partPointer needs numParts + 1 entries");
+    auto d_input_prime = torch::empty_like(d_output);
+    check(eppgcn_ours_backward(d_input_prime.data_ptr<float>(), d_output.data_ptr<float>(), i32(id), i32(partPointer),
+                               i32(edgeList), f32(degrees), static_cast<int>(d_output.size(0)),
+                               static_cast<int>(d_output.size(1)), numParts, partSize > 0 ? partSize : 1, layer, blockx,
+                               blocky, stream_of(d_output)),
+          "ours_backward");
+    auto d_input = torch::mm(d_input_prime, W.transpose(0, 1));
+    auto d_weight = torch::mm(X.transpose(0, 1), d_input_prime);
+    return {d_input, d_weight};
+}
+
+// ---------------------------------------------------------------- path preparation
+std::vector<Tensor> build_part(int partSize, Tensor indptr)
+{
+    TORCH_CHECK(partSize >= 1, "partSize must be >= 1");
+    TORCH_CHECK(indptr.scalar_type() == torch::kInt32 && indptr.dim() == 1 && indptr.numel() >= 1,
+                "indptr must be a 1-D int32 tensor");
+    auto dptr = indptr.is_cuda() ? indptr.contiguous() : indptr.contiguous().to(torch::kCUDA);
+    const int num_nodes = static_cast<int>(dptr.numel() - 1);
+    const int64_t num_edges = (dptr[num_nodes] - dptr[0]).item<int64_t>();
+    const int64_t capacity = num_edges / partSize + num_nodes + 1;
+    auto part_ptr = torch::empty({capacity}, dptr.options());
+    auto part2node = torch::empty({capacity > 1 ? capacity - 1 : 1}, dptr.options());
+    const size_t bytes = eppgcn_split_workspace_bytes(num_nodes);
+    auto ws = workspace(bytes, dptr);
+    int64_t num_parts = 0;
+    check(eppgcn_build_part(dptr.data_ptr<int32_t>(), num_nodes, partSize, part_ptr.data_ptr<int32_t>(),
+                            part2node.data_ptr<int32_t>(), capacity, ws.data_ptr(), bytes, nullptr, &num_parts,
+                            stream_of(dptr)),
+          "build_part");
+    return {part_ptr.narrow(0, 0, num_parts + 1), part2node.narrow(0, 0, num_parts)};
+}
+
+struct Compacted {
+    Tensor id, edge_list;
+    int64_t valid_len;
+};
+
+Compacted compact(const Tensor& edge_mask, const Tensor& column_index)
+{
+    CHECK_I32(edge_mask); CHECK_I32(column_index);
+    TORCH_CHECK(column_index.numel() >= edge_mask.numel(), "column_index is shorter than edge_mask");
+    const int64_t length = edge_mask.numel();
+    Compacted c{torch::empty_like(edge_mask), torch::empty({length}, column_index.options()), 0};
+    const size_t bytes = eppgcn_compact_workspace_bytes(length);
+    auto ws = workspace(bytes, edge_mask);
+    check(eppgcn_compact_back_edge(i32(edge_mask), i32(column_index), c.id.data_ptr<int32_t>(),
+                                   c.edge_list.data_ptr<int32_t>(), length, ws.data_ptr(), bytes, nullptr,
+                                   &c.valid_len, stream_of(edge_mask)),
+          "compact_back_edge");
+    return c;
+}
+
+int64_t valid_nodes(const Tensor& node_deg)
+{
+    CHECK_I32(node_deg);
+    auto d = torch::empty({1}, node_deg.options());
+    int64_t v = 0;
+    check(eppgcn_count_nonzero(i32(node_deg), node_deg.numel(), d.data_ptr<int32_t>(), &v, stream_of(node_deg)),
+          "count_nonzero");
+    return v;
+}
+
+struct Split {
+    Tensor part_pointer;
+    int64_t num_parts;
+};
+
+Split split(const Tensor& node_deg, int64_t num_edges, int part_size)
+{
+    CHECK_I32(node_deg);
+    TORCH_CHECK(part_size >= 1, "back_part_size must be >= 1");
+    TORCH_CHECK(num_edges >= 0, "num_edges must be >= 0");
+    Split s{torch::empty({num_edges + 1}, node_deg.options()), 0};
+    const size_t bytes = eppgcn_split_workspace_bytes(node_deg.numel());
+    auto ws = workspace(bytes, node_deg);
+    check(eppgcn_split_back_part(i32(node_deg), static_cast<int>(node_deg.numel()), part_size,
+                                 s.part_pointer.data_ptr<int32_t>(), num_edges + 1, ws.data_ptr(), bytes, nullptr,
+                                 &s.num_parts, nullptr, stream_of(node_deg)),
+          "split_back_part");
+    return s;
+}
+
+std::vector<Tensor> compact_back_edge(Tensor edge_mask, Tensor column_index)
+{
+    auto c = compact(edge_mask, column_index);
+    auto info = torch::zeros({1}, torch::kFloat64);
+    info[0] = static_cast<double>(c.valid_len);
+    return {c.id, c.edge_list, info};
+}
+
+int get_map_back_part_size(Tensor node_deg, int valid_len)
+{
+    int clamped = 0;
+    const int ps = eppgcn_map_back_part_size(valid_nodes(node_deg), valid_len, &clamped);
+    if (clamped)
+        TORCH_WARN_ONCE("get_map_back_part_size: the fitted regression gives a group size below 1 for this graph; "
+                        "using 1 (pass a constant group size instead)");
+    return ps;
+}
+
+std::vector<Tensor> split_back_part(Tensor node_deg, int num_edges, int back_part_size)
+{
+    auto s = split(node_deg, num_edges, back_part_size);
+    auto info = torch::zeros({1}, torch::kInt32);
+    info[0] = static_cast<int>(s.num_parts);
+    return {s.part_pointer, info};
+}
+
+// Legacy all-in-one (EPPGCN.cpp:229-280): compaction, threshold rule when back_part_size == 0, split.
+std::vector<Tensor> build_back_part(Tensor edge_mask, Tensor column_index, Tensor node_deg, int back_part_size, int dim)
+{
+    (void)dim;
+    auto c = compact(edge_mask, column_index);
+    if (back_part_size == 0) {
+        back_part_size = eppgcn_threshold_back_part_size(valid_nodes(node_deg), c.valid_len);
+        TORCH_CHECK(back_part_size > 0, "build_back_part: the threshold rule has no group size for an average kept "
+                                        "degree >= 512; pass back_part_size explicitly");
+    }
+    auto s = split(node_deg, edge_mask.numel(), back_part_size);
+    auto info = torch::zeros({2}, torch::kFloat64);
+    info[0] = static_cast<double>(back_part_size);
+    info[1] = static_cast<double>(s.num_parts);
+    return {c.id, c.edge_list, s.part_pointer, info};
+}
+
+Tensor get_ginfo(Tensor node_deg, int valid_len)
+{
+    CHECK_I32(node_deg);
+    auto hist = torch::empty({10}, node_deg.options());
+    auto re = torch::zeros({10}, torch::kFloat32);
+    check(eppgcn_get_ginfo(i32(node_deg), node_deg.numel(), valid_len, hist.data_ptr<int32_t>(), re.data_ptr<float>(),
+                           stream_of(node_deg)),
+          "get_ginfo");
+    return re;
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
+{
+    m.def("forward", &forward, "neighbour-group forward: mm + aggregation (HIP)");
+    m.def("backward", &backward, "unpruned backward: aggregation + 2 mm (HIP)");
+    m.def("mask_forward", &mask_forward, "mark the backward execution path of one layer (HIP)");
+    m.def("ours_backward", &ours_backward, "pruned backward over the compacted path: aggregation + 2 mm (HIP)");
+    m.def("print_time", &eppgcn_print_time, "print accumulated kernel times");
+    m.def("clear_time", &eppgcn_clear_time, "reset accumulated kernel times");
+    m.def("set_timing", [](bool on) { eppgcn_set_timing(on ? 1 : 0); }, "enable per-call kernel timing");
+    m.def("get_time_ms", &eppgcn_get_time_ms, "accumulated kernel time in ms");
+
+    m.def("build_part", &build_part, "forward neighbour groups (HIP)");
+    m.def("build_back_part", &build_back_part, "compaction + group split in one call (HIP)");
+    m.def("compact_back_edge", &compact_back_edge, "compact the kept edges of one layer (HIP)");
+    m.def("get_map_back_part_size", &get_map_back_part_size, "backward group size from the fitted regression");
+    m.def("split_back_part", &split_back_part, "split kept edges into backward groups (HIP)");
+    m.def("get_ginfo", &get_ginfo, "degree-distribution features of the kept path");
+}

@@ -1,0 +1,205 @@
+"""GPU tests of the `GNNAdvisor` extension module and the autograd layer on top of it: the
+twelve reference exports with their positional signatures, error behaviour (raise, never abort),
+gradients against a dense float64 model, and the end-to-end loss trajectory against the host-CPU
+sparse trainer."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from oracle import closed_forms as cf
+from tests.helpers import hub_csr, random_symmetric_csr, scale_inv_sqrt
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def GNNA():
+    import eppgcn_amd
+    mod = eppgcn_amd.gnnadvisor()
+    import GNNAdvisor            # the reference's import line works after gnnadvisor()
+    assert GNNAdvisor is mod
+    return mod
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def test_exports_match_the_reference_surface(GNNA):
+    for name in ["forward", "backward", "mask_forward", "ours_backward", "print_time", "clear_time", "build_part",
+                 "build_back_part", "compact_back_edge", "get_map_back_part_size", "split_back_part", "get_ginfo"]:
+        assert callable(getattr(GNNA, name))
+
+
+def test_build_part_accepts_cpu_indptr_and_returns_int32(GNNA):
+    indptr, col = hub_csr(3000, 2000, 1)
+    for ps in (1, 7, 32):
+        want_pp, want_p2n = co.build_part(ps, indptr)
+        for t in (torch.from_numpy(indptr), dev(indptr)):
+            pp, p2n = GNNA.build_part(ps, t)
+            # the reference's caller then does .int().to(device): both must be no-ops
+            pp, p2n = pp.int().to("cuda"), p2n.int().to("cuda")
+            assert pp.dtype == torch.int32 and np.array_equal(pp.cpu().numpy(), want_pp)
+            assert np.array_equal(p2n.cpu().numpy(), want_p2n)
+
+
+def test_forward_and_both_backwards_with_dense_products(GNNA):
+    indptr, col = hub_csr(2000, 1500, 2)
+    n = indptr.size - 1
+    rng = np.random.default_rng(0)
+    s = scale_inv_sqrt(indptr)
+    x = rng.standard_normal((n, 96)).astype(np.float32)
+    w = rng.uniform(-0.25, 0.25, (96, 16)).astype(np.float32)
+    pp, p2n = co.build_part(6, indptr)
+    args = (dev(indptr), dev(col), dev(s), dev(pp), dev(p2n), 6, 16, 8)
+    y = GNNA.forward(dev(x), dev(w), *args)[0].cpu().numpy()
+    t64 = x.astype(np.float64) @ w.astype(np.float64)
+    want = cf.aggregate_csr64(indptr, col, s, t64)
+    assert np.linalg.norm(y - want) / np.linalg.norm(want) < 1e-5
+
+    src = rng.random(n) < 0.2
+    dy = (rng.standard_normal((n, 16)) * src[:, None]).astype(np.float32)
+    g64 = cf.aggregate_csr64(indptr, col, s, dy)
+    want_dx, want_dw = g64 @ w.T.astype(np.float64), x.T.astype(np.float64) @ g64
+    dx, dw = GNNA.backward(dev(dy), dev(x), dev(w), *args)
+    assert np.linalg.norm(dx.cpu().numpy() - want_dx) / np.linalg.norm(want_dx) < 1e-5
+    assert np.linalg.norm(dw.cpu().numpy() - want_dw) / np.linalg.norm(want_dw) < 1e-5
+
+    # pruned path through the module's own preparation functions
+    e = col.size
+    bem = torch.full((e,), -1, dtype=torch.int32, device="cuda")
+    degs = torch.zeros(n, dtype=torch.int32, device="cuda")
+    GNNA.mask_forward(dev(p2n), dev(pp), dev(col), dev(src), torch.zeros(0, dtype=torch.bool, device="cuda"),
+                      bem, degs, 2, 2, 4, 16)
+    ids, edge_list, info = GNNA.compact_back_edge(bem, dev(col))
+    v = int(info[0].item())
+    assert v == int(src[col].sum()) and not info.is_cuda
+    ps = GNNA.get_map_back_part_size(degs, v)
+    assert ps == max(1, cf.map_back_part_size(cf.compact_count(degs.cpu().numpy()), v))
+    part_pointer, pinfo = GNNA.split_back_part(degs, e, ps)
+    want_pp, want_p = cf.split_back_part(degs.cpu().numpy(), e, ps)
+    assert int(pinfo[0].item()) == want_p and pinfo.dtype == torch.int32 and not pinfo.is_cuda
+    assert np.array_equal(part_pointer.cpu().numpy(), want_pp)
+    dx2, dw2 = GNNA.ours_backward(dev(dy), dev(x), dev(w), ids, part_pointer, edge_list, dev(s), ps, want_p, 1, 4, 16)
+    assert np.linalg.norm(dx2.cpu().numpy() - want_dx) / np.linalg.norm(want_dx) < 1e-5
+    assert np.linalg.norm(dw2.cpu().numpy() - want_dw) / np.linalg.norm(want_dw) < 1e-5
+
+    # legacy all-in-one call: same lists, threshold group size
+    ids3, el3, pp3, info3 = GNNA.build_back_part(bem, dev(col), degs, 0, 16)
+    ps3 = cf.threshold_back_part_size(cf.compact_count(degs.cpu().numpy()), v)
+    assert int(info3[0].item()) == ps3
+    want_pp3, want_p3 = cf.split_back_part(degs.cpu().numpy(), e, ps3)
+    assert int(info3[1].item()) == want_p3 and np.array_equal(pp3.cpu().numpy(), want_pp3)
+    assert torch.equal(ids3, ids) and torch.equal(el3, edge_list)
+    assert np.allclose(GNNA.get_ginfo(degs, v).numpy(), cf.get_ginfo(degs.cpu().numpy(), v), rtol=1e-6)
+
+
+def test_argument_errors_raise_runtime_error(GNNA):
+    x = torch.randn(8, 4, device="cuda")
+    w = torch.randn(4, 3, device="cuda")
+    i = torch.zeros(9, dtype=torch.int32, device="cuda")
+    s = torch.ones(8, device="cuda")
+    with pytest.raises(RuntimeError):
+        GNNA.forward(x.cpu(), w, i, i, s, i, i[:8], 1, 1, 1)                  # not on the GPU
+    with pytest.raises(RuntimeError):
+        GNNA.forward(x.t(), w, i, i, s, i, i[:8], 1, 1, 1)                   # not contiguous / wrong shape
+    with pytest.raises(RuntimeError):
+        GNNA.forward(x, w, i.long(), i, s, i, i[:8], 1, 1, 1)                # wrong index dtype
+    with pytest.raises(RuntimeError):
+        GNNA.forward(x, w, i, i, s, i[:3], i[:8], 1, 1, 1)                   # part pointers too short
+    with pytest.raises(RuntimeError):
+        GNNA.split_back_part(i, 10, 0)                                       # group size 0
+    with pytest.raises(RuntimeError):
+        GNNA.compact_back_edge(i.float(), i)                                 # wrong dtype
+    assert torch.isfinite(x).all()                                           # the process is still alive
+
+
+def _dense_model_grads(indptr, col, s, x, w0, w1, train, y):
+    """float64 autograd of the same 2-layer model with a dense normalised adjacency."""
+    n = indptr.size - 1
+    a = torch.zeros(n, n, dtype=torch.float64)
+    a[torch.from_numpy(cf.row_index(indptr)), torch.from_numpy(col.astype(np.int64))] = 1.0
+    w32 = (torch.from_numpy(s)[:, None] * torch.from_numpy(s)[None, :]).double()
+    a = a * w32
+    w0 = torch.tensor(w0, dtype=torch.float64, requires_grad=True)
+    w1 = torch.tensor(w1, dtype=torch.float64, requires_grad=True)
+    h = torch.relu(a @ (torch.from_numpy(x).double() @ w0))
+    out = a @ (h @ w1)
+    loss = torch.nn.functional.nll_loss(torch.log_softmax(out, 1)[torch.from_numpy(train)], torch.from_numpy(y)[torch.from_numpy(train)])
+    loss.backward()
+    return float(loss), w0.grad.numpy(), w1.grad.numpy()
+
+
+def test_autograd_layer_gradients_vs_dense_float64(GNNA):
+    from eppgcn_amd import graphs, train
+    indptr, col = random_symmetric_csr(400, 1500, 3)
+    n = indptr.size - 1
+    g = graphs.Graph("t", n, dev(indptr), dev(col), dev(scale_inv_sqrt(indptr)))
+    rng = np.random.default_rng(1)
+    mask = rng.random(n) < 0.15
+    tr = train.Trainer(g, dim=24, hidden=16, num_classes=22, train_mask=torch.from_numpy(mask), backsize=4,
+                       labels="uniform")
+    x = tr.dataset.x.cpu().numpy()
+    y = tr.dataset.y.cpu().numpy()
+    w0 = tr.model.convs[0].weights.detach().cpu().numpy()
+    w1 = tr.model.convs[1].weights.detach().cpu().numpy()
+    want_loss, want_g0, want_g1 = _dense_model_grads(indptr, col, scale_inv_sqrt(indptr), x, w0, w1, mask, y)
+    tr.optimizer = torch.optim.SGD(tr.model.parameters(), lr=0.0)      # keep the weights fixed
+    loss = tr.train_step(True)
+    assert abs(float(loss) - want_loss) < 1e-5 * max(1.0, abs(want_loss))
+    g0 = tr.model.convs[0].weights.grad.cpu().numpy()
+    g1 = tr.model.convs[1].weights.grad.cpu().numpy()
+    assert np.linalg.norm(g0 - want_g0) / np.linalg.norm(want_g0) < 1e-4
+    assert np.linalg.norm(g1 - want_g1) / np.linalg.norm(want_g1) < 1e-4
+    # later iterations reuse the prepared path and give the same gradients
+    tr.train_step(False)
+    assert np.allclose(tr.model.convs[0].weights.grad.cpu().numpy(), g0, rtol=1e-4, atol=1e-7)
+
+
+@pytest.mark.parametrize("cfg", ["cfg1_uniform", "cfg2_chunglu"])
+def test_loss_trajectory_matches_cpu_sparse_trainer(GNNA, cfg):
+    """Same seeds -> the GPU path and the CPU-sparse baseline follow the same loss curve."""
+    import torch.nn.functional as F
+    from eppgcn_amd import graphs, train
+    g_cpu = graphs.make_graph(cfg)
+    g = g_cpu.to("cuda")
+    mask = graphs.bernoulli_mask(g.num_nodes, 0.1)
+    tr = train.Trainer(g, train_mask=mask, backsize_mode="map", labels="uniform")
+    gpu_losses = [float(tr.train_step(i == 0)) for i in range(100)]
+
+    n = g_cpu.num_nodes
+    row = g_cpu.row_index()
+    a = torch.sparse_csr_tensor(g_cpu.row_pointers.long(), g_cpu.column_index.long(),
+                                (g_cpu.degrees[row] * g_cpu.degrees[g_cpu.column_index.long()]).double(), size=(n, n))
+    x = graphs.normal32(1, (n, 96)).double()
+    y = graphs.uniform_labels(4, n, 22)
+    w0 = graphs.uniform_weights(3, 96, 16).double().requires_grad_()
+    w1 = graphs.uniform_weights(4, 16, 22).double().requires_grad_()
+    opt = torch.optim.Adam([w0, w1], lr=0.01)
+    cpu_losses = []
+    for _ in range(100):
+        opt.zero_grad()
+        out = torch.sparse.mm(a, torch.relu(torch.sparse.mm(a, x @ w0)) @ w1)
+        loss = F.nll_loss(F.log_softmax(out, 1)[mask], y[mask])
+        loss.backward()
+        opt.step()
+        cpu_losses.append(float(loss))
+    gpu_losses, cpu_losses = np.array(gpu_losses), np.array(cpu_losses)
+    assert cpu_losses[-1] < cpu_losses[0]
+    assert np.max(np.abs(gpu_losses - cpu_losses) / np.abs(cpu_losses)) < 2e-3
+
+
+def test_print_time_lines(GNNA, capfd):
+    from eppgcn_amd import graphs, train
+    g = graphs.make_graph("cfg1_uniform", device="cuda")
+    tr = train.Trainer(g)
+    res = tr.run(epochs=3, warmup=2, kernel_timing=True)
+    assert res["for_agg_time"] > 0 and res["back_agg_time"] > 0
+    GNNA.set_timing(True)
+    tr.train_step(False)
+    GNNA.set_timing(False)
+    tr.model.convs[0].print_time()
+    out = capfd.readouterr().out
+    for key in ("for_agg_time:", "back_agg_time:", "l1_back_agg_time:", "l2_back_agg_time:", "mask_time:"):
+        assert key in out

@@ -1,0 +1,103 @@
+"""CPU tests of the host-side pieces: benchmark graph generators, parameter records, byte
+accounting.  No GPU, no HIP calls."""
+import numpy as np
+import pytest
+import torch
+
+from eppgcn_amd import graphs, param, workload
+
+
+def _check_graph(g):
+    indptr, col = g.row_pointers.numpy().astype(np.int64), g.column_index.numpy().astype(np.int64)
+    n = g.num_nodes
+    assert indptr[0] == 0 and indptr[-1] == col.size and indptr.size == n + 1
+    row = np.repeat(np.arange(n), np.diff(indptr))
+    keys = row * n + col
+    assert np.all(np.diff(keys) > 0), "columns sorted and unique inside each row"
+    assert np.array_equal(np.sort(col * n + row), keys), "symmetric"
+    assert np.all(np.isin(np.arange(n) * n + np.arange(n), keys)), "one self-loop per vertex"
+    deg = np.diff(indptr)
+    assert np.allclose(g.degrees.numpy(), 1 / np.sqrt(deg), rtol=1e-6)
+
+
+def test_cfg1_uniform_graph_matches_the_configuration():
+    g = graphs.make_graph("cfg1_uniform")
+    assert (g.num_nodes, g.num_edges) == (2708, 2 * 5278 + 2708)
+    _check_graph(g)
+    assert torch.equal(g.column_index, graphs.make_graph("cfg1_uniform").column_index)   # seeded
+
+
+def test_cfg2_chung_lu_graph_matches_the_configuration():
+    g = graphs.make_graph("cfg2_chunglu")
+    assert (g.num_nodes, g.num_edges) == (19717, 2 * 44325 + 19717)
+    _check_graph(g)
+    deg = np.diff(g.row_pointers.numpy())
+    assert deg.max() > 50 * np.median(deg)        # heavy tail
+
+
+def test_rmat_generator_is_skewed_and_device_independent_arithmetic():
+    g = graphs.rmat_graph(12, 8, seed=0)
+    _check_graph(g)
+    assert g.num_nodes == 4096 and 30000 < g.num_edges <= 2 * 8 * 4096 + 4096
+    deg = np.diff(g.row_pointers.numpy())
+    assert deg.max() > 20 * deg.mean()
+    # quadrant probabilities: the top-left quadrant of the first level gets ~a of the pairs
+    src, dst = graphs.rmat_pairs(12, 200000, seed=1)
+    top_left = ((src < 2048) & (dst < 2048)).double().mean().item()
+    assert abs(top_left - 0.57) < 0.01
+    bottom_right = ((src >= 2048) & (dst >= 2048)).double().mean().item()
+    assert abs(bottom_right - 0.05) < 0.01
+
+
+def test_scale_vector_both_fillings():
+    indptr = torch.tensor([0, 4, 4, 13], dtype=torch.int32)
+    assert torch.allclose(graphs.scale_vector(indptr, "inv_sqrt"), torch.tensor([0.5, 1.0, 1 / 3]))
+    assert torch.allclose(graphs.scale_vector(indptr, "sqrt"), torch.tensor([2.0, 1.0, 3.0]))
+
+
+def test_mask_weights_features_are_seeded_and_distributed():
+    m = graphs.bernoulli_mask(200000, 0.1, 2)
+    assert abs(m.double().mean().item() - 0.1) < 0.005 and torch.equal(m, graphs.bernoulli_mask(200000, 0.1, 2))
+    w = graphs.uniform_weights(3, 96, 16)
+    assert w.abs().max() <= 0.25 and abs(w.mean().item()) < 0.02
+    x = graphs.normal32(1, (50000, 4))
+    assert abs(x.mean().item()) < 0.02 and abs(x.std().item() - 1) < 0.02
+
+
+def test_get_block_size_table_is_one_wavefront():
+    for dim, want in [(1, (2, 32)), (7, (2, 32)), (8, (4, 16)), (16, (4, 16)), (22, (4, 16)), (31, (4, 16)),
+                      (32, (8, 8)), (95, (8, 8)), (96, (16, 4)), (191, (16, 4)), (192, (32, 2)), (256, (32, 2)),
+                      (4096, (32, 2))]:
+        assert param.getBlockSize(dim) == want
+        assert want[0] * want[1] == 64
+
+
+class _DS:
+    num_nodes, avg_degree, num_features = 1000, 31.6, 96
+
+
+def test_decider_rules():
+    info = param.inputProperty(None, None, None, 32, 32, 8, 100, hiddenDim=16, dataset_obj=_DS(), manual_mode=False)
+    info.decider()
+    assert info.partSize == 31 and info.warpPerBlock_input == 8 and info.warpPerBlock_hidden == 8
+    assert info.set_input().dimWorker == 32 and info.set_hidden().dimWorker == 16
+    ds = _DS()
+    ds.avg_degree = 0.4
+    info = param.inputProperty(None, None, None, 32, 32, 8, 100, hiddenDim=16, dataset_obj=ds, manual_mode=False)
+    info.decider()
+    assert info.partSize == 1                      # never 0
+    info = param.inputProperty(None, None, None, 5, 32, 8, 100, hiddenDim=16, dataset_obj=_DS(), manual_mode=True)
+    info.decider()
+    assert info.partSize == 5                      # manual group size respected
+    with pytest.raises(ValueError):
+        param.inputProperty()
+
+
+def test_algorithmic_bytes_nominal_values():
+    n, e = 4_194_304, 134_000_000
+    assert abs(workload.bytes_forward(n, e, 16) / 1e9 - 9.95) < 0.05
+    assert abs(workload.bytes_forward(n, e, 22) / 1e9 - 13.27) < 0.05
+    assert workload.bytes_forward(10, 100, 16) == 100 * 72 + 10 * 72
+    assert workload.bytes_pruned_backward(10, 50, 7, 22) == 50 * 96 + 10 * 88 + 56
+    assert workload.bytes_compact(100, 10) == 400 + 120
+    assert workload.bytes_compulsory(10, 100, 16) == 400 + 80 + 1280
