@@ -38,9 +38,13 @@ def parse():
     ap.add_argument("--backsize", type=int, default=32)
     ap.add_argument("--part_size", type=int, default=0, help="forward group size (0 = int(avg degree))")
     ap.add_argument("--team", type=int, default=0, help="force lanes per group (0 = automatic)")
+    ap.add_argument("--no_workspace", action="store_true",
+                    help="aggregate without the feature workspace (per-edge scale gather, no scratch)")
     ap.add_argument("--no_cpu_baseline", action="store_true")
     ap.add_argument("--no_train", action="store_true", help="skip the 100-epoch training timing")
     ap.add_argument("--train_epochs", type=int, default=100)
+    ap.add_argument("--copy_probe", action="store_true",
+                    help="also launch a plain 1 GiB device copy 3 times (calibrates byte counters under rocprofv3)")
     ap.add_argument("--verbose", action="store_true")
     return ap.parse_args()
 
@@ -84,25 +88,26 @@ def main():
     dy22 = graphs.normal32(1, (n, 22), dev, 2) * wl.train_mask[:, None]
     dy16 = graphs.normal32(1, (n, 16), dev, 3) * wl.ngh_masks[0][:, None]
     out16, out22 = torch.empty_like(x16), torch.empty_like(x22)
+    ws16, ws22 = (torch.empty_like(x16), torch.empty_like(x22)) if not args.no_workspace else (None, None)
     p_last, p_first = wl.paths[1], wl.paths[0]
     if args.team:
         capi.set_team_size(args.team)
 
     def fwd16():
         capi.spmm_forward(x16, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 32, 8,
-                          g.row_pointers, out16)
+                          g.row_pointers, out16, workspace=ws16)
 
     def fwd22():
         capi.spmm_forward(x22, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 16, 8,
-                          g.row_pointers, out22)
+                          g.row_pointers, out22, workspace=ws22)
 
     def bwd22():
         capi.ours_backward(dy22, p_last.ids, p_last.part_pointer, p_last.edge_list, g.degrees, p_last.num_parts,
-                           p_last.part_size, 2, 4, 16, out22)
+                           p_last.part_size, 2, 4, 16, out22, workspace=ws22)
 
     def bwd16():
         capi.ours_backward(dy16, p_first.ids, p_first.part_pointer, p_first.edge_list, g.degrees,
-                           p_first.num_parts, p_first.part_size, 1, 4, 16, out16)
+                           p_first.num_parts, p_first.part_size, 1, 4, 16, out16, workspace=ws16)
 
     kernels = [
         ("fwd_agg_d16", fwd16, workload.bytes_forward(n, e, 16)),
@@ -142,6 +147,13 @@ def main():
                             "pct_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS * 100, 2)}
     capi.set_timing(False)
     capi.clear_time()
+    if args.copy_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     dominant = max(per_kernel, key=lambda k: per_kernel[k]["ms"])
     dk = per_kernel[dominant]
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": dk["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -157,7 +169,8 @@ def main():
                    "forward_groups": wl.num_parts, "backsize_mode": args.backsize_mode,
                    "backward_group_size": [p.part_size for p in wl.paths],
                    "kept_edges": [p.valid_len for p in wl.paths],
-                   "backward_groups": [p.num_parts for p in wl.paths], "max_degree": g.stats()["max_degree"]},
+                   "backward_groups": [p.num_parts for p in wl.paths], "max_degree": g.stats()["max_degree"],
+                   "feature_workspace": not args.no_workspace},
         "agg_ms_per_epoch": round(ms_per_step, 4), "alg_bytes_per_epoch": bytes_epoch,
         "pct_of_peak_hbm": round(value / PEAK_HBM_GBS * 100, 2),
         "per_kernel": per_kernel, "path_preparation_s": round(prep_s, 3),

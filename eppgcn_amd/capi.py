@@ -12,7 +12,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libeppgcn_hip.so")
+LIB_PATH = os.environ.get("EPPGCN_HIP_LIB") or os.path.join(_HERE, "lib", "libeppgcn_hip.so")
 
 EXPORTS = [
     "eppgcn_last_error", "eppgcn_abi_version", "eppgcn_spmm_forward", "eppgcn_spmm_backward",
@@ -42,9 +42,9 @@ def load():
     p, i, i64, sz = C.c_void_p, C.c_int, C.c_int64, C.c_size_t
     lib.eppgcn_last_error.restype = C.c_char_p
     lib.eppgcn_abi_version.restype = i
-    lib.eppgcn_spmm_forward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p]
-    lib.eppgcn_spmm_backward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p]
-    lib.eppgcn_ours_backward.argtypes = [p, p, p, p, p, p, i, i, i, i, i, i, i, p]
+    lib.eppgcn_spmm_forward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, p]
+    lib.eppgcn_spmm_backward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, p]
+    lib.eppgcn_ours_backward.argtypes = [p, p, p, p, p, p, i, i, i, i, i, i, i, p, p]
     lib.eppgcn_mask_forward.argtypes = [p, p, p, p, p, p, p, i, i64, i, i, i, p]
     lib.eppgcn_compact_workspace_bytes.argtypes = [i64]
     lib.eppgcn_compact_workspace_bytes.restype = sz
@@ -108,8 +108,21 @@ def _mask_bytes(t, name):
 
 
 # --------------------------------------------------------------------------- aggregation
+def _feature_workspace(workspace, feats):
+    """None -> per-edge scale gather (no scratch); True -> allocate; a tensor -> use it (it may be
+    `feats` itself, which is then overwritten with the scaled features)."""
+    if workspace is None or workspace is False:
+        return None
+    if workspace is True:
+        return torch.empty_like(feats)
+    _dev(workspace, torch.float32, "workspace")
+    if workspace.numel() < feats.numel():
+        raise EppgcnError("workspace needs num_nodes * dim floats")
+    return workspace
+
+
 def spmm_forward(feats, column_index, degrees, part_ptr, part2node, part_size=32, dim_worker=32,
-                 warp_per_block=8, row_pointers=None, out=None, backward=False):
+                 warp_per_block=8, row_pointers=None, out=None, backward=False, workspace=True):
     """out[N, D] = neighbour-group aggregation of feats (``backward=True`` uses the unpruned
     backward entry point; same operator)."""
     lib = load()
@@ -125,13 +138,14 @@ def spmm_forward(feats, column_index, degrees, part_ptr, part2node, part_size=32
     if out is None:
         out = torch.empty_like(feats)
     fn = lib.eppgcn_spmm_backward if backward else lib.eppgcn_spmm_forward
+    ws = _feature_workspace(workspace, feats)
     _check(fn(_ptr(out), _ptr(feats), _ptr(row_pointers), _ptr(column_index), _ptr(degrees), _ptr(part_ptr),
-              _ptr(part2node), n, dim, num_parts, part_size, dim_worker, warp_per_block, _stream()))
+              _ptr(part2node), n, dim, num_parts, part_size, dim_worker, warp_per_block, _ptr(ws), _stream()))
     return out
 
 
 def ours_backward(d_output, ids, part_pointer, edge_list, degrees, num_parts, part_size=32, layer=1,
-                  blockx=4, blocky=16, out=None):
+                  blockx=4, blocky=16, out=None, workspace=True):
     lib = load()
     _dev(d_output, torch.float32, "d_output"); _dev(ids, torch.int32, "ids")
     _dev(part_pointer, torch.int32, "part_pointer"); _dev(edge_list, torch.int32, "edge_list")
@@ -141,9 +155,10 @@ def ours_backward(d_output, ids, part_pointer, edge_list, degrees, num_parts, pa
         raise EppgcnError("part_pointer needs num_parts + 1 entries")
     if out is None:
         out = torch.empty_like(d_output)
+    ws = _feature_workspace(workspace, d_output)
     _check(lib.eppgcn_ours_backward(_ptr(out), _ptr(d_output), _ptr(ids), _ptr(part_pointer), _ptr(edge_list),
                                     _ptr(degrees), n, dim, int(num_parts), part_size, layer, blockx, blocky,
-                                    _stream()))
+                                    _ptr(ws), _stream()))
     return out
 
 

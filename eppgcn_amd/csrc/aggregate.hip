@@ -6,27 +6,38 @@
 // (:626-670).  Same contract, different machine mapping:
 //
 //   out[r, :] = sum over the slots e of every group of row r of
-//               fl32(s[r] * s[col[e]]) * in[col[e], :]
+//               s[r] * s[col[e]] * in[col[e], :]
 //
 // Mapping.  A wave of 64 lanes is cut into teams of TS lanes; a team owns one
 // neighbour group and its lanes stripe the feature row in contiguous vectors of
 // VW floats (lane l of the team holds columns [l*VW, l*VW+VW), then +TS*VW ...),
 // so one gather instruction fetches 64/TS whole neighbour rows with contiguous
 // bytes per row.  The groups of a wave are consecutive, hence their CSR slots are
-// one contiguous range: the wave first stages that range coalesced into LDS as
-// (column id, neighbour scale) pairs, which turns the per-neighbour dependent
-// chain "id -> scale -> row" into three batched phases with many requests in
-// flight.  Partial sums live in registers.  Flush: a row whose groups all sit in
-// this wave is reduced across teams with DPP / ds_swizzle and written with plain
-// stores; a row with a single group is stored directly; only rows spread over
-// several waves use float atomics.
+// one contiguous range: the wave first stages that range coalesced into LDS,
+// which turns the per-neighbour dependent chain "id -> row" into batched phases
+// with many requests in flight.  Partial sums live in registers.
+//
+// Neighbour scale.  Gathering s[col[e]] per edge costs one extra random memory
+// request per edge (measured: a quarter of the kernel time at width 16).  With a
+// workspace the features are scaled once per call (ws[c,:] = s[c]*in[c,:], one
+// streaming pass) and the kernel gathers pre-scaled rows and multiplies by s[r]
+// at the flush.  Without a workspace the kernel stages (id, scale) pairs and
+// weights every row by fl32(s[r]*s[c]) as the reference does.
+//
+// Flush.  Groups of one row that sit in the same wave are first summed across
+// teams in registers (DPP rotations / ds_swizzle when the whole wave is one row,
+// a segmented shuffle reduction otherwise).  A row that lies entirely inside the
+// wave is then written with plain stores; only rows spread over several waves
+// use float atomics, once per wave instead of once per group.
+// Precondition: the groups of one row are consecutive (build_part and the path
+// splitter produce them that way).
 #include "common.hpp"
 
 namespace eppgcn {
 
 constexpr int kAggBlock = 256;
 constexpr int kAggWaves = kAggBlock / kWave;
-constexpr int kStageCap = 512;   // staged (column, scale) pairs per wave and pass
+constexpr int kStageCap = 512;   // staged slots per wave and pass
 
 // ---------------------------------------------------------------- vectors
 template <int VW> struct Vec;
@@ -80,15 +91,33 @@ struct CompactedGroups {
     }
 };
 
+// ---------------------------------------------------------------- pre-scaling pass
+// dst[r, :] = scale[r] * src[r, :]; one thread per float4 (or float) element.
+template <int VW>
+__global__ __launch_bounds__(256) void scale_rows_kernel(float* __restrict__ dst, const float* __restrict__ src,
+                                                         const float* __restrict__ scale, long long total_vecs,
+                                                         int vecs_per_row)
+{
+    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+    for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs; i += stride) {
+        const float s = scale[i / vecs_per_row];
+        Vec<VW> v = Vec<VW>::load(src + i * VW);
+#pragma unroll
+        for (int j = 0; j < VW; ++j) v.v[j] *= s;
+        v.store(dst + i * VW);
+    }
+}
+
 // ---------------------------------------------------------------- kernel
-template <int VW, int TS, int CPL, int U, class Groups>
+template <int VW, int TS, int CPL, int U, bool kPrescaled, class Groups>
 __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
     float* __restrict__ out, const float* __restrict__ in, const int* __restrict__ col,
     const float* __restrict__ scale, Groups groups, int num_parts, int width, int ld)
 {
     constexpr int TPW = kWave / TS;      // teams (= groups) per wave
     using V = Vec<VW>;
-    __shared__ int2 stage[kAggWaves][kStageCap];
+    __shared__ int stage_col[kAggWaves][kStageCap];
+    __shared__ float stage_scale[kAggWaves][kPrescaled ? 1 : kStageCap];
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
@@ -121,34 +150,42 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
 #pragma unroll
         for (int j = 0; j < VW; ++j) acc[k].v[j] = 0.f;
 
-    int2* my_stage = stage[wave];
+    int* my_col = stage_col[wave];
+    float* my_scale = stage_scale[wave];
     for (int cb = wbeg; cb < wend; cb += kStageCap) {
         const int cn = min(kStageCap, wend - cb);
-        // phase 1+2: coalesced column ids, then one scale gather per staged slot
+        // stage the pass: coalesced column ids (and, without pre-scaling, one scale gather per slot)
         {
             int c[kStageCap / kWave];
-            float sc[kStageCap / kWave];
 #pragma unroll
             for (int r = 0; r < kStageCap / kWave; ++r) {
                 const int i = lane + r * kWave;
                 c[r] = i < cn ? col[cb + i] : 0;
             }
+            if constexpr (!kPrescaled) {
+                float sc[kStageCap / kWave];
 #pragma unroll
-            for (int r = 0; r < kStageCap / kWave; ++r) {
-                const int i = lane + r * kWave;
-                sc[r] = i < cn ? scale[c[r]] : 0.f;
+                for (int r = 0; r < kStageCap / kWave; ++r) {
+                    const int i = lane + r * kWave;
+                    sc[r] = i < cn ? scale[c[r]] : 0.f;
+                }
+#pragma unroll
+                for (int r = 0; r < kStageCap / kWave; ++r) {
+                    const int i = lane + r * kWave;
+                    if (i < cn) my_scale[i] = sc[r];
+                }
             }
 #pragma unroll
             for (int r = 0; r < kStageCap / kWave; ++r) {
                 const int i = lane + r * kWave;
-                if (i < cn) my_stage[i] = make_int2(c[r], __float_as_int(sc[r]));
+                if (i < cn) my_col[i] = c[r];
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        // phase 3: every team walks the part of its group that lies in this pass
+        // every team walks the part of its group that lies in this pass, U rows in flight
         const int lo = max(gbeg, cb);
         const int hi = live ? min(gend, cb + cn) : lo;
         for (int i = lo; i < hi; i += U) {
@@ -157,9 +194,10 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const bool ok = i + u < hi;
-                const int2 st = my_stage[ok ? i + u - cb : 0];
-                w[u] = ok ? s_row * __int_as_float(st.y) : 0.f;
-                const float* src = in + static_cast<size_t>(st.x) * ld;
+                const int slot = ok ? i + u - cb : 0;
+                const int c = my_col[slot];
+                if constexpr (!kPrescaled) w[u] = ok ? s_row * my_scale[slot] : 0.f;
+                const float* src = in + static_cast<size_t>(c) * ld;
 #pragma unroll
                 for (int k = 0; k < CPL; ++k) {
                     const int ch = tl + k * TS;
@@ -176,50 +214,69 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
 #pragma unroll
                 for (int k = 0; k < CPL; ++k)
 #pragma unroll
-                    for (int j = 0; j < VW; ++j) acc[k].v[j] = fmaf(w[u], v[u][k].v[j], acc[k].v[j]);
+                    for (int j = 0; j < VW; ++j) {
+                        if constexpr (kPrescaled) acc[k].v[j] += v[u][k].v[j];
+                        else acc[k].v[j] = fmaf(w[u], v[u][k].v[j], acc[k].v[j]);
+                    }
         }
         __builtin_amdgcn_wave_barrier();   // all teams are done with the stage before it is refilled
+    }
+    if constexpr (kPrescaled) {
+#pragma unroll
+        for (int k = 0; k < CPL; ++k)
+#pragma unroll
+            for (int j = 0; j < VW; ++j) acc[k].v[j] *= s_row;
     }
 
     // ---- flush
     const bool prev = live && groups.has_prev(p, row, gbeg);
     const bool next = live && groups.has_next(p, row, gend, num_parts);
+    bool head = live;          // this team writes its (possibly combined) sum
+    bool outside = prev || next;   // the row also has groups in other waves
     if constexpr (TPW > 1) {
         const int row0 = __shfl(row, 0, kWave);
-        const bool one_row = np > 1 && __all(!active || (live && row == row0));
-        if (one_row) {
-            // every group of this wave belongs to one row: reduce across teams in registers
+        if (np > 1 && __all(!active || (live && row == row0))) {
+            // the whole wave is one row: butterfly over the teams with DPP / swizzle
 #pragma unroll
             for (int k = 0; k < CPL; ++k)
 #pragma unroll
                 for (int j = 0; j < VW; ++j) acc[k].v[j] = cross_team_sum<TS>(acc[k].v[j]);
-            const bool outside = __shfl(static_cast<int>(prev), 0, kWave) ||
-                                 __shfl(static_cast<int>(next), (np - 1) * TS, kWave);
-            if (team == 0) {
-                float* dst = out + static_cast<size_t>(row0) * ld;
+            head = team == 0;
+            outside = __shfl(static_cast<int>(prev), 0, kWave) != 0 ||
+                      __shfl(static_cast<int>(next), (np - 1) * TS, kWave) != 0;
+        } else if (__any(prev || next)) {
+            // several rows: segmented reduction towards the first team of every run of equal
+            // rows; the run's "continues in the next wave" flag travels with the sums
+            const int key = live ? row : -1 - team;          // dead teams never merge
+            const int key_up = __shfl_up(key, TS, kWave);
+            int more = next ? 1 : 0;
 #pragma unroll
-                for (int k = 0; k < CPL; ++k) {
-                    const int ch = tl + k * TS;
-                    if (ch < chunks) {
-                        if (outside) {
+            for (int d = 1; d < TPW; d <<= 1) {
+                const int other = __shfl_down(key, d * TS, kWave);
+                const int other_more = __shfl_down(more, d * TS, kWave);
+                const bool take = team + d < TPW && other == key;
+                if (take) more |= other_more;
 #pragma unroll
-                            for (int j = 0; j < VW; ++j) unsafeAtomicAdd(dst + ch * VW + j, acc[k].v[j]);
-                        } else {
-                            acc[k].store(dst + ch * VW);
-                        }
+                for (int k = 0; k < CPL; ++k)
+#pragma unroll
+                    for (int j = 0; j < VW; ++j) {
+                        const float o = __shfl_down(acc[k].v[j], d * TS, kWave);
+                        if (take) acc[k].v[j] += o;
                     }
-                }
             }
-            return;
+            head = live && (team == 0 || key_up != key);
+            // a head's predecessor group is outside its run, so `prev` says whether the row
+            // started in an earlier wave; `more` whether it goes on after the run's last team
+            outside = prev || more != 0;
         }
     }
-    if (live) {
+    if (head) {
         float* dst = out + static_cast<size_t>(row) * ld;
 #pragma unroll
         for (int k = 0; k < CPL; ++k) {
             const int ch = tl + k * TS;
             if (ch < chunks) {
-                if (prev || next) {
+                if (outside) {
 #pragma unroll
                     for (int j = 0; j < VW; ++j) unsafeAtomicAdd(dst + ch * VW + j, acc[k].v[j]);
                 } else {
@@ -237,33 +294,31 @@ struct AggTuning {
 static AggTuning g_tuning;
 void set_agg_force_team(int ts) { g_tuning.force_team = ts; }
 
-template <int VW, int TS, int CPL, int U, class Groups>
+template <int VW, int TS, int CPL, int U, bool kPrescaled, class Groups>
 static hipError_t launch_one(float* out, const float* in, const int* col, const float* scale, Groups g,
                              int num_parts, int width, int ld, hipStream_t stream)
 {
     constexpr int TPW = kWave / TS;
     const long long groups_per_block = static_cast<long long>(TPW) * kAggWaves;
     const long long grid = (num_parts + groups_per_block - 1) / groups_per_block;
-    hipLaunchKernelGGL((aggregate_kernel<VW, TS, CPL, U, Groups>), dim3(static_cast<unsigned>(grid)),
+    hipLaunchKernelGGL((aggregate_kernel<VW, TS, CPL, U, kPrescaled, Groups>), dim3(static_cast<unsigned>(grid)),
                        dim3(kAggBlock), 0, stream, out, in, col, scale, g, num_parts, width, ld);
     return hipGetLastError();
 }
 
 // One column slab of at most 64*4 vectors of VW floats.
-template <int VW, class Groups>
+template <int VW, bool kPrescaled, class Groups>
 static hipError_t launch_slab(float* out, const float* in, const int* col, const float* scale, Groups g,
                               int num_parts, int width, int ld, hipStream_t stream)
 {
     const int chunks = width / VW;
     int ts = 4;
     while (ts < 64 && ts < chunks) ts <<= 1;
-    if (g_tuning.force_team >= 4 && g_tuning.force_team <= 64 &&
-        (g_tuning.force_team & (g_tuning.force_team - 1)) == 0 && chunks <= 4 * g_tuning.force_team &&
-        (g_tuning.force_team == 64 || chunks <= 2 * g_tuning.force_team))
-        ts = g_tuning.force_team;
+    const int ft = g_tuning.force_team;
+    if (ft >= 4 && ft <= 64 && (ft & (ft - 1)) == 0 && chunks <= 4 * ft && (ft == 64 || chunks <= 2 * ft)) ts = ft;
     const int cpl = (chunks + ts - 1) / ts;
 #define EPPGCN_LAUNCH(TS_, CPL_, U_) \
-    return launch_one<VW, TS_, CPL_, U_, Groups>(out, in, col, scale, g, num_parts, width, ld, stream)
+    return launch_one<VW, TS_, CPL_, U_, kPrescaled, Groups>(out, in, col, scale, g, num_parts, width, ld, stream)
     if (cpl <= 1) {
         switch (ts) {
             case 4: EPPGCN_LAUNCH(4, 1, 8);
@@ -286,13 +341,40 @@ static hipError_t launch_slab(float* out, const float* in, const int* col, const
 #undef EPPGCN_LAUNCH
 }
 
+int launch_scale_rows(float* dst, const float* src, const float* scale, int num_nodes, int dim, hipStream_t stream)
+{
+    const long long total = static_cast<long long>(num_nodes) * dim;
+    if (total == 0) return kOk;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src);
+    int vw = 1;
+    if (dim % 4 == 0 && bits % 16 == 0) vw = 4;
+    else if (dim % 2 == 0 && bits % 8 == 0) vw = 2;
+    const long long vecs = total / vw;
+    long long blocks = (vecs + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    const dim3 grid(static_cast<unsigned>(blocks)), block(256);
+    if (vw == 4) hipLaunchKernelGGL(scale_rows_kernel<4>, grid, block, 0, stream, dst, src, scale, vecs, dim / 4);
+    else if (vw == 2) hipLaunchKernelGGL(scale_rows_kernel<2>, grid, block, 0, stream, dst, src, scale, vecs, dim / 2);
+    else hipLaunchKernelGGL(scale_rows_kernel<1>, grid, block, 0, stream, dst, src, scale, vecs, dim);
+    EPPGCN_HIP(hipGetLastError());
+    return kOk;
+}
+
+// workspace: nullptr, or num_nodes*dim floats (may alias `in` when the caller gives up the
+// unscaled features).
 template <class Groups>
 static int aggregate_dispatch(float* out, const float* in, const int* col, const float* scale, Groups g,
-                              int num_nodes, int dim, int num_parts, hipStream_t stream, double* sink, double* sink2)
+                              int num_nodes, int dim, int num_parts, float* workspace, hipStream_t stream,
+                              double* sink, double* sink2)
 {
     EPPGCN_HIP(hipMemsetAsync(out, 0, static_cast<size_t>(num_nodes) * dim * sizeof(float), stream));
     if (num_parts == 0) return kOk;
-    KernelTimer timer(stream, sink, sink2);   // brackets the aggregation kernel(s) only, not the clear
+    const bool prescaled = workspace != nullptr;
+    if (prescaled) {
+        if (int rc = launch_scale_rows(workspace, in, scale, num_nodes, dim, stream)) return rc;
+        in = workspace;
+    }
+    KernelTimer timer(stream, sink, sink2);   // brackets the aggregation kernel alone
     const uintptr_t bits = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(in);
     int vw = 1;
     if (dim % 4 == 0 && bits % 16 == 0) vw = 4;
@@ -301,9 +383,13 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
     for (int c0 = 0; c0 < dim; c0 += slab) {
         const int width = dim - c0 < slab ? dim - c0 : slab;
         hipError_t e;
-        if (vw == 4) e = launch_slab<4>(out + c0, in + c0, col, scale, g, num_parts, width, dim, stream);
-        else if (vw == 2) e = launch_slab<2>(out + c0, in + c0, col, scale, g, num_parts, width, dim, stream);
-        else e = launch_slab<1>(out + c0, in + c0, col, scale, g, num_parts, width, dim, stream);
+#define EPPGCN_SLAB(VW_)                                                                                              \
+    (prescaled ? launch_slab<VW_, true>(out + c0, in + c0, col, scale, g, num_parts, width, dim, stream)              \
+               : launch_slab<VW_, false>(out + c0, in + c0, col, scale, g, num_parts, width, dim, stream))
+        if (vw == 4) e = EPPGCN_SLAB(4);
+        else if (vw == 2) e = EPPGCN_SLAB(2);
+        else e = EPPGCN_SLAB(1);
+#undef EPPGCN_SLAB
         if (e != hipSuccess) return hip_fail(e, "aggregate kernel launch");
     }
     return kOk;
@@ -311,18 +397,18 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
 
 int aggregate_forward_groups(float* out, const float* in, const int* col, const float* scale,
                              const int* part_ptr, const int* part2node, int num_nodes, int dim,
-                             int num_parts, hipStream_t stream, double* sink, double* sink2)
+                             int num_parts, float* workspace, hipStream_t stream, double* sink, double* sink2)
 {
     return aggregate_dispatch(out, in, col, scale, ForwardGroups{part_ptr, part2node}, num_nodes, dim,
-                              num_parts, stream, sink, sink2);
+                              num_parts, workspace, stream, sink, sink2);
 }
 
 int aggregate_compacted_groups(float* out, const float* in, const int* ids, const int* part_ptr,
                                const int* edge_list, const float* scale, int num_nodes, int dim,
-                               int num_parts, hipStream_t stream, double* sink, double* sink2)
+                               int num_parts, float* workspace, hipStream_t stream, double* sink, double* sink2)
 {
     return aggregate_dispatch(out, in, edge_list, scale, CompactedGroups{part_ptr, ids}, num_nodes, dim,
-                              num_parts, stream, sink, sink2);
+                              num_parts, workspace, stream, sink, sink2);
 }
 
 }  // namespace eppgcn

@@ -12,9 +12,9 @@ namespace eppgcn {
 
 // ---- implemented in aggregate.hip / prepare.hip
 int aggregate_forward_groups(float*, const float*, const int*, const float*, const int*, const int*, int, int, int,
-                             hipStream_t, double*, double*);
+                             float*, hipStream_t, double*, double*);
 int aggregate_compacted_groups(float*, const float*, const int*, const int*, const int*, const float*, int, int, int,
-                               hipStream_t, double*, double*);
+                               float*, hipStream_t, double*, double*);
 void set_agg_force_team(int);
 size_t compact_workspace_bytes(long long);
 size_t split_workspace_bytes(long long);
@@ -62,11 +62,12 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 1; }
+int eppgcn_abi_version(void) { return 2; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
-                        int dim, int num_parts, int part_size, int dim_worker, int warp_per_block, void* stream)
+                        int dim, int num_parts, int part_size, int dim_worker, int warp_per_block, float* workspace,
+                        void* stream)
 {
     (void)row_pointers;
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
@@ -75,14 +76,15 @@ int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers
     EPPGCN_REQUIRE(out && in && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (column_index && part_pointers && part2node), "null index pointer");
     EPPGCN_REQUIRE(aligned(out, 4) && aligned(in, 4), "feature pointers must be 4-byte aligned");
+    EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != out), "workspace must be 16-byte aligned and distinct from the output");
     return aggregate_forward_groups(out, in, column_index, degrees, part_pointers, part2node, num_nodes, dim, num_parts,
-                                    static_cast<hipStream_t>(stream), &g_for_agg_ms, nullptr);
+                                    workspace, static_cast<hipStream_t>(stream), &g_for_agg_ms, nullptr);
 }
 
 int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* row_pointers,
                          const int32_t* column_index, const float* degrees, const int32_t* part_pointers,
                          const int32_t* part2node, int num_nodes, int dim, int num_parts, int part_size, int dim_worker,
-                         int warp_per_block, void* stream)
+                         int warp_per_block, float* workspace, void* stream)
 {
     (void)row_pointers;
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
@@ -91,13 +93,14 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
     EPPGCN_REQUIRE(d_input && d_output && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (column_index && part_pointers && part2node), "null index pointer");
     EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
+    EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != d_input), "workspace must be 16-byte aligned and distinct from the output");
     return aggregate_forward_groups(d_input, d_output, column_index, degrees, part_pointers, part2node, num_nodes, dim,
-                                    num_parts, static_cast<hipStream_t>(stream), &g_back_agg_ms, nullptr);
+                                    num_parts, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms, nullptr);
 }
 
 int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
                          const int32_t* edge_list, const float* degrees, int num_nodes, int dim, int num_parts,
-                         int part_size, int layer, int blockx, int blocky, void* stream)
+                         int part_size, int layer, int blockx, int blocky, float* workspace, void* stream)
 {
     (void)part_size;   // the reference's kernel ignores it too (EPPGCN_kernel.cu:636)
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
@@ -107,8 +110,9 @@ int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* i
     EPPGCN_REQUIRE(d_input && d_output && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (ids && part_pointer && edge_list), "null index pointer");
     EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
+    EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != d_input), "workspace must be 16-byte aligned and distinct from the output");
     return aggregate_compacted_groups(d_input, d_output, ids, part_pointer, edge_list, degrees, num_nodes, dim,
-                                      num_parts, static_cast<hipStream_t>(stream), &g_back_agg_ms,
+                                      num_parts, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms,
                                       layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr);
 }
 

@@ -150,10 +150,18 @@ def test_heuristics_and_ginfo(api):
 def _forward_case(api, indptr, col, s, x, ps, what):
     n = indptr.size - 1
     pp, p2n = co.build_part(ps, indptr)
-    got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp), dev(p2n), part_size=ps).cpu().numpy()
     want = co.spmm_f64(x, indptr, col, s)
     bound = cf.abs_sum_bound(indptr, col, s, x)
-    assert_close(got, want, bound, what)
+    dx = dev(x)
+    # three scale modes: per-edge gather (no scratch), scratch workspace, workspace aliasing the input
+    plain = api.spmm_forward(dx, dev(col), dev(s), dev(pp), dev(p2n), part_size=ps, workspace=None).cpu().numpy()
+    assert_close(plain, want, bound, what + " [no workspace]")
+    got = api.spmm_forward(dx, dev(col), dev(s), dev(pp), dev(p2n), part_size=ps, workspace=True).cpu().numpy()
+    assert_close(got, want, bound, what + " [workspace]")
+    assert np.array_equal(dx.cpu().numpy(), x), "a separate workspace must leave the input untouched"
+    alias = api.spmm_forward(dx, dev(col), dev(s), dev(pp), dev(p2n), part_size=ps, workspace=dx).cpu().numpy()
+    assert_close(alias, want, bound, what + " [aliased workspace]")
+    assert np.array_equal(dx.cpu().numpy(), (s[:, None] * x).astype(np.float32)), "aliased input holds s*x"
     return got
 
 
@@ -263,6 +271,8 @@ def test_pruned_backward_vs_checker_and_unpruned(api, name, dim, ratio):
         oid, oedge, bpp, p = _gpu_path(api, indptr, col, src, 5, ps_back)
         got = api.ours_backward(dev(dy), oid, bpp, oedge, dev(s), p, part_size=ps_back).cpu().numpy()
         assert_close(got, want, bound, f"{name} D={dim} r={ratio} ps={ps_back}")
+        plain = api.ours_backward(dev(dy), oid, bpp, oedge, dev(s), p, part_size=ps_back, workspace=None)
+        assert_close(plain.cpu().numpy(), want, bound, f"{name} D={dim} r={ratio} ps={ps_back} [no workspace]")
         ref32 = co.ours_backward(dy, oid.cpu().numpy(), bpp.cpu().numpy(), oedge.cpu().numpy(), s, p)
         assert_close(got, ref32.astype(np.float64), 2 * bound, "vs fp32 restatement")
         # pruning really ignores gradient rows outside the mask
