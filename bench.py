@@ -88,7 +88,8 @@ def main():
     dy22 = graphs.normal32(1, (n, 22), dev, 2) * wl.train_mask[:, None]
     dy16 = graphs.normal32(1, (n, 16), dev, 3) * wl.ngh_masks[0][:, None]
     out16, out22 = torch.empty_like(x16), torch.empty_like(x22)
-    ws16, ws22 = (torch.empty_like(x16), torch.empty_like(x22)) if not args.no_workspace else (None, None)
+    ws16, ws22 = ((capi.feature_workspace(n, 16, dev), capi.feature_workspace(n, 22, dev))
+                  if not args.no_workspace else (None, None))
     p_last, p_first = wl.paths[1], wl.paths[0]
     if args.team:
         capi.set_team_size(args.team)

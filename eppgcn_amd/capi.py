@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("EPPGCN_HIP_LIB") or os.path.join(_HERE, "lib", "libeppgcn_hip.so")
 
 EXPORTS = [
-    "eppgcn_last_error", "eppgcn_abi_version", "eppgcn_spmm_forward", "eppgcn_spmm_backward",
+    "eppgcn_last_error", "eppgcn_abi_version", "eppgcn_feature_workspace_floats", "eppgcn_spmm_forward", "eppgcn_spmm_backward",
     "eppgcn_ours_backward", "eppgcn_mask_forward", "eppgcn_compact_workspace_bytes",
     "eppgcn_split_workspace_bytes", "eppgcn_compact_back_edge", "eppgcn_count_nonzero",
     "eppgcn_map_back_part_size", "eppgcn_threshold_back_part_size", "eppgcn_split_back_part",
@@ -42,9 +42,11 @@ def load():
     p, i, i64, sz = C.c_void_p, C.c_int, C.c_int64, C.c_size_t
     lib.eppgcn_last_error.restype = C.c_char_p
     lib.eppgcn_abi_version.restype = i
-    lib.eppgcn_spmm_forward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, p]
-    lib.eppgcn_spmm_backward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, p]
-    lib.eppgcn_ours_backward.argtypes = [p, p, p, p, p, p, i, i, i, i, i, i, i, p, p]
+    lib.eppgcn_feature_workspace_floats.argtypes = [i64, i]
+    lib.eppgcn_feature_workspace_floats.restype = sz
+    lib.eppgcn_spmm_forward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, sz, p]
+    lib.eppgcn_spmm_backward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, sz, p]
+    lib.eppgcn_ours_backward.argtypes = [p, p, p, p, p, p, i, i, i, i, i, i, i, p, sz, p]
     lib.eppgcn_mask_forward.argtypes = [p, p, p, p, p, p, p, i, i64, i, i, i, p]
     lib.eppgcn_compact_workspace_bytes.argtypes = [i64]
     lib.eppgcn_compact_workspace_bytes.restype = sz
@@ -114,11 +116,15 @@ def _feature_workspace(workspace, feats):
     if workspace is None or workspace is False:
         return None
     if workspace is True:
-        return torch.empty_like(feats)
+        return feature_workspace(feats.shape[0], feats.shape[1], feats.device)
     _dev(workspace, torch.float32, "workspace")
-    if workspace.numel() < feats.numel():
-        raise EppgcnError("workspace needs num_nodes * dim floats")
     return workspace
+
+
+def feature_workspace(num_nodes: int, dim: int, device):
+    """A scratch tensor large enough for the pre-scaled, padded copy of [num_nodes, dim] features."""
+    return torch.empty(load().eppgcn_feature_workspace_floats(int(num_nodes), int(dim)), dtype=torch.float32,
+                       device=device)
 
 
 def spmm_forward(feats, column_index, degrees, part_ptr, part2node, part_size=32, dim_worker=32,
@@ -140,7 +146,8 @@ def spmm_forward(feats, column_index, degrees, part_ptr, part2node, part_size=32
     fn = lib.eppgcn_spmm_backward if backward else lib.eppgcn_spmm_forward
     ws = _feature_workspace(workspace, feats)
     _check(fn(_ptr(out), _ptr(feats), _ptr(row_pointers), _ptr(column_index), _ptr(degrees), _ptr(part_ptr),
-              _ptr(part2node), n, dim, num_parts, part_size, dim_worker, warp_per_block, _ptr(ws), _stream()))
+              _ptr(part2node), n, dim, num_parts, part_size, dim_worker, warp_per_block, _ptr(ws),
+              0 if ws is None else ws.numel(), _stream()))
     return out
 
 
@@ -158,7 +165,7 @@ def ours_backward(d_output, ids, part_pointer, edge_list, degrees, num_parts, pa
     ws = _feature_workspace(workspace, d_output)
     _check(lib.eppgcn_ours_backward(_ptr(out), _ptr(d_output), _ptr(ids), _ptr(part_pointer), _ptr(edge_list),
                                     _ptr(degrees), n, dim, int(num_parts), part_size, layer, blockx, blocky,
-                                    _ptr(ws), _stream()))
+                                    _ptr(ws), 0 if ws is None else ws.numel(), _stream()))
     return out
 
 

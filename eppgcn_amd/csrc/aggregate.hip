@@ -92,27 +92,45 @@ struct CompactedGroups {
 };
 
 // ---------------------------------------------------------------- pre-scaling pass
-// dst[r, :] = scale[r] * src[r, :]; one thread per float4 (or float) element.
-template <int VW>
+// dst[r, j] = scale[r] * src[r, j] for j < dim and 0 for dim <= j < ld_dst.  The destination
+// row pitch ld_dst is a multiple of 4 floats, so every thread writes one aligned float4; rows
+// padded to whole 32-byte sectors let the gather fetch fewer sectors per row and use 16-byte
+// loads for widths such as 22 whose rows are only 8-byte aligned in the caller's layout.
 __global__ __launch_bounds__(256) void scale_rows_kernel(float* __restrict__ dst, const float* __restrict__ src,
                                                          const float* __restrict__ scale, long long total_vecs,
-                                                         int vecs_per_row)
+                                                         int vecs_per_row, int dim)
 {
     const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
     for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs; i += stride) {
-        const float s = scale[i / vecs_per_row];
-        Vec<VW> v = Vec<VW>::load(src + i * VW);
-#pragma unroll
-        for (int j = 0; j < VW; ++j) v.v[j] *= s;
-        v.store(dst + i * VW);
+        const long long r = i / vecs_per_row;
+        const int c0 = static_cast<int>(i - r * vecs_per_row) * 4;
+        const float s = scale[r];
+        const float* row = src + r * dim;
+        float4 v;
+        v.x = c0 + 0 < dim ? s * row[c0 + 0] : 0.f;
+        v.y = c0 + 1 < dim ? s * row[c0 + 1] : 0.f;
+        v.z = c0 + 2 < dim ? s * row[c0 + 2] : 0.f;
+        v.w = c0 + 3 < dim ? s * row[c0 + 3] : 0.f;
+        *reinterpret_cast<float4*>(dst + i * 4) = v;
     }
 }
 
+// In-place / unpadded form for a workspace that aliases the input: dst[i] = scale[row(i)] * src[i].
+__global__ __launch_bounds__(256) void scale_rows_flat_kernel(float* __restrict__ dst, const float* __restrict__ src,
+                                                              const float* __restrict__ scale, long long total, int dim)
+{
+    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+    for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride)
+        dst[i] = scale[i / dim] * src[i];
+}
+
 // ---------------------------------------------------------------- kernel
-template <int VW, int TS, int CPL, int U, bool kPrescaled, class Groups>
+// VW: floats per load of the input (row pitch ld_in, `chunks` vectors per row are read);
+// OVW: floats per store of the output (row pitch ld_out, columns < width_out are written).
+template <int VW, int OVW, int TS, int CPL, int U, bool kPrescaled, class Groups>
 __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
     float* __restrict__ out, const float* __restrict__ in, const int* __restrict__ col,
-    const float* __restrict__ scale, Groups groups, int num_parts, int width, int ld)
+    const float* __restrict__ scale, Groups groups, int num_parts, int chunks, int ld_in, int width_out, int ld_out)
 {
     constexpr int TPW = kWave / TS;      // teams (= groups) per wave
     using V = Vec<VW>;
@@ -128,7 +146,6 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
     const int np = min(TPW, static_cast<int>(num_parts - p0));
     const int p = static_cast<int>(p0) + team;
     const bool active = team < np;
-    const int chunks = width / VW;                       // vectors per feature row
 
     int gbeg = 0, gend = 0, row = 0;
     float s_row = 0.f;
@@ -197,7 +214,7 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
                 const int slot = ok ? i + u - cb : 0;
                 const int c = my_col[slot];
                 if constexpr (!kPrescaled) w[u] = ok ? s_row * my_scale[slot] : 0.f;
-                const float* src = in + static_cast<size_t>(c) * ld;
+                const float* src = in + static_cast<size_t>(c) * ld_in;
 #pragma unroll
                 for (int k = 0; k < CPL; ++k) {
                     const int ch = tl + k * TS;
@@ -271,16 +288,23 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
         }
     }
     if (head) {
-        float* dst = out + static_cast<size_t>(row) * ld;
+        float* dst = out + static_cast<size_t>(row) * ld_out;
 #pragma unroll
         for (int k = 0; k < CPL; ++k) {
-            const int ch = tl + k * TS;
-            if (ch < chunks) {
-                if (outside) {
+            const int c0 = (tl + k * TS) * VW;
 #pragma unroll
-                    for (int j = 0; j < VW; ++j) unsafeAtomicAdd(dst + ch * VW + j, acc[k].v[j]);
-                } else {
-                    acc[k].store(dst + ch * VW);
+            for (int piece = 0; piece < VW / OVW; ++piece) {
+                const int c = c0 + piece * OVW;
+                if (c < width_out) {          // width_out is a multiple of OVW: a piece is all in or all out
+                    if (outside) {
+#pragma unroll
+                        for (int j = 0; j < OVW; ++j) unsafeAtomicAdd(dst + c + j, acc[k].v[piece * OVW + j]);
+                    } else {
+                        Vec<OVW> o;
+#pragma unroll
+                        for (int j = 0; j < OVW; ++j) o.v[j] = acc[k].v[piece * OVW + j];
+                        o.store(dst + c);
+                    }
                 }
             }
         }
@@ -294,31 +318,39 @@ struct AggTuning {
 static AggTuning g_tuning;
 void set_agg_force_team(int ts) { g_tuning.force_team = ts; }
 
-template <int VW, int TS, int CPL, int U, bool kPrescaled, class Groups>
+struct AggShape {
+    int chunks;      // input vectors read per row
+    int ld_in;       // input row pitch (floats)
+    int width_out;   // output columns written
+    int ld_out;      // output row pitch (floats)
+};
+
+template <int VW, int OVW, int TS, int CPL, int U, bool kPrescaled, class Groups>
 static hipError_t launch_one(float* out, const float* in, const int* col, const float* scale, Groups g,
-                             int num_parts, int width, int ld, hipStream_t stream)
+                             int num_parts, AggShape sh, hipStream_t stream)
 {
     constexpr int TPW = kWave / TS;
     const long long groups_per_block = static_cast<long long>(TPW) * kAggWaves;
     const long long grid = (num_parts + groups_per_block - 1) / groups_per_block;
-    hipLaunchKernelGGL((aggregate_kernel<VW, TS, CPL, U, kPrescaled, Groups>), dim3(static_cast<unsigned>(grid)),
-                       dim3(kAggBlock), 0, stream, out, in, col, scale, g, num_parts, width, ld);
+    hipLaunchKernelGGL((aggregate_kernel<VW, OVW, TS, CPL, U, kPrescaled, Groups>),
+                       dim3(static_cast<unsigned>(grid)), dim3(kAggBlock), 0, stream, out, in, col, scale, g,
+                       num_parts, sh.chunks, sh.ld_in, sh.width_out, sh.ld_out);
     return hipGetLastError();
 }
 
-// One column slab of at most 64*4 vectors of VW floats.
-template <int VW, bool kPrescaled, class Groups>
+// One column slab of at most 64*4 input vectors of VW floats.
+template <int VW, int OVW, bool kPrescaled, class Groups>
 static hipError_t launch_slab(float* out, const float* in, const int* col, const float* scale, Groups g,
-                              int num_parts, int width, int ld, hipStream_t stream)
+                              int num_parts, AggShape sh, hipStream_t stream)
 {
-    const int chunks = width / VW;
+    const int chunks = sh.chunks;
     int ts = 4;
     while (ts < 64 && ts < chunks) ts <<= 1;
     const int ft = g_tuning.force_team;
     if (ft >= 4 && ft <= 64 && (ft & (ft - 1)) == 0 && chunks <= 4 * ft && (ft == 64 || chunks <= 2 * ft)) ts = ft;
     const int cpl = (chunks + ts - 1) / ts;
 #define EPPGCN_LAUNCH(TS_, CPL_, U_) \
-    return launch_one<VW, TS_, CPL_, U_, kPrescaled, Groups>(out, in, col, scale, g, num_parts, width, ld, stream)
+    return launch_one<VW, OVW, TS_, CPL_, U_, kPrescaled, Groups>(out, in, col, scale, g, num_parts, sh, stream)
     if (cpl <= 1) {
         switch (ts) {
             case 4: EPPGCN_LAUNCH(4, 1, 8);
@@ -341,27 +373,46 @@ static hipError_t launch_slab(float* out, const float* in, const int* col, const
 #undef EPPGCN_LAUNCH
 }
 
-int launch_scale_rows(float* dst, const float* src, const float* scale, int num_nodes, int dim, hipStream_t stream)
+// Row pitch of the pre-scaled workspace: whole 16-byte vectors for narrow rows, whole 32-byte
+// sectors above 8 columns.
+int workspace_pitch(int dim) { return dim <= 8 ? (dim + 3) / 4 * 4 : (dim + 7) / 8 * 8; }
+
+size_t feature_workspace_floats(long long num_nodes, int dim)
 {
-    const long long total = static_cast<long long>(num_nodes) * dim;
-    if (total == 0) return kOk;
-    const uintptr_t bits = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src);
-    int vw = 1;
-    if (dim % 4 == 0 && bits % 16 == 0) vw = 4;
-    else if (dim % 2 == 0 && bits % 8 == 0) vw = 2;
-    const long long vecs = total / vw;
-    long long blocks = (vecs + 255) / 256;
-    if (blocks > 256 * 32) blocks = 256 * 32;
-    const dim3 grid(static_cast<unsigned>(blocks)), block(256);
-    if (vw == 4) hipLaunchKernelGGL(scale_rows_kernel<4>, grid, block, 0, stream, dst, src, scale, vecs, dim / 4);
-    else if (vw == 2) hipLaunchKernelGGL(scale_rows_kernel<2>, grid, block, 0, stream, dst, src, scale, vecs, dim / 2);
-    else hipLaunchKernelGGL(scale_rows_kernel<1>, grid, block, 0, stream, dst, src, scale, vecs, dim);
+    return static_cast<size_t>(num_nodes) * static_cast<size_t>(workspace_pitch(dim));
+}
+
+static int launch_scale_rows(float* dst, const float* src, const float* scale, int num_nodes, int dim, int ld_dst,
+                             hipStream_t stream)
+{
+    if (static_cast<long long>(num_nodes) * dim == 0) return kOk;
+    if (dst == src || ld_dst == dim) {
+        const long long total = static_cast<long long>(num_nodes) * dim;
+        long long blocks = (total + 255) / 256;
+        if (blocks > 256 * 32) blocks = 256 * 32;
+        hipLaunchKernelGGL(scale_rows_flat_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, dst, src,
+                           scale, total, dim);
+    } else {
+        const long long vecs = static_cast<long long>(num_nodes) * (ld_dst / 4);
+        long long blocks = (vecs + 255) / 256;
+        if (blocks > 256 * 32) blocks = 256 * 32;
+        hipLaunchKernelGGL(scale_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, dst, src, scale,
+                           vecs, ld_dst / 4, dim);
+    }
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }
 
-// workspace: nullptr, or num_nodes*dim floats (may alias `in` when the caller gives up the
-// unscaled features).
+static int vector_width(int pitch, int width, const void* p)
+{
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+    if (pitch % 4 == 0 && width % 4 == 0 && a % 16 == 0) return 4;
+    if (pitch % 2 == 0 && width % 2 == 0 && a % 8 == 0) return 2;
+    return 1;
+}
+
+// workspace: nullptr (per-edge scale gather), the input pointer itself (scaled in place, pitch dim)
+// or a separate buffer of feature_workspace_floats() floats (padded pitch).
 template <class Groups>
 static int aggregate_dispatch(float* out, const float* in, const int* col, const float* scale, Groups g,
                               int num_nodes, int dim, int num_parts, float* workspace, hipStream_t stream,
@@ -370,25 +421,43 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
     EPPGCN_HIP(hipMemsetAsync(out, 0, static_cast<size_t>(num_nodes) * dim * sizeof(float), stream));
     if (num_parts == 0) return kOk;
     const bool prescaled = workspace != nullptr;
+    int ld_in = dim;
     if (prescaled) {
-        if (int rc = launch_scale_rows(workspace, in, scale, num_nodes, dim, stream)) return rc;
+        ld_in = workspace == in ? dim : workspace_pitch(dim);
+        if (int rc = launch_scale_rows(workspace, in, scale, num_nodes, dim, ld_in, stream)) return rc;
         in = workspace;
     }
     KernelTimer timer(stream, sink, sink2);   // brackets the aggregation kernel alone
-    const uintptr_t bits = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(in);
-    int vw = 1;
-    if (dim % 4 == 0 && bits % 16 == 0) vw = 4;
-    else if (dim % 2 == 0 && bits % 8 == 0) vw = 2;
-    const int slab = 256 * vw;                          // columns one launch covers
-    for (int c0 = 0; c0 < dim; c0 += slab) {
-        const int width = dim - c0 < slab ? dim - c0 : slab;
+    // rows with the caller's pitch are read and written with the same vector width; padded
+    // workspace rows are read 16 bytes at a time whatever the output alignment allows
+    int ovw_eff = vector_width(dim, dim, out);
+    int vw;
+    if (ld_in == dim) {
+        const int vin = vector_width(dim, dim, in);
+        vw = ovw_eff = vin < ovw_eff ? vin : ovw_eff;
+    } else {
+        vw = vector_width(ld_in, ld_in, in);
+        if (vw < ovw_eff) ovw_eff = vw;
+    }
+    const int slab = 256 * vw;                          // input columns one launch covers
+    for (int c0 = 0; c0 < ld_in; c0 += slab) {
+        if (c0 >= dim) break;
+        AggShape sh;
+        const int in_cols = ld_in - c0 < slab ? ld_in - c0 : slab;
+        sh.chunks = in_cols / vw;
+        sh.ld_in = ld_in;
+        sh.width_out = dim - c0 < slab ? dim - c0 : slab;
+        sh.ld_out = dim;
         hipError_t e;
-#define EPPGCN_SLAB(VW_)                                                                                              \
-    (prescaled ? launch_slab<VW_, true>(out + c0, in + c0, col, scale, g, num_parts, width, dim, stream)              \
-               : launch_slab<VW_, false>(out + c0, in + c0, col, scale, g, num_parts, width, dim, stream))
-        if (vw == 4) e = EPPGCN_SLAB(4);
-        else if (vw == 2) e = EPPGCN_SLAB(2);
-        else e = EPPGCN_SLAB(1);
+#define EPPGCN_SLAB(VW_, OVW_)                                                                                 \
+    (prescaled ? launch_slab<VW_, OVW_, true>(out + c0, in + c0, col, scale, g, num_parts, sh, stream)         \
+               : launch_slab<VW_, OVW_, false>(out + c0, in + c0, col, scale, g, num_parts, sh, stream))
+        if (vw == 4 && ovw_eff == 4) e = EPPGCN_SLAB(4, 4);
+        else if (vw == 4 && ovw_eff == 2) e = EPPGCN_SLAB(4, 2);
+        else if (vw == 4) e = EPPGCN_SLAB(4, 1);
+        else if (vw == 2 && ovw_eff == 2) e = EPPGCN_SLAB(2, 2);
+        else if (vw == 2) e = EPPGCN_SLAB(2, 1);
+        else e = EPPGCN_SLAB(1, 1);
 #undef EPPGCN_SLAB
         if (e != hipSuccess) return hip_fail(e, "aggregate kernel launch");
     }

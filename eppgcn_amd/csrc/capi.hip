@@ -16,6 +16,7 @@ int aggregate_forward_groups(float*, const float*, const int*, const float*, con
 int aggregate_compacted_groups(float*, const float*, const int*, const int*, const int*, const float*, int, int, int,
                                float*, hipStream_t, double*, double*);
 void set_agg_force_team(int);
+size_t feature_workspace_floats(long long, int);
 size_t compact_workspace_bytes(long long);
 size_t split_workspace_bytes(long long);
 int launch_mask_forward(const int*, const int*, const int*, const uint8_t*, uint8_t*, int*, int*, int, long long, int,
@@ -67,7 +68,7 @@ int eppgcn_abi_version(void) { return 2; }
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
                         int dim, int num_parts, int part_size, int dim_worker, int warp_per_block, float* workspace,
-                        void* stream)
+                        size_t workspace_floats, void* stream)
 {
     (void)row_pointers;
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
@@ -76,7 +77,10 @@ int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers
     EPPGCN_REQUIRE(out && in && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (column_index && part_pointers && part2node), "null index pointer");
     EPPGCN_REQUIRE(aligned(out, 4) && aligned(in, 4), "feature pointers must be 4-byte aligned");
-    EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != out), "workspace must be 16-byte aligned and distinct from the output");
+    EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != out),
+                   "workspace must be 16-byte aligned and distinct from the output");
+    EPPGCN_REQUIRE(!workspace || workspace == in || workspace_floats >= feature_workspace_floats(num_nodes, dim),
+                   "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
     return aggregate_forward_groups(out, in, column_index, degrees, part_pointers, part2node, num_nodes, dim, num_parts,
                                     workspace, static_cast<hipStream_t>(stream), &g_for_agg_ms, nullptr);
 }
@@ -84,7 +88,7 @@ int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers
 int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* row_pointers,
                          const int32_t* column_index, const float* degrees, const int32_t* part_pointers,
                          const int32_t* part2node, int num_nodes, int dim, int num_parts, int part_size, int dim_worker,
-                         int warp_per_block, float* workspace, void* stream)
+                         int warp_per_block, float* workspace, size_t workspace_floats, void* stream)
 {
     (void)row_pointers;
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
@@ -93,14 +97,18 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
     EPPGCN_REQUIRE(d_input && d_output && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (column_index && part_pointers && part2node), "null index pointer");
     EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
-    EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != d_input), "workspace must be 16-byte aligned and distinct from the output");
+    EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != d_input),
+                   "workspace must be 16-byte aligned and distinct from the output");
+    EPPGCN_REQUIRE(!workspace || workspace == d_output || workspace_floats >= feature_workspace_floats(num_nodes, dim),
+                   "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
     return aggregate_forward_groups(d_input, d_output, column_index, degrees, part_pointers, part2node, num_nodes, dim,
                                     num_parts, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms, nullptr);
 }
 
 int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
                          const int32_t* edge_list, const float* degrees, int num_nodes, int dim, int num_parts,
-                         int part_size, int layer, int blockx, int blocky, float* workspace, void* stream)
+                         int part_size, int layer, int blockx, int blocky, float* workspace,
+                         size_t workspace_floats, void* stream)
 {
     (void)part_size;   // the reference's kernel ignores it too (EPPGCN_kernel.cu:636)
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
@@ -110,7 +118,10 @@ int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* i
     EPPGCN_REQUIRE(d_input && d_output && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (ids && part_pointer && edge_list), "null index pointer");
     EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
-    EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != d_input), "workspace must be 16-byte aligned and distinct from the output");
+    EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != d_input),
+                   "workspace must be 16-byte aligned and distinct from the output");
+    EPPGCN_REQUIRE(!workspace || workspace == d_output || workspace_floats >= feature_workspace_floats(num_nodes, dim),
+                   "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
     return aggregate_compacted_groups(d_input, d_output, ids, part_pointer, edge_list, degrees, num_nodes, dim,
                                       num_parts, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms,
                                       layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr);
@@ -131,6 +142,10 @@ int eppgcn_mask_forward(const int32_t* part2node, const int32_t* part_pointers, 
                                num_parts, num_edges, is_last_layer ? 1 : 0, static_cast<hipStream_t>(stream));
 }
 
+size_t eppgcn_feature_workspace_floats(int64_t num_nodes, int dim)
+{
+    return (num_nodes <= 0 || dim <= 0) ? 0 : feature_workspace_floats(num_nodes, dim);
+}
 size_t eppgcn_compact_workspace_bytes(int64_t length) { return compact_workspace_bytes(length < 0 ? 0 : length); }
 size_t eppgcn_split_workspace_bytes(int64_t num_nodes) { return split_workspace_bytes(num_nodes < 0 ? 0 : num_nodes); }
 

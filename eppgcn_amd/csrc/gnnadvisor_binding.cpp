@@ -60,6 +60,12 @@ Tensor workspace(size_t bytes, const Tensor& like)
     return torch::empty({static_cast<int64_t>((bytes + 7) / 8)}, like.options().dtype(torch::kInt64));
 }
 
+Tensor feature_scratch(const Tensor& feats)
+{
+    const size_t n = eppgcn_feature_workspace_floats(feats.size(0), static_cast<int>(feats.size(1)));
+    return torch::empty({static_cast<int64_t>(n)}, feats.options());
+}
+
 // ---------------------------------------------------------------- forward / backward
 std::vector<Tensor> forward(Tensor input, Tensor weight, Tensor row_pointers, Tensor column_index, Tensor degrees,
                             Tensor part_pointers, Tensor part2Node, int partSize, int dimWorker, int warpPerBlock)
@@ -71,10 +77,15 @@ std::vector<Tensor> forward(Tensor input, Tensor weight, Tensor row_pointers, Te
     TORCH_CHECK(part_pointers.numel() >= part2Node.numel() + 1, "part_pointers needs num_parts + 1 entries");
     auto tmp = torch::mm(input, weight);
     auto output = torch::empty_like(tmp);
+    // tmp is ours: when its rows need no padding it is scaled in place, otherwise into scratch
+    const size_t ws_floats = eppgcn_feature_workspace_floats(tmp.size(0), static_cast<int>(tmp.size(1)));
+    auto scaled = ws_floats == static_cast<size_t>(tmp.numel())
+                      ? tmp
+                      : torch::empty({static_cast<int64_t>(ws_floats)}, tmp.options());
     check(eppgcn_spmm_forward(output.data_ptr<float>(), tmp.data_ptr<float>(), i32(row_pointers), i32(column_index),
                               f32(degrees), i32(part_pointers), i32(part2Node), static_cast<int>(tmp.size(0)),
                               static_cast<int>(tmp.size(1)), static_cast<int>(part2Node.numel()), partSize, dimWorker,
-                              warpPerBlock, tmp.data_ptr<float>() /* scaled in place: tmp is ours */, stream_of(input)),
+                              warpPerBlock, scaled.data_ptr<float>(), ws_floats, stream_of(input)),
           "forward");
     return {output};
 }
@@ -88,12 +99,12 @@ std::vector<Tensor> backward(Tensor d_output, Tensor X, Tensor W, Tensor row_poi
     TORCH_CHECK(d_output.dim() == 2 && degrees.numel() == d_output.size(0), "shape mismatch");
     TORCH_CHECK(part_pointers.numel() >= part2Node.numel() + 1, "part_pointers needs num_parts + 1 entries");
     auto d_input_prime = torch::empty_like(d_output);
-    auto scaled = torch::empty_like(d_output);   // d_output belongs to autograd: scale into scratch
+    auto scaled = feature_scratch(d_output);     // d_output belongs to autograd: scale into scratch
     check(eppgcn_spmm_backward(d_input_prime.data_ptr<float>(), d_output.data_ptr<float>(), i32(row_pointers),
                                i32(column_index), f32(degrees), i32(part_pointers), i32(part2Node),
                                static_cast<int>(d_output.size(0)), static_cast<int>(d_output.size(1)),
                                static_cast<int>(part2Node.numel()), partSize, dimWorker, warpPerBlock,
-                               scaled.data_ptr<float>(), stream_of(d_output)),
+                               scaled.data_ptr<float>(), static_cast<size_t>(scaled.numel()), stream_of(d_output)),
           "backward");
     auto d_input = torch::mm(d_input_prime, W.transpose(0, 1));
     auto d_weight = torch::mm(X.transpose(0, 1), d_input_prime);
@@ -128,11 +139,12 @@ std::vector<Tensor> ours_backward(Tensor d_output, Tensor X, Tensor W, Tensor id
     TORCH_CHECK(numParts >= 0 && partPointer.numel() >= static_cast<int64_t>(numParts) + 1,
                 "partPointer needs numParts + 1 entries");
     auto d_input_prime = torch::empty_like(d_output);
-    auto scaled = torch::empty_like(d_output);   // d_output belongs to autograd: scale into scratch
+    auto scaled = feature_scratch(d_output);     // d_output belongs to autograd: scale into scratch
     check(eppgcn_ours_backward(d_input_prime.data_ptr<float>(), d_output.data_ptr<float>(), i32(id), i32(partPointer),
                                i32(edgeList), f32(degrees), static_cast<int>(d_output.size(0)),
                                static_cast<int>(d_output.size(1)), numParts, partSize > 0 ? partSize : 1, layer, blockx,
-                               blocky, scaled.data_ptr<float>(), stream_of(d_output)),
+                               blocky, scaled.data_ptr<float>(), static_cast<size_t>(scaled.numel()),
+                               stream_of(d_output)),
           "ours_backward");
     auto d_input = torch::mm(d_input_prime, W.transpose(0, 1));
     auto d_weight = torch::mm(X.transpose(0, 1), d_input_prime);

@@ -22,13 +22,15 @@
  *     matching *_workspace_bytes() call returns, 8-byte aligned.  The library
  *     itself allocates no device memory.
  *   - The aggregation functions take an optional feature workspace of
- *     num_nodes*dim floats (16-byte aligned).  With it the features are scaled
- *     by `degrees` once per call and the kernel gathers pre-scaled rows, which
- *     removes one random memory request per edge; with NULL the kernel gathers
- *     the neighbour's scale per edge and needs no scratch.  The workspace may be
- *     the input pointer itself when the caller no longer needs the unscaled
- *     input (it is then overwritten with degrees[r]*in[r,:]).  Results of the
- *     two modes agree to rounding (a few ulp per term).
+ *     eppgcn_feature_workspace_floats(num_nodes, dim) floats, 16-byte aligned
+ *     (its size is passed as workspace_floats and checked).  With it the
+ *     features are scaled by `degrees` once per call into rows padded to whole
+ *     32-byte sectors and the kernel gathers pre-scaled rows, which removes one
+ *     random memory request per edge; with NULL the kernel gathers the
+ *     neighbour's scale per edge and needs no scratch.  The workspace may be the
+ *     input pointer itself when the caller no longer needs the unscaled input
+ *     (it is then overwritten with degrees[r]*in[r,:], unpadded).  Results of the
+ *     modes agree to rounding (a few ulp per term).
  */
 #ifndef EPPGCN_HIP_H_
 #define EPPGCN_HIP_H_
@@ -55,6 +57,9 @@ int eppgcn_abi_version(void);
  * Aggregation.
  * ------------------------------------------------------------------------- */
 
+/* Floats a separate feature workspace must hold for [num_nodes, dim] features. */
+size_t eppgcn_feature_workspace_floats(int64_t num_nodes, int dim);
+
 /* Forward neighbour-group aggregation:
  *   out[r,:] = sum_{e in groups of r} fl32(degrees[r]*degrees[col[e]]) * in[col[e],:]
  * `out` ([num_nodes, dim]) is fully overwritten (rows without groups become 0).
@@ -68,7 +73,7 @@ int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers
                         const int32_t* part_pointers, const int32_t* part2node,
                         int num_nodes, int dim, int num_parts,
                         int part_size, int dim_worker, int warp_per_block,
-                        float* workspace, void* stream);
+                        float* workspace, size_t workspace_floats, void* stream);
 
 /* Unpruned backward aggregation: the same operator applied to d_output (valid
  * because the normalised adjacency is symmetric).  Stands in for
@@ -79,7 +84,7 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
                          const int32_t* part_pointers, const int32_t* part2node,
                          int num_nodes, int dim, int num_parts,
                          int part_size, int dim_worker, int warp_per_block,
-                         float* workspace, void* stream);
+                         float* workspace, size_t workspace_floats, void* stream);
 
 /* Pruned backward aggregation over the compacted execution path:
  *   d_input[id_p,:] += sum_{k in group p} fl32(degrees[id_p]*degrees[edge_list[k]]) * d_output[edge_list[k],:]
@@ -91,7 +96,7 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
 int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids,
                          const int32_t* part_pointer, const int32_t* edge_list, const float* degrees,
                          int num_nodes, int dim, int num_parts, int part_size, int layer,
-                         int blockx, int blocky, float* workspace, void* stream);
+                         int blockx, int blocky, float* workspace, size_t workspace_floats, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Execution-path preparation.
