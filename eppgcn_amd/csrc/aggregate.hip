@@ -38,6 +38,11 @@ namespace eppgcn {
 constexpr int kAggBlock = 256;
 constexpr int kAggWaves = kAggBlock / kWave;
 constexpr int kStageCap = 512;   // staged slots per wave and pass
+// Staged slot s lives at LDS word s + s/32: teams read their groups at strides that are
+// often a power of two (a backward group size of 32 puts all 16 teams of a wave on one bank);
+// one pad word per 32 slots spreads such strides over the 32 banks.
+constexpr int kStageWords = kStageCap + kStageCap / 32;
+__device__ __forceinline__ int stage_index(int slot) { return slot + (slot >> 5); }
 
 // ---------------------------------------------------------------- vectors
 template <int VW> struct Vec;
@@ -134,8 +139,8 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
 {
     constexpr int TPW = kWave / TS;      // teams (= groups) per wave
     using V = Vec<VW>;
-    __shared__ int stage_col[kAggWaves][kStageCap];
-    __shared__ float stage_scale[kAggWaves][kPrescaled ? 1 : kStageCap];
+    __shared__ int stage_col[kAggWaves][kStageWords];
+    __shared__ float stage_scale[kAggWaves][kPrescaled ? 1 : kStageWords];
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
@@ -189,13 +194,13 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
 #pragma unroll
                 for (int r = 0; r < kStageCap / kWave; ++r) {
                     const int i = lane + r * kWave;
-                    if (i < cn) my_scale[i] = sc[r];
+                    if (i < cn) my_scale[stage_index(i)] = sc[r];
                 }
             }
 #pragma unroll
             for (int r = 0; r < kStageCap / kWave; ++r) {
                 const int i = lane + r * kWave;
-                if (i < cn) my_col[i] = c[r];
+                if (i < cn) my_col[stage_index(i)] = c[r];
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -211,7 +216,7 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const bool ok = i + u < hi;
-                const int slot = ok ? i + u - cb : 0;
+                const int slot = stage_index(ok ? i + u - cb : 0);
                 const int c = my_col[slot];
                 if constexpr (!kPrescaled) w[u] = ok ? s_row * my_scale[slot] : 0.f;
                 const float* src = in + static_cast<size_t>(c) * ld_in;

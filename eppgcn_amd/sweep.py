@@ -1,0 +1,104 @@
+"""Backward-path stress sweep (benchmark configuration 5): on one graph, train-mask ratios x
+aggregation widths x backward group sizes.  For every cell: path-preparation time (marking,
+compaction, split), pruned backward time, unpruned backward time, algorithmic GB/s.
+
+    python -m eppgcn_amd.sweep [--config cfg3_rmat20] [--ratios 0.01 0.1 0.5]
+                               [--widths 16 64 256] [--groups 8 16 32 64] [--reps 5]
+
+Prints one JSON line per cell and a final summary line.  Needs the MI355X.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import time
+
+import torch
+
+from . import capi, graphs, workload
+
+
+def _events_ms(fn, reps):
+    fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / reps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--config", default="cfg3_rmat20")
+    ap.add_argument("--ratios", type=float, nargs="+", default=[0.01, 0.1, 0.5])
+    ap.add_argument("--widths", type=int, nargs="+", default=[16, 64, 256])
+    ap.add_argument("--groups", type=int, nargs="+", default=[8, 16, 32, 64])
+    ap.add_argument("--reps", type=int, default=5)
+    args = ap.parse_args()
+
+    capi.load()
+    dev = torch.device("cuda:0")
+    g = graphs.make_graph(args.config, device=dev)
+    n, e = g.num_nodes, g.num_edges
+    ps = max(1, int(g.avg_degree))
+    part_ptr, part2node = capi.build_part(ps, g.row_pointers, e)
+    cells = []
+    for ratio in args.ratios:
+        mask = graphs.bernoulli_mask(n, ratio, 2, dev)
+        bem = torch.full((e,), -1, dtype=torch.int32, device=dev)
+        degs = torch.zeros(n, dtype=torch.int32, device=dev)
+
+        def mark():
+            bem.fill_(-1)
+            degs.zero_()
+            capi.mask_forward(part2node, part_ptr, g.column_index, mask, None, bem, degs, True)
+
+        mark_ms = _events_ms(mark, args.reps)
+        compact_ms = _events_ms(lambda: capi.compact_back_edge(bem, g.column_index), args.reps)
+        ids, edge_list, valid_len = capi.compact_back_edge(bem, g.column_index)
+        valid_node = capi.count_nonzero(degs)
+        for gs in args.groups:
+            split_ms = _events_ms(lambda: capi.split_back_part(degs, e, gs), args.reps)
+            part_pointer, num_parts, _ = capi.split_back_part(degs, e, gs)
+            for width in args.widths:
+                dy = graphs.normal32(7, (n, width), dev) * mask[:, None]
+                out = torch.empty_like(dy)
+                ws = capi.feature_workspace(n, width, dev)
+                capi.set_timing(True)
+                capi.clear_time()
+                for _ in range(args.reps):
+                    capi.ours_backward(dy, ids, part_pointer, edge_list, g.degrees, num_parts, gs, 1, 4, 16, out, ws)
+                pruned_ms = capi.get_time_ms(1) / args.reps
+                capi.clear_time()
+                for _ in range(args.reps):
+                    capi.spmm_forward(dy, g.column_index, g.degrees, part_ptr, part2node, ps, 32, 8, None, out, True, ws)
+                unpruned_ms = capi.get_time_ms(1) / args.reps
+                capi.set_timing(False)
+                capi.clear_time()
+                nbytes = workload.bytes_pruned_backward(n, valid_len, num_parts, width)
+                cell = {"config": args.config, "ratio": ratio, "width": width, "group_size": gs,
+                        "kept_edges": valid_len, "kept_rows": valid_node, "groups": num_parts,
+                        "mark_ms": round(mark_ms, 4), "compact_ms": round(compact_ms, 4), "split_ms": round(split_ms, 4),
+                        "pruned_bwd_ms": round(pruned_ms, 4), "unpruned_bwd_ms": round(unpruned_ms, 4),
+                        "pruned_GBps": round(nbytes / pruned_ms / 1e6, 1),
+                        "unpruned_GBps": round(workload.bytes_forward(n, e, width) / unpruned_ms / 1e6, 1),
+                        "speedup": round(unpruned_ms / pruned_ms, 2)}
+                cells.append(cell)
+                print(json.dumps(cell), flush=True)
+    best = {}
+    for c in cells:
+        key = (c["ratio"], c["width"])
+        if key not in best or c["pruned_bwd_ms"] < best[key]["pruned_bwd_ms"]:
+            best[key] = c
+    print(json.dumps({"summary": "best group size per (ratio, width)",
+                      "best": [{"ratio": k[0], "width": k[1], "group_size": v["group_size"],
+                                "pruned_bwd_ms": v["pruned_bwd_ms"], "speedup": v["speedup"]}
+                               for k, v in sorted(best.items())]}), flush=True)
+
+
+if __name__ == "__main__":
+    t0 = time.time()
+    main()
