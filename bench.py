@@ -38,6 +38,7 @@ def parse():
     ap.add_argument("--backsize", type=int, default=32)
     ap.add_argument("--part_size", type=int, default=0, help="forward group size (0 = int(avg degree))")
     ap.add_argument("--team", type=int, default=0, help="force lanes per group (0 = automatic)")
+    ap.add_argument("--rounds", type=int, default=0, help="force group rounds per wave (0 = automatic)")
     ap.add_argument("--no_workspace", action="store_true",
                     help="aggregate without the feature workspace (per-edge scale gather, no scratch)")
     ap.add_argument("--no_cpu_baseline", action="store_true")
@@ -93,6 +94,8 @@ def main():
     p_last, p_first = wl.paths[1], wl.paths[0]
     if args.team:
         capi.set_team_size(args.team)
+    if args.rounds:
+        capi.set_rounds(args.rounds)
 
     def fwd16():
         capi.spmm_forward(x16, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 32, 8,

@@ -20,7 +20,7 @@ EXPORTS = [
     "eppgcn_split_workspace_bytes", "eppgcn_compact_back_edge", "eppgcn_count_nonzero",
     "eppgcn_map_back_part_size", "eppgcn_threshold_back_part_size", "eppgcn_split_back_part",
     "eppgcn_build_part", "eppgcn_get_ginfo", "eppgcn_set_timing", "eppgcn_print_time",
-    "eppgcn_clear_time", "eppgcn_get_time_ms", "eppgcn_set_team_size",
+    "eppgcn_clear_time", "eppgcn_get_time_ms", "eppgcn_set_team_size", "eppgcn_set_rounds",
 ]
 
 _lib = None
@@ -67,6 +67,8 @@ def load():
     lib.eppgcn_get_time_ms.restype = C.c_double
     lib.eppgcn_set_team_size.argtypes = [i]
     lib.eppgcn_set_team_size.restype = None
+    lib.eppgcn_set_rounds.argtypes = [i]
+    lib.eppgcn_set_rounds.restype = None
     for name in ("eppgcn_spmm_forward", "eppgcn_spmm_backward", "eppgcn_ours_backward", "eppgcn_mask_forward",
                  "eppgcn_compact_back_edge", "eppgcn_count_nonzero", "eppgcn_map_back_part_size",
                  "eppgcn_threshold_back_part_size", "eppgcn_split_back_part", "eppgcn_build_part",
@@ -288,3 +290,7 @@ def get_time_ms(which: int) -> float:
 
 def set_team_size(lanes: int):
     load().eppgcn_set_team_size(int(lanes))
+
+
+def set_rounds(rounds: int):
+    load().eppgcn_set_rounds(int(rounds))

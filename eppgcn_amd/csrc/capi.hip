@@ -12,10 +12,11 @@ namespace eppgcn {
 
 // ---- implemented in aggregate.hip / prepare.hip
 int aggregate_forward_groups(float*, const float*, const int*, const float*, const int*, const int*, int, int, int,
-                             float*, hipStream_t, double*, double*);
+                             int, float*, hipStream_t, double*, double*);
 int aggregate_compacted_groups(float*, const float*, const int*, const int*, const int*, const float*, int, int, int,
-                               float*, hipStream_t, double*, double*);
+                               int, float*, hipStream_t, double*, double*);
 void set_agg_force_team(int);
+void set_agg_force_rounds(int);
 size_t feature_workspace_floats(long long, int);
 size_t compact_workspace_bytes(long long);
 size_t split_workspace_bytes(long long);
@@ -82,7 +83,7 @@ int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers
     EPPGCN_REQUIRE(!workspace || workspace == in || workspace_floats >= feature_workspace_floats(num_nodes, dim),
                    "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
     return aggregate_forward_groups(out, in, column_index, degrees, part_pointers, part2node, num_nodes, dim, num_parts,
-                                    workspace, static_cast<hipStream_t>(stream), &g_for_agg_ms, nullptr);
+                                    part_size, workspace, static_cast<hipStream_t>(stream), &g_for_agg_ms, nullptr);
 }
 
 int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* row_pointers,
@@ -102,7 +103,7 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
     EPPGCN_REQUIRE(!workspace || workspace == d_output || workspace_floats >= feature_workspace_floats(num_nodes, dim),
                    "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
     return aggregate_forward_groups(d_input, d_output, column_index, degrees, part_pointers, part2node, num_nodes, dim,
-                                    num_parts, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms, nullptr);
+                                    num_parts, part_size, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms, nullptr);
 }
 
 int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
@@ -110,7 +111,7 @@ int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* i
                          int part_size, int layer, int blockx, int blocky, float* workspace,
                          size_t workspace_floats, void* stream)
 {
-    (void)part_size;   // the reference's kernel ignores it too (EPPGCN_kernel.cu:636)
+    // part_size only sizes the work per wave (the reference's kernel ignores it, EPPGCN_kernel.cu:636)
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
     EPPGCN_REQUIRE(blockx > 0 && blocky > 0, "launch hints must be positive");
     EPPGCN_REQUIRE(layer >= 1, "layer is 1-based");
@@ -123,7 +124,7 @@ int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* i
     EPPGCN_REQUIRE(!workspace || workspace == d_output || workspace_floats >= feature_workspace_floats(num_nodes, dim),
                    "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
     return aggregate_compacted_groups(d_input, d_output, ids, part_pointer, edge_list, degrees, num_nodes, dim,
-                                      num_parts, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms,
+                                      num_parts, part_size > 0 ? part_size : 1, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms,
                                       layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr);
 }
 
@@ -315,5 +316,6 @@ double eppgcn_get_time_ms(int which)
 }
 
 void eppgcn_set_team_size(int lanes) { set_agg_force_team(lanes); }
+void eppgcn_set_rounds(int rounds) { set_agg_force_rounds(rounds); }
 
 }  // extern "C"

@@ -186,6 +186,9 @@ double eppgcn_get_time_ms(int which);
 /* Forces the number of lanes per neighbour group in the aggregation kernels
  * (power of two in 4..64; 0 = choose from the feature width).  For tuning runs. */
 void eppgcn_set_team_size(int lanes);
+/* Forces the number of consecutive group rounds one wave processes (0 = choose from
+ * the group size so that a wave gathers about 512 rows).  For tuning runs. */
+void eppgcn_set_rounds(int rounds);
 
 #ifdef __cplusplus
 }

@@ -207,6 +207,37 @@ def test_forward_aggregation_forced_team_sizes(api, team, dim):
         api.set_team_size(0)
 
 
+@pytest.mark.parametrize("rounds", [1, 2, 3, 7, 64])
+@pytest.mark.parametrize("dim", [16, 22, 64, 256])
+def test_forward_and_pruned_forced_rounds_exact_integer_sums(api, rounds, dim):
+    """Waves that process several consecutive group rounds carry a row's partial sum from one
+    round to the next: with s == 1 and small integer features the result must still be exactly
+    the neighbour sum, for rows shorter than a group and rows spanning many rounds and waves."""
+    indptr, col = hub_csr(3000, 2500, 17)
+    n = indptr.size - 1
+    x = np.random.default_rng(rounds).integers(-8, 9, (n, dim)).astype(np.float32)
+    s = np.ones(n, np.float32)
+    want = np.zeros((n, dim), np.float64)
+    np.add.at(want, cf.row_index(indptr), x[col].astype(np.float64))
+    src = np.random.default_rng(3).random(n) < 0.4
+    want_b = np.zeros((n, dim), np.float64)
+    keep = src[col]
+    np.add.at(want_b, cf.row_index(indptr)[keep], (x * src[:, None])[col[keep]].astype(np.float64))
+    try:
+        api.set_rounds(rounds)
+        for ps in (1, 2, 9, 32):
+            pp, p2n = co.build_part(ps, indptr)
+            for ws in (None, True):
+                got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp), dev(p2n), part_size=ps, workspace=ws)
+                assert np.array_equal(got.cpu().numpy().astype(np.float64), want), f"ps={ps} ws={ws}"
+            oid, oedge, bpp, p = _gpu_path(api, indptr, col, src, 5, ps)
+            dy = dev((x * src[:, None]).astype(np.float32))
+            gb = api.ours_backward(dy, oid, bpp, oedge, dev(s), p, part_size=ps)
+            assert np.array_equal(gb.cpu().numpy().astype(np.float64), want_b), f"pruned ps={ps}"
+    finally:
+        api.set_rounds(0)
+
+
 def test_forward_unit_scale_integer_features_bit_exact(api):
     """With s == 1 and small integer features every partial sum is exact in fp32, so any
     grouping, lane mapping or atomic order must give exactly the neighbour sum."""
