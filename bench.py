@@ -39,6 +39,10 @@ def parse():
     ap.add_argument("--part_size", type=int, default=0, help="forward group size (0 = int(avg degree))")
     ap.add_argument("--team", type=int, default=0, help="force lanes per group (0 = automatic)")
     ap.add_argument("--rounds", type=int, default=0, help="force group rounds per wave (0 = automatic)")
+    ap.add_argument("--plan_shift", type=int, default=0, help="force log2 of the plan's column block")
+    ap.add_argument("--plan_keep", type=int, default=-1, help="rows with at most this many groups stay together")
+    ap.add_argument("--no_plan", action="store_true",
+                    help="process the groups in CSR order instead of the column-blocked execution plan")
     ap.add_argument("--no_workspace", action="store_true",
                     help="aggregate without the feature workspace (per-edge scale gather, no scratch)")
     ap.add_argument("--no_cpu_baseline", action="store_true")
@@ -75,8 +79,13 @@ def main():
     g = graphs.make_graph(args.config, device=dev)
     torch.cuda.synchronize()
     log(args, "graph", g.stats(), f"{time.perf_counter() - t0:.1f}s")
+    if args.plan_shift:
+        capi.set_plan_shift(args.plan_shift)
+    if args.plan_keep >= 0:
+        capi.set_plan_keep_rows(args.plan_keep)
     t0 = time.perf_counter()
-    wl = workload.prepare(g, 2, args.train_ratio, 2, args.part_size or None, args.backsize_mode, args.backsize)
+    wl = workload.prepare(g, 2, args.train_ratio, 2, args.part_size or None, args.backsize_mode, args.backsize,
+                          plan=not (args.no_plan or args.no_workspace))
     torch.cuda.synchronize()
     prep_s = time.perf_counter() - t0
     n, e = g.num_nodes, g.num_edges
@@ -99,19 +108,20 @@ def main():
 
     def fwd16():
         capi.spmm_forward(x16, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 32, 8,
-                          g.row_pointers, out16, workspace=ws16)
+                          g.row_pointers, out16, workspace=ws16, plan=wl.plans.get(16))
 
     def fwd22():
         capi.spmm_forward(x22, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 16, 8,
-                          g.row_pointers, out22, workspace=ws22)
+                          g.row_pointers, out22, workspace=ws22, plan=wl.plans.get(22))
 
     def bwd22():
         capi.ours_backward(dy22, p_last.ids, p_last.part_pointer, p_last.edge_list, g.degrees, p_last.num_parts,
-                           p_last.part_size, 2, 4, 16, out22, workspace=ws22)
+                           p_last.part_size, 2, 4, 16, out22, workspace=ws22, plan=p_last.plan)
 
     def bwd16():
         capi.ours_backward(dy16, p_first.ids, p_first.part_pointer, p_first.edge_list, g.degrees,
-                           p_first.num_parts, p_first.part_size, 1, 4, 16, out16, workspace=ws16)
+                           p_first.num_parts, p_first.part_size, 1, 4, 16, out16, workspace=ws16,
+                           plan=p_first.plan)
 
     kernels = [
         ("fwd_agg_d16", fwd16, workload.bytes_forward(n, e, 16)),
@@ -174,7 +184,8 @@ def main():
                    "backward_group_size": [p.part_size for p in wl.paths],
                    "kept_edges": [p.valid_len for p in wl.paths],
                    "backward_groups": [p.num_parts for p in wl.paths], "max_degree": g.stats()["max_degree"],
-                   "feature_workspace": not args.no_workspace},
+                   "feature_workspace": not args.no_workspace,
+                   "column_blocked_plan": not (args.no_plan or args.no_workspace)},
         "agg_ms_per_epoch": round(ms_per_step, 4), "alg_bytes_per_epoch": bytes_epoch,
         "pct_of_peak_hbm": round(value / PEAK_HBM_GBS * 100, 2),
         "per_kernel": per_kernel, "path_preparation_s": round(prep_s, 3),

@@ -15,12 +15,13 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("EPPGCN_HIP_LIB") or os.path.join(_HERE, "lib", "libeppgcn_hip.so")
 
 EXPORTS = [
-    "eppgcn_last_error", "eppgcn_abi_version", "eppgcn_feature_workspace_floats", "eppgcn_spmm_forward", "eppgcn_spmm_backward",
+    "eppgcn_last_error", "eppgcn_abi_version", "eppgcn_feature_workspace_floats", "eppgcn_plan_bytes",
+    "eppgcn_plan_workspace_bytes", "eppgcn_build_plan", "eppgcn_spmm_forward", "eppgcn_spmm_backward",
     "eppgcn_ours_backward", "eppgcn_mask_forward", "eppgcn_compact_workspace_bytes",
     "eppgcn_split_workspace_bytes", "eppgcn_compact_back_edge", "eppgcn_count_nonzero",
     "eppgcn_map_back_part_size", "eppgcn_threshold_back_part_size", "eppgcn_split_back_part",
     "eppgcn_build_part", "eppgcn_get_ginfo", "eppgcn_set_timing", "eppgcn_print_time",
-    "eppgcn_clear_time", "eppgcn_get_time_ms", "eppgcn_set_team_size", "eppgcn_set_rounds",
+    "eppgcn_clear_time", "eppgcn_get_time_ms", "eppgcn_set_team_size", "eppgcn_set_rounds", "eppgcn_set_plan_shift", "eppgcn_set_plan_keep_rows",
 ]
 
 _lib = None
@@ -44,9 +45,15 @@ def load():
     lib.eppgcn_abi_version.restype = i
     lib.eppgcn_feature_workspace_floats.argtypes = [i64, i]
     lib.eppgcn_feature_workspace_floats.restype = sz
-    lib.eppgcn_spmm_forward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, sz, p]
-    lib.eppgcn_spmm_backward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, sz, p]
-    lib.eppgcn_ours_backward.argtypes = [p, p, p, p, p, p, i, i, i, i, i, i, i, p, sz, p]
+    lib.eppgcn_plan_bytes.argtypes = [i64, i64]
+    lib.eppgcn_plan_bytes.restype = sz
+    lib.eppgcn_plan_workspace_bytes.argtypes = [i64]
+    lib.eppgcn_plan_workspace_bytes.restype = sz
+    lib.eppgcn_build_plan.argtypes = [p, p, p, p, i, i64, i, i, p, sz, p, sz, p]
+    lib.eppgcn_build_plan.restype = i
+    lib.eppgcn_spmm_forward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, sz, p, p]
+    lib.eppgcn_spmm_backward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, sz, p, p]
+    lib.eppgcn_ours_backward.argtypes = [p, p, p, p, p, p, i, i, i, i, i, i, i, p, sz, p, p]
     lib.eppgcn_mask_forward.argtypes = [p, p, p, p, p, p, p, i, i64, i, i, i, p]
     lib.eppgcn_compact_workspace_bytes.argtypes = [i64]
     lib.eppgcn_compact_workspace_bytes.restype = sz
@@ -69,6 +76,10 @@ def load():
     lib.eppgcn_set_team_size.restype = None
     lib.eppgcn_set_rounds.argtypes = [i]
     lib.eppgcn_set_rounds.restype = None
+    lib.eppgcn_set_plan_shift.argtypes = [i]
+    lib.eppgcn_set_plan_shift.restype = None
+    lib.eppgcn_set_plan_keep_rows.argtypes = [i]
+    lib.eppgcn_set_plan_keep_rows.restype = None
     for name in ("eppgcn_spmm_forward", "eppgcn_spmm_backward", "eppgcn_ours_backward", "eppgcn_mask_forward",
                  "eppgcn_compact_back_edge", "eppgcn_count_nonzero", "eppgcn_map_back_part_size",
                  "eppgcn_threshold_back_part_size", "eppgcn_split_back_part", "eppgcn_build_part",
@@ -129,8 +140,62 @@ def feature_workspace(num_nodes: int, dim: int, device):
                        device=device)
 
 
+class Plan:
+    """A column-blocked execution plan (device buffer + the sizes it was built for)."""
+
+    def __init__(self, buffer, base_ptr, num_parts, num_slots):
+        self.buffer, self.base_ptr, self.num_parts, self.num_slots = buffer, base_ptr, num_parts, num_slots
+
+    def view(self):
+        """(ptr, row, flags, col) as torch tensors, for tests."""
+        def al(x):
+            return (x + 255) // 256 * 256
+        p, s = self.num_parts, self.num_slots
+        off = self.base_ptr - self.buffer.data_ptr()
+        raw = self.buffer.view(torch.uint8)
+        o1 = off + al(4 * (p + 1)); o2 = o1 + al(4 * p); o3 = o2 + al(p)
+        return (raw[off: off + 4 * (p + 1)].view(torch.int32), raw[o1: o1 + 4 * p].view(torch.int32),
+                raw[o2: o2 + p], raw[o3: o3 + 4 * s].view(torch.int32))
+
+
+def _aligned_buffer(nbytes, device):
+    buf = torch.empty(nbytes + 256, dtype=torch.uint8, device=device)
+    return buf, (buf.data_ptr() + 255) // 256 * 256
+
+
+def build_plan(part_ptr, column_index, num_parts: int, num_slots: int, num_nodes: int, dim: int,
+               part2node=None, ids=None):
+    """Column-blocked execution plan of the groups; build once per graph and group array and pass it
+    as ``plan=`` to the aggregation calls.  Forward groups: give part2node; backward path: give ids."""
+    lib = load()
+    _dev(part_ptr, torch.int32, "part_ptr"); _dev(column_index, torch.int32, "column_index")
+    if (part2node is None) == (ids is None):
+        raise EppgcnError("give exactly one of part2node (forward groups) and ids (backward path)")
+    if part_ptr.numel() < num_parts + 1:
+        raise EppgcnError("part_ptr needs num_parts + 1 entries")
+    if column_index.numel() < num_slots:
+        raise EppgcnError("column_index is shorter than num_slots")
+    nbytes = lib.eppgcn_plan_bytes(int(num_parts), int(num_slots))
+    buf, base = _aligned_buffer(nbytes, part_ptr.device)
+    wbytes = lib.eppgcn_plan_workspace_bytes(int(num_parts))
+    ws, wbase = _aligned_buffer(wbytes, part_ptr.device)
+    _check(lib.eppgcn_build_plan(_ptr(part_ptr), _ptr(column_index), _ptr(part2node), _ptr(ids), int(num_parts),
+                                 int(num_slots), int(num_nodes), int(dim), C.c_void_p(base), nbytes,
+                                 C.c_void_p(wbase), wbytes, _stream()))
+    torch.cuda.current_stream().synchronize()      # the workspace is released on return
+    return Plan(buf, base, int(num_parts), int(num_slots))
+
+
+def _plan_ptr(plan, num_parts):
+    if plan is None:
+        return None
+    if plan.num_parts != num_parts:
+        raise EppgcnError("the plan was built for a different number of groups")
+    return C.c_void_p(plan.base_ptr)
+
+
 def spmm_forward(feats, column_index, degrees, part_ptr, part2node, part_size=32, dim_worker=32,
-                 warp_per_block=8, row_pointers=None, out=None, backward=False, workspace=True):
+                 warp_per_block=8, row_pointers=None, out=None, backward=False, workspace=True, plan=None):
     """out[N, D] = neighbour-group aggregation of feats (``backward=True`` uses the unpruned
     backward entry point; same operator)."""
     lib = load()
@@ -149,12 +214,12 @@ def spmm_forward(feats, column_index, degrees, part_ptr, part2node, part_size=32
     ws = _feature_workspace(workspace, feats)
     _check(fn(_ptr(out), _ptr(feats), _ptr(row_pointers), _ptr(column_index), _ptr(degrees), _ptr(part_ptr),
               _ptr(part2node), n, dim, num_parts, part_size, dim_worker, warp_per_block, _ptr(ws),
-              0 if ws is None else ws.numel(), _stream()))
+              0 if ws is None else ws.numel(), _plan_ptr(plan, num_parts), _stream()))
     return out
 
 
 def ours_backward(d_output, ids, part_pointer, edge_list, degrees, num_parts, part_size=32, layer=1,
-                  blockx=4, blocky=16, out=None, workspace=True):
+                  blockx=4, blocky=16, out=None, workspace=True, plan=None):
     lib = load()
     _dev(d_output, torch.float32, "d_output"); _dev(ids, torch.int32, "ids")
     _dev(part_pointer, torch.int32, "part_pointer"); _dev(edge_list, torch.int32, "edge_list")
@@ -167,7 +232,8 @@ def ours_backward(d_output, ids, part_pointer, edge_list, degrees, num_parts, pa
     ws = _feature_workspace(workspace, d_output)
     _check(lib.eppgcn_ours_backward(_ptr(out), _ptr(d_output), _ptr(ids), _ptr(part_pointer), _ptr(edge_list),
                                     _ptr(degrees), n, dim, int(num_parts), part_size, layer, blockx, blocky,
-                                    _ptr(ws), 0 if ws is None else ws.numel(), _stream()))
+                                    _ptr(ws), 0 if ws is None else ws.numel(),
+                                    _plan_ptr(plan, int(num_parts)), _stream()))
     return out
 
 
@@ -294,3 +360,11 @@ def set_team_size(lanes: int):
 
 def set_rounds(rounds: int):
     load().eppgcn_set_rounds(int(rounds))
+
+
+def set_plan_shift(shift: int):
+    load().eppgcn_set_plan_shift(int(shift))
+
+
+def set_plan_keep_rows(groups: int):
+    load().eppgcn_set_plan_keep_rows(int(groups))

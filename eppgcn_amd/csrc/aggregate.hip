@@ -31,6 +31,8 @@
 // use float atomics, once per wave instead of once per group.
 // Precondition: the groups of one row are consecutive (build_part and the path
 // splitter produce them that way).
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace eppgcn {
@@ -71,6 +73,14 @@ template <> struct Vec<4> {
 };
 
 // ---------------------------------------------------------------- group sources
+// What the kernel asks about group p (p = position in processing order):
+//   row_of       the row the group adds into
+//   has_prev     the row has groups before this one that this position does not follow
+//   has_next     ... after this one
+//   joins_left   the group continues the group at position p-1 (same row, adjacent)
+//   joins_right  the group at position p+1 continues this one
+// For groups processed in their own order the two pairs coincide.
+
 // Forward groups: (part_ptr, part2node) as build_part produces them.
 struct ForwardGroups {
     const int* part_ptr;
@@ -81,6 +91,8 @@ struct ForwardGroups {
     {
         return p + 1 < num_parts && part2node[p + 1] == row;
     }
+    __device__ bool joins_left(int, bool prev) const { return prev; }
+    __device__ bool joins_right(int, bool next) const { return next; }
 };
 
 // Backward groups over the compacted path: the row of a group is the id of its
@@ -94,6 +106,22 @@ struct CompactedGroups {
     {
         return p + 1 < num_parts && ids[gend] == row;
     }
+    __device__ bool joins_left(int, bool prev) const { return prev; }
+    __device__ bool joins_right(int, bool next) const { return next; }
+};
+
+// Groups of an execution plan: re-ordered copy with precomputed row and adjacency flags
+// (bit0 has_prev, bit1 has_next, bit2 joins_left, bit3 joins_right; all in terms of the
+// original group order, see schedule.hip).
+struct PlanGroups {
+    const int* part_ptr;
+    const int* row;
+    const uint8_t* flags;
+    __device__ int row_of(int p, int) const { return row[p]; }
+    __device__ bool has_prev(int p, int, int) const { return (flags[p] & 1) != 0; }
+    __device__ bool has_next(int p, int, int, int) const { return (flags[p] & 2) != 0; }
+    __device__ bool joins_left(int p, bool) const { return (flags[p] & 4) != 0; }
+    __device__ bool joins_right(int p, bool) const { return (flags[p] & 8) != 0; }
 };
 
 // ---------------------------------------------------------------- pre-scaling pass
@@ -132,17 +160,24 @@ __global__ __launch_bounds__(256) void scale_rows_flat_kernel(float* __restrict_
 // ---------------------------------------------------------------- kernel
 // VW: floats per load of the input (row pitch ld_in, `chunks` vectors per row are read);
 // OVW: floats per store of the output (row pitch ld_out, columns < width_out are written).
+//
 // A wave runs `rounds` rounds; round r covers the TPW consecutive groups starting at
-// (wave * rounds + r) * TPW.  When the last row of a round goes on in the next round of the
-// same wave its partial sum is carried in registers instead of being flushed, so a long row
-// costs one flush per wave, not one per group.
+// (wave * rounds + r) * TPW.  When the last run of a round is continued by the first group of
+// the next round of the same wave its partial sum is carried in registers instead of being
+// flushed, so a long row costs one flush per wave, not one per group.
+//
+// A "run" is a maximal stretch of adjacent teams whose groups continue one another (same row,
+// adjacent in the original group order).  Only such groups are summed across teams, so that
+// has_prev of a run's first group and has_next of its last group tell whether the row has
+// groups the wave does not hold: if not, the run is stored plainly, otherwise added atomically.
 template <int VW, int OVW, int TS, int CPL, int U, bool kPrescaled, class Groups>
 __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
     float* __restrict__ out, const float* __restrict__ in, const int* __restrict__ col,
     const float* __restrict__ scale, Groups groups, int num_parts, int rounds, int chunks, int ld_in, int width_out,
     int ld_out)
 {
-    constexpr int TPW = kWave / TS;      // teams (= groups) per wave and round
+    constexpr int TPW = kWave / TS;                  // teams (= groups) per wave and round
+    constexpr int kPasses = kStageCap / kWave;       // load instructions per staging pass
     using V = Vec<VW>;
     __shared__ int stage_col[kAggWaves][kStageWords];
     __shared__ float stage_scale[kAggWaves][kPrescaled ? 1 : kStageWords];
@@ -155,9 +190,9 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
     float* my_scale = stage_scale[wave];
     const long long wave_first = (static_cast<long long>(blockIdx.x) * kAggWaves + wave) * TPW * rounds;
 
-    V carry[CPL];                // partial sum of the row that continues from the previous round (team 0)
+    V carry[CPL];                // partial sum of the run that continues from the previous round (team 0)
     bool carry_valid = false;    // wave-uniform
-    bool carry_outside = false;  // the carried row started before this wave
+    bool carry_outside = false;  // the carried run's row has groups before the run
     int carry_row = 0;
 #pragma unroll
     for (int k = 0; k < CPL; ++k)
@@ -192,31 +227,31 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
 #pragma unroll
             for (int j = 0; j < VW; ++j) acc[k].v[j] = 0.f;
 
+        // the groups of the round are one contiguous slot range: stage it with coalesced loads
         for (int cb = wbeg; cb < wend; cb += kStageCap) {
             const int cn = min(kStageCap, wend - cb);
-            // stage the pass: coalesced column ids (and, without pre-scaling, one scale gather per slot)
             {
-                int c[kStageCap / kWave];
+                int c[kPasses];
 #pragma unroll
-                for (int r = 0; r < kStageCap / kWave; ++r) {
+                for (int r = 0; r < kPasses; ++r) {
                     const int i = lane + r * kWave;
                     c[r] = i < cn ? col[cb + i] : 0;
                 }
                 if constexpr (!kPrescaled) {
-                    float sc[kStageCap / kWave];
+                    float sc[kPasses];
 #pragma unroll
-                    for (int r = 0; r < kStageCap / kWave; ++r) {
+                    for (int r = 0; r < kPasses; ++r) {
                         const int i = lane + r * kWave;
                         sc[r] = i < cn ? scale[c[r]] : 0.f;
                     }
 #pragma unroll
-                    for (int r = 0; r < kStageCap / kWave; ++r) {
+                    for (int r = 0; r < kPasses; ++r) {
                         const int i = lane + r * kWave;
                         if (i < cn) my_scale[stage_index(i)] = sc[r];
                     }
                 }
 #pragma unroll
-                for (int r = 0; r < kStageCap / kWave; ++r) {
+                for (int r = 0; r < kPasses; ++r) {
                     const int i = lane + r * kWave;
                     if (i < cn) my_col[stage_index(i)] = c[r];
                 }
@@ -234,9 +269,9 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const bool ok = i + u < hi;
-                    const int slot = stage_index(ok ? i + u - cb : 0);
-                    const int c = my_col[slot];
-                    if constexpr (!kPrescaled) w[u] = ok ? s_row * my_scale[slot] : 0.f;
+                    const int word = stage_index(ok ? i + u - cb : 0);
+                    const int c = my_col[word];
+                    if constexpr (!kPrescaled) w[u] = ok ? s_row * my_scale[word] : 0.f;
                     const float* src = in + static_cast<size_t>(c) * ld_in;
 #pragma unroll
                     for (int k = 0; k < CPL; ++k) {
@@ -268,12 +303,14 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
                 for (int j = 0; j < VW; ++j) acc[k].v[j] *= s_row;
         }
 
-        // ---- combine with the carried row, reduce across teams, flush or carry on
+        // ---- combine with the carried run, reduce across teams, flush or carry on
         bool prev = live && groups.has_prev(p, row, gbeg);
         const bool next = live && groups.has_next(p, row, gend, num_parts);
+        const bool joins_left = live && groups.joins_left(p, prev);
+        const bool joins_right = live && groups.joins_right(p, next);
         bool orphan = false;           // a carried sum met an empty group (malformed input): never store plainly
         if (carry_valid && team == 0) {
-            // by construction the first group of this round belongs to the carried row
+            // the first group of this round continues the carried run
             if (!live) { live = true; row = carry_row; orphan = true; }
 #pragma unroll
             for (int k = 0; k < CPL; ++k)
@@ -282,29 +319,33 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
             prev = carry_outside;          // what lies before the carried part, not before this group
         }
         bool head = live;              // this team writes its (possibly combined) sum
-        int more = (next || orphan) ? 1 : 0;   // the run goes on after its last team
+        // flags of the run's last group: bit0 the row has groups after it, bit1 the next group continues it
+        int tail = ((next || orphan) ? 1 : 0) | (joins_right ? 2 : 0);
         if constexpr (TPW > 1) {
-            const int row0 = __shfl(row, 0, kWave);
-            if (np > 1 && __all(!active || (live && row == row0))) {
-                // the whole round is one row: butterfly over the teams with DPP / swizzle
+            // a team starts a run unless it continues its (live) left neighbour
+            const int live_up = __shfl_up(static_cast<int>(live), TS, kWave);
+            const bool starts = !(team > 0 && joins_left && live_up != 0);
+            const uint64_t start_lanes = __ballot(starts && tl == 0 && active);
+            if (np > 1 && start_lanes == 1ull && __all(!active || live)) {
+                // the whole round is one run: butterfly over the teams with DPP / swizzle
 #pragma unroll
                 for (int k = 0; k < CPL; ++k)
 #pragma unroll
                     for (int j = 0; j < VW; ++j) acc[k].v[j] = cross_team_sum<TS>(acc[k].v[j]);
                 head = team == 0;
                 prev = __shfl(static_cast<int>(prev), 0, kWave) != 0;
-                more = __shfl(more, (np - 1) * TS, kWave);
-            } else if (__any(prev || next)) {
-                // several rows: segmented reduction towards the first team of every run of equal
-                // rows; the "goes on" flag of the run's last team travels towards the head with the sums
-                const int key = live ? row : -1 - team;          // dead teams never merge
-                const int key_up = __shfl_up(key, TS, kWave);
+                tail = __shfl(tail, (np - 1) * TS, kWave);
+            } else if (__any(live && !starts)) {
+                // several runs: segmented reduction towards the first team of every run; the flags of
+                // the run's last team travel towards the head with the sums
+                const uint64_t upto = (lane | (TS - 1)) == 63 ? ~0ull : ((2ull << (lane | (TS - 1))) - 1ull);
+                const int key = live ? __popcll(start_lanes & upto) : -1 - team;   // run number, monotone
 #pragma unroll
                 for (int d = 1; d < TPW; d <<= 1) {
                     const int other = __shfl_down(key, d * TS, kWave);
-                    const int other_more = __shfl_down(more, d * TS, kWave);
+                    const int other_tail = __shfl_down(tail, d * TS, kWave);
                     const bool take = team + d < TPW && other == key;
-                    if (take) more = other_more;     // the flag of the furthest team covered so far
+                    if (take) tail = other_tail;
 #pragma unroll
                     for (int k = 0; k < CPL; ++k)
 #pragma unroll
@@ -313,20 +354,18 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
                             if (take) acc[k].v[j] += o;
                         }
                 }
-                head = live && (team == 0 || key_up != key);
+                head = live && starts;
             }
         }
-        // the last run of the round is carried into the next round when it goes on there
+        // the last run of the round is carried into the next round when the next group continues it
         carry_valid = false;
         if (more_rounds) {
             const uint64_t heads = __ballot(head && tl == 0);
-            if (heads) {
+            const int last_team_lane = (np - 1) * TS;
+            if (heads && __shfl(static_cast<int>(live), last_team_lane, kWave) != 0) {
                 const int h = 63 - __builtin_clzll(heads);           // first lane of the last head team
-                const int last_team_lane = (np - 1) * TS;
-                // the run of head h reaches the round's last team iff its row is that team's row
-                const bool reaches_end = __shfl(row, h, kWave) == __shfl(row, last_team_lane, kWave) &&
-                                         __shfl(static_cast<int>(live), last_team_lane, kWave) != 0;
-                if (reaches_end && __shfl(more, h, kWave) != 0) {
+                // runs are contiguous, so the last head's run ends at the round's last team
+                if ((__shfl(tail, h, kWave) & 2) != 0) {
                     carry_valid = true;
                     carry_outside = __shfl(static_cast<int>(prev), h, kWave) != 0;
                     carry_row = __shfl(row, h, kWave);
@@ -339,7 +378,7 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
             }
         }
         if (head) {
-            const bool outside = prev || more != 0;     // the row also has groups this wave does not hold
+            const bool outside = prev || (tail & 1) != 0;   // the row also has groups this wave does not hold
             float* dst = out + static_cast<size_t>(row) * ld_out;
 #pragma unroll
             for (int k = 0; k < CPL; ++k) {
@@ -423,7 +462,7 @@ static hipError_t launch_slab(float* out, const float* in, const int* col, const
     int ts = 4;
     while (ts < 64 && ts < chunks) ts <<= 1;
     const int ft = g_tuning.force_team;
-    if (ft >= 4 && ft <= 64 && (ft & (ft - 1)) == 0 && chunks <= 4 * ft && (ft == 64 || chunks <= 2 * ft)) ts = ft;
+    if (ft >= 4 && ft <= 64 && (ft & (ft - 1)) == 0 && chunks <= ft) ts = ft;   // only wider teams can be forced
     const int cpl = (chunks + ts - 1) / ts;
 #define EPPGCN_LAUNCH(TS_, CPL_, U_) \
     return launch_one<VW, OVW, TS_, CPL_, U_, kPrescaled, Groups>(out, in, col, scale, g, num_parts, sh, stream)
@@ -436,17 +475,21 @@ static hipError_t launch_slab(float* out, const float* in, const int* col, const
             default: EPPGCN_LAUNCH(64, 1, 8);
         }
     } else if (cpl == 2) {
-        switch (ts) {
-            case 4: EPPGCN_LAUNCH(4, 2, 4);
-            case 8: EPPGCN_LAUNCH(8, 2, 4);
-            case 16: EPPGCN_LAUNCH(16, 2, 4);
-            case 32: EPPGCN_LAUNCH(32, 2, 4);
-            default: EPPGCN_LAUNCH(64, 2, 4);
-        }
+        EPPGCN_LAUNCH(64, 2, 4);
     } else {
         EPPGCN_LAUNCH(64, 4, 2);
     }
 #undef EPPGCN_LAUNCH
+}
+
+// Plans are only used with pre-scaled features: the per-edge-scale form is not instantiated for them.
+template <int VW, int OVW, class Groups>
+static hipError_t slab_either(bool prescaled, float* out, const float* in, const int* col, const float* scale,
+                              Groups g, int num_parts, AggShape sh, hipStream_t stream)
+{
+    if (prescaled) return launch_slab<VW, OVW, true>(out, in, col, scale, g, num_parts, sh, stream);
+    if constexpr (std::is_same<Groups, PlanGroups>::value) return hipErrorInvalidValue;
+    else return launch_slab<VW, OVW, false>(out, in, col, scale, g, num_parts, sh, stream);
 }
 
 // Row pitch of the pre-scaled workspace: whole 16-byte vectors for narrow rows, whole 32-byte
@@ -494,10 +537,10 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
                               int num_nodes, int dim, int num_parts, int group_size, float* workspace,
                               hipStream_t stream, double* sink, double* sink2)
 {
-    EPPGCN_HIP(hipMemsetAsync(out, 0, static_cast<size_t>(num_nodes) * dim * sizeof(float), stream));
-    if (num_parts == 0) return kOk;
     const bool prescaled = workspace != nullptr;
     int ld_in = dim;
+    EPPGCN_HIP(hipMemsetAsync(out, 0, static_cast<size_t>(num_nodes) * dim * sizeof(float), stream));
+    if (num_parts == 0) return kOk;
     if (prescaled) {
         ld_in = workspace == in ? dim : workspace_pitch(dim);
         if (int rc = launch_scale_rows(workspace, in, scale, num_nodes, dim, ld_in, stream)) return rc;
@@ -526,9 +569,7 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
         sh.width_out = dim - c0 < slab ? dim - c0 : slab;
         sh.ld_out = dim;
         hipError_t e;
-#define EPPGCN_SLAB(VW_, OVW_)                                                                                 \
-    (prescaled ? launch_slab<VW_, OVW_, true>(out + c0, in + c0, col, scale, g, num_parts, sh, stream)         \
-               : launch_slab<VW_, OVW_, false>(out + c0, in + c0, col, scale, g, num_parts, sh, stream))
+#define EPPGCN_SLAB(VW_, OVW_) slab_either<VW_, OVW_>(prescaled, out + c0, in + c0, col, scale, g, num_parts, sh, stream)
         if (vw == 4 && ovw_eff == 4) e = EPPGCN_SLAB(4, 4);
         else if (vw == 4 && ovw_eff == 2) e = EPPGCN_SLAB(4, 2);
         else if (vw == 4) e = EPPGCN_SLAB(4, 1);
@@ -541,22 +582,33 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
     return kOk;
 }
 
+// plan: nullptr, or an execution plan built for exactly these groups (used with a workspace).
 int aggregate_forward_groups(float* out, const float* in, const int* col, const float* scale,
-                             const int* part_ptr, const int* part2node, int num_nodes, int dim,
+                             const int* part_ptr, const int* part2node, const void* plan, int num_nodes, int dim,
                              int num_parts, int group_size, float* workspace, hipStream_t stream, double* sink,
                              double* sink2)
 {
-    return aggregate_dispatch(out, in, col, scale, ForwardGroups{part_ptr, part2node}, num_nodes, dim,
-                              num_parts, group_size, workspace, stream, sink, sink2);
+    if (plan && workspace && num_parts > 0) {
+        const PlanView v = plan_view(const_cast<void*>(plan), num_parts);
+        return aggregate_dispatch(out, in, v.col, scale, PlanGroups{v.ptr, v.row, v.flags}, num_nodes, dim, num_parts,
+                                  group_size, workspace, stream, sink, sink2);
+    }
+    return aggregate_dispatch(out, in, col, scale, ForwardGroups{part_ptr, part2node}, num_nodes, dim, num_parts,
+                              group_size, workspace, stream, sink, sink2);
 }
 
 int aggregate_compacted_groups(float* out, const float* in, const int* ids, const int* part_ptr,
-                               const int* edge_list, const float* scale, int num_nodes, int dim,
+                               const int* edge_list, const float* scale, const void* plan, int num_nodes, int dim,
                                int num_parts, int group_size, float* workspace, hipStream_t stream, double* sink,
                                double* sink2)
 {
-    return aggregate_dispatch(out, in, edge_list, scale, CompactedGroups{part_ptr, ids}, num_nodes, dim,
-                              num_parts, group_size, workspace, stream, sink, sink2);
+    if (plan && workspace && num_parts > 0) {
+        const PlanView v = plan_view(const_cast<void*>(plan), num_parts);
+        return aggregate_dispatch(out, in, v.col, scale, PlanGroups{v.ptr, v.row, v.flags}, num_nodes, dim, num_parts,
+                                  group_size, workspace, stream, sink, sink2);
+    }
+    return aggregate_dispatch(out, in, edge_list, scale, CompactedGroups{part_ptr, ids}, num_nodes, dim, num_parts,
+                              group_size, workspace, stream, sink, sink2);
 }
 
 }  // namespace eppgcn

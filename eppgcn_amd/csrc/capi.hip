@@ -11,10 +11,16 @@
 namespace eppgcn {
 
 // ---- implemented in aggregate.hip / prepare.hip
-int aggregate_forward_groups(float*, const float*, const int*, const float*, const int*, const int*, int, int, int,
-                             int, float*, hipStream_t, double*, double*);
-int aggregate_compacted_groups(float*, const float*, const int*, const int*, const int*, const float*, int, int, int,
-                               int, float*, hipStream_t, double*, double*);
+int aggregate_forward_groups(float*, const float*, const int*, const float*, const int*, const int*, const void*, int,
+                             int, int, int, float*, hipStream_t, double*, double*);
+int aggregate_compacted_groups(float*, const float*, const int*, const int*, const int*, const float*, const void*,
+                               int, int, int, int, float*, hipStream_t, double*, double*);
+size_t plan_workspace_bytes(long long);
+int schedule_shift(int);
+void set_schedule_shift(int);
+void set_plan_keep_rows(int);
+int launch_build_plan(const int*, const int*, const int*, const int*, int, long long, int, int, void*, size_t, void*,
+                      size_t, hipStream_t);
 void set_agg_force_team(int);
 void set_agg_force_rounds(int);
 size_t feature_workspace_floats(long long, int);
@@ -64,12 +70,12 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 2; }
+int eppgcn_abi_version(void) { return 3; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
                         int dim, int num_parts, int part_size, int dim_worker, int warp_per_block, float* workspace,
-                        size_t workspace_floats, void* stream)
+                        size_t workspace_floats, const void* plan, void* stream)
 {
     (void)row_pointers;
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
@@ -78,18 +84,19 @@ int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers
     EPPGCN_REQUIRE(out && in && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (column_index && part_pointers && part2node), "null index pointer");
     EPPGCN_REQUIRE(aligned(out, 4) && aligned(in, 4), "feature pointers must be 4-byte aligned");
+    EPPGCN_REQUIRE(!plan || aligned(plan, 256), "plan must be 256-byte aligned");
     EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != out),
                    "workspace must be 16-byte aligned and distinct from the output");
     EPPGCN_REQUIRE(!workspace || workspace == in || workspace_floats >= feature_workspace_floats(num_nodes, dim),
                    "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
-    return aggregate_forward_groups(out, in, column_index, degrees, part_pointers, part2node, num_nodes, dim, num_parts,
-                                    part_size, workspace, static_cast<hipStream_t>(stream), &g_for_agg_ms, nullptr);
+    return aggregate_forward_groups(out, in, column_index, degrees, part_pointers, part2node, plan, num_nodes, dim,
+                                    num_parts, part_size, workspace, static_cast<hipStream_t>(stream), &g_for_agg_ms, nullptr);
 }
 
 int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* row_pointers,
                          const int32_t* column_index, const float* degrees, const int32_t* part_pointers,
                          const int32_t* part2node, int num_nodes, int dim, int num_parts, int part_size, int dim_worker,
-                         int warp_per_block, float* workspace, size_t workspace_floats, void* stream)
+                         int warp_per_block, float* workspace, size_t workspace_floats, const void* plan, void* stream)
 {
     (void)row_pointers;
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
@@ -98,18 +105,19 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
     EPPGCN_REQUIRE(d_input && d_output && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (column_index && part_pointers && part2node), "null index pointer");
     EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
+    EPPGCN_REQUIRE(!plan || aligned(plan, 256), "plan must be 256-byte aligned");
     EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != d_input),
                    "workspace must be 16-byte aligned and distinct from the output");
     EPPGCN_REQUIRE(!workspace || workspace == d_output || workspace_floats >= feature_workspace_floats(num_nodes, dim),
                    "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
-    return aggregate_forward_groups(d_input, d_output, column_index, degrees, part_pointers, part2node, num_nodes, dim,
-                                    num_parts, part_size, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms, nullptr);
+    return aggregate_forward_groups(d_input, d_output, column_index, degrees, part_pointers, part2node, plan,
+                                    num_nodes, dim, num_parts, part_size, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms, nullptr);
 }
 
 int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
                          const int32_t* edge_list, const float* degrees, int num_nodes, int dim, int num_parts,
                          int part_size, int layer, int blockx, int blocky, float* workspace,
-                         size_t workspace_floats, void* stream)
+                         size_t workspace_floats, const void* plan, void* stream)
 {
     // part_size only sizes the work per wave (the reference's kernel ignores it, EPPGCN_kernel.cu:636)
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
@@ -119,12 +127,13 @@ int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* i
     EPPGCN_REQUIRE(d_input && d_output && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (ids && part_pointer && edge_list), "null index pointer");
     EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
+    EPPGCN_REQUIRE(!plan || aligned(plan, 256), "plan must be 256-byte aligned");
     EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != d_input),
                    "workspace must be 16-byte aligned and distinct from the output");
     EPPGCN_REQUIRE(!workspace || workspace == d_output || workspace_floats >= feature_workspace_floats(num_nodes, dim),
                    "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
-    return aggregate_compacted_groups(d_input, d_output, ids, part_pointer, edge_list, degrees, num_nodes, dim,
-                                      num_parts, part_size > 0 ? part_size : 1, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms,
+    return aggregate_compacted_groups(d_input, d_output, ids, part_pointer, edge_list, degrees, plan, num_nodes,
+                                      dim, num_parts, part_size > 0 ? part_size : 1, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms,
                                       layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr);
 }
 
@@ -147,6 +156,23 @@ size_t eppgcn_feature_workspace_floats(int64_t num_nodes, int dim)
 {
     return (num_nodes <= 0 || dim <= 0) ? 0 : feature_workspace_floats(num_nodes, dim);
 }
+size_t eppgcn_plan_bytes(int64_t num_parts, int64_t num_slots) { return plan_bytes(num_parts, num_slots); }
+size_t eppgcn_plan_workspace_bytes(int64_t num_parts) { return plan_workspace_bytes(num_parts); }
+
+int eppgcn_build_plan(const int32_t* part_pointers, const int32_t* column_index, const int32_t* part2node,
+                      const int32_t* ids, int num_parts, int64_t num_slots, int num_nodes, int dim, void* plan,
+                      size_t plan_size, void* workspace, size_t workspace_bytes, void* stream)
+{
+    EPPGCN_REQUIRE(num_parts >= 0 && num_slots >= 0 && num_nodes >= 0 && dim > 0, "negative size");
+    if (num_parts == 0) return kOk;
+    EPPGCN_REQUIRE(part_pointers && column_index && plan, "null pointer");
+    EPPGCN_REQUIRE((part2node != nullptr) != (ids != nullptr), "give exactly one of part2node (forward) and ids (backward)");
+    EPPGCN_REQUIRE(aligned(plan, 256) && workspace && aligned(workspace, 256), "plan and workspace must be 256-byte aligned");
+    return launch_build_plan(part_pointers, column_index, part2node, ids, num_parts, num_slots, num_nodes,
+                             schedule_shift(dim), plan, plan_size, workspace, workspace_bytes,
+                             static_cast<hipStream_t>(stream));
+}
+
 size_t eppgcn_compact_workspace_bytes(int64_t length) { return compact_workspace_bytes(length < 0 ? 0 : length); }
 size_t eppgcn_split_workspace_bytes(int64_t num_nodes) { return split_workspace_bytes(num_nodes < 0 ? 0 : num_nodes); }
 
@@ -317,5 +343,7 @@ double eppgcn_get_time_ms(int which)
 
 void eppgcn_set_team_size(int lanes) { set_agg_force_team(lanes); }
 void eppgcn_set_rounds(int rounds) { set_agg_force_rounds(rounds); }
+void eppgcn_set_plan_shift(int shift) { set_schedule_shift(shift); }
+void eppgcn_set_plan_keep_rows(int groups) { set_plan_keep_rows(groups); }
 
 }  // extern "C"

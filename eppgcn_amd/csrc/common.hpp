@@ -40,6 +40,34 @@ int hip_fail(hipError_t e, const char* what);
         }                                                       \
     } while (0)
 
+// ---------------------------------------------------------------- execution plan layout
+// One caller-owned buffer: ptr[P+1] | row[P] | flags[P] | col[S], each part 256-byte aligned
+// (contents described in schedule.hip).  Offsets depend on the group count alone.
+struct PlanView {
+    int* ptr;
+    int* row;
+    uint8_t* flags;
+    int* col;
+};
+inline size_t plan_align(size_t x) { return (x + 255) / 256 * 256; }
+inline size_t plan_bytes(long long num_parts, long long num_slots)
+{
+    const size_t p = static_cast<size_t>(num_parts > 0 ? num_parts : 0);
+    const size_t s = static_cast<size_t>(num_slots > 0 ? num_slots : 0);
+    return plan_align(4 * (p + 1)) + plan_align(4 * p) + plan_align(p) + plan_align(4 * s);
+}
+inline PlanView plan_view(void* plan, long long num_parts)
+{
+    const size_t p = static_cast<size_t>(num_parts);
+    char* b = static_cast<char*>(plan);
+    PlanView v;
+    v.ptr = reinterpret_cast<int*>(b);
+    v.row = reinterpret_cast<int*>(b + plan_align(4 * (p + 1)));
+    v.flags = reinterpret_cast<uint8_t*>(b + plan_align(4 * (p + 1)) + plan_align(4 * p));
+    v.col = reinterpret_cast<int*>(b + plan_align(4 * (p + 1)) + plan_align(4 * p) + plan_align(p));
+    return v;
+}
+
 // ---------------------------------------------------------------- kernel timers
 // Optional event timing of the kernels of one call (off by default: calls stay
 // asynchronous).  When enabled the destructor synchronises on the stop event and

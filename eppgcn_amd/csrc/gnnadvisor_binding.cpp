@@ -14,11 +14,15 @@
 //     exact for any edge count;
 //   - split_back_part's part_pointer has num_edges + 1 entries, so the terminator
 //     is always in bounds;
-//   - get_map_back_part_size never returns less than 1.
+//   - get_map_back_part_size never returns less than 1;
+//   - the module keeps, per group array it has seen, a column-blocked execution plan for the
+//     aggregation kernels (built on first use, about 4 bytes per edge, the 8 most recently used
+//     kept); it affects speed only.
 #include <torch/extension.h>
 
 #include <c10/hip/HIPStream.h>
 
+#include <list>
 #include <vector>
 
 #include "eppgcn_hip.h"
@@ -60,6 +64,95 @@ Tensor workspace(size_t bytes, const Tensor& like)
     return torch::empty({static_cast<int64_t>((bytes + 7) / 8)}, like.options().dtype(torch::kInt64));
 }
 
+// ---------------------------------------------------------------- plan cache
+// The column-blocked execution plan depends only on the groups and the column ids, which a
+// training run passes unchanged every epoch.  Entries are keyed by storage address, length,
+// tensor version and block-size class, and hold references to the key tensors so that an
+// address cannot be reused for other data while its entry lives.
+struct PlanEntry {
+    const void* part_ptr;
+    const void* col;
+    const void* rows;
+    int64_t num_parts;
+    int64_t version_part, version_col, version_rows;
+    int dim_class;
+    Tensor keep_part, keep_col, keep_rows, plan;
+    const void* plan_ptr;
+};
+std::list<PlanEntry> g_plans;
+constexpr size_t kMaxPlans = 8;
+
+int dim_class_of(int dim) { return dim <= 32 ? 0 : dim <= 128 ? 1 : 2; }
+int dim_of_class(int c) { return c == 0 ? 32 : c == 1 ? 128 : 256; }
+
+Tensor aligned_bytes(size_t bytes, const Tensor& like, void** base)
+{
+    auto t = torch::empty({static_cast<int64_t>(bytes + 256)}, like.options().dtype(torch::kUInt8));
+    *base = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(t.data_ptr()) + 255) / 256 * 256);
+    return t;
+}
+
+// rows: part2Node (forward groups, is_forward) or the per-edge id list (backward path);
+// num_slots < 0: read it from part_ptr[num_parts] when the plan has to be built
+const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& rows, bool is_forward, int64_t num_parts,
+                     int64_t num_slots, int num_nodes, int dim)
+{
+    if (num_parts <= 0) return nullptr;
+    const int dc = dim_class_of(dim);
+    for (auto it = g_plans.begin(); it != g_plans.end(); ++it) {
+        if (it->part_ptr == part_ptr.data_ptr() && it->col == col.data_ptr() && it->rows == rows.data_ptr() &&
+            it->num_parts == num_parts && it->dim_class == dc &&
+            it->version_part == static_cast<int64_t>(part_ptr._version()) &&
+            it->version_col == static_cast<int64_t>(col._version()) &&
+            it->version_rows == static_cast<int64_t>(rows._version())) {
+            g_plans.splice(g_plans.begin(), g_plans, it);   // most recently used first
+            return g_plans.front().plan_ptr;
+        }
+    }
+    if (num_slots < 0) num_slots = part_ptr[num_parts].item<int64_t>();   // slots the groups cover (one 4-byte read)
+    PlanEntry e{part_ptr.data_ptr(), col.data_ptr(), rows.data_ptr(), num_parts,
+                static_cast<int64_t>(part_ptr._version()), static_cast<int64_t>(col._version()),
+                static_cast<int64_t>(rows._version()), dc, part_ptr, col, rows, Tensor(), nullptr};
+    const size_t bytes = eppgcn_plan_bytes(num_parts, num_slots);
+    void* base = nullptr;
+    e.plan = aligned_bytes(bytes, part_ptr, &base);
+    e.plan_ptr = base;
+    const size_t wbytes = eppgcn_plan_workspace_bytes(num_parts);
+    void* wbase = nullptr;
+    auto ws = aligned_bytes(wbytes, part_ptr, &wbase);
+    check(eppgcn_build_plan(part_ptr.data_ptr<int32_t>(), col.data_ptr<int32_t>(),
+                            is_forward ? rows.data_ptr<int32_t>() : nullptr,
+                            is_forward ? nullptr : rows.data_ptr<int32_t>(), static_cast<int>(num_parts), num_slots,
+                            num_nodes, dim_of_class(dc), base, bytes, wbase, wbytes, stream_of(part_ptr)),
+          "build_plan");
+    g_plans.push_front(std::move(e));
+    if (g_plans.size() > kMaxPlans) g_plans.pop_back();
+    return g_plans.front().plan_ptr;
+}
+
+// A heavily pruned path gathers from few distinct rows, which stay cached without a plan: plans are
+// built for paths that keep at least half of the edges.  The decision is remembered per path.
+struct PathChoice {
+    const void* part_ptr;
+    int64_t num_parts;
+    bool use_plan;
+};
+std::vector<PathChoice> g_path_choices;
+
+const void* backward_plan(const Tensor& part_pointer, const Tensor& edge_list, const Tensor& ids, int64_t num_parts,
+                          int num_nodes, int dim)
+{
+    if (num_parts <= 0) return nullptr;
+    for (const auto& c : g_path_choices)
+        if (c.part_ptr == part_pointer.data_ptr() && c.num_parts == num_parts)
+            return c.use_plan ? plan_for(part_pointer, edge_list, ids, false, num_parts, -1, num_nodes, dim) : nullptr;
+    const int64_t valid_len = part_pointer[num_parts].item<int64_t>();
+    const bool use = 2 * valid_len >= edge_list.numel();
+    if (g_path_choices.size() >= 64) g_path_choices.erase(g_path_choices.begin());
+    g_path_choices.push_back({part_pointer.data_ptr(), num_parts, use});
+    return use ? plan_for(part_pointer, edge_list, ids, false, num_parts, valid_len, num_nodes, dim) : nullptr;
+}
+
 Tensor feature_scratch(const Tensor& feats)
 {
     const size_t n = eppgcn_feature_workspace_floats(feats.size(0), static_cast<int>(feats.size(1)));
@@ -85,7 +178,11 @@ std::vector<Tensor> forward(Tensor input, Tensor weight, Tensor row_pointers, Te
     check(eppgcn_spmm_forward(output.data_ptr<float>(), tmp.data_ptr<float>(), i32(row_pointers), i32(column_index),
                               f32(degrees), i32(part_pointers), i32(part2Node), static_cast<int>(tmp.size(0)),
                               static_cast<int>(tmp.size(1)), static_cast<int>(part2Node.numel()), partSize, dimWorker,
-                              warpPerBlock, scaled.data_ptr<float>(), ws_floats, stream_of(input)),
+                              warpPerBlock, scaled.data_ptr<float>(), ws_floats,
+                              plan_for(part_pointers, column_index, part2Node, true, part2Node.numel(),
+                                       column_index.numel(), static_cast<int>(tmp.size(0)),
+                                       static_cast<int>(tmp.size(1))),
+                              stream_of(input)),
           "forward");
     return {output};
 }
@@ -104,7 +201,11 @@ std::vector<Tensor> backward(Tensor d_output, Tensor X, Tensor W, Tensor row_poi
                                i32(column_index), f32(degrees), i32(part_pointers), i32(part2Node),
                                static_cast<int>(d_output.size(0)), static_cast<int>(d_output.size(1)),
                                static_cast<int>(part2Node.numel()), partSize, dimWorker, warpPerBlock,
-                               scaled.data_ptr<float>(), static_cast<size_t>(scaled.numel()), stream_of(d_output)),
+                               scaled.data_ptr<float>(), static_cast<size_t>(scaled.numel()),
+                               plan_for(part_pointers, column_index, part2Node, true, part2Node.numel(),
+                                        column_index.numel(), static_cast<int>(d_output.size(0)),
+                                        static_cast<int>(d_output.size(1))),
+                               stream_of(d_output)),
           "backward");
     auto d_input = torch::mm(d_input_prime, W.transpose(0, 1));
     auto d_weight = torch::mm(X.transpose(0, 1), d_input_prime);
@@ -144,6 +245,8 @@ std::vector<Tensor> ours_backward(Tensor d_output, Tensor X, Tensor W, Tensor id
                                i32(edgeList), f32(degrees), static_cast<int>(d_output.size(0)),
                                static_cast<int>(d_output.size(1)), numParts, partSize > 0 ? partSize : 1, layer, blockx,
                                blocky, scaled.data_ptr<float>(), static_cast<size_t>(scaled.numel()),
+                               backward_plan(partPointer, edgeList, id, numParts, static_cast<int>(d_output.size(0)),
+                                             static_cast<int>(d_output.size(1))),
                                stream_of(d_output)),
           "ours_backward");
     auto d_input = torch::mm(d_input_prime, W.transpose(0, 1));
@@ -289,6 +392,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("clear_time", &eppgcn_clear_time, "reset accumulated kernel times");
     m.def("set_timing", [](bool on) { eppgcn_set_timing(on ? 1 : 0); }, "enable per-call kernel timing");
     m.def("get_time_ms", &eppgcn_get_time_ms, "accumulated kernel time in ms");
+    m.def("clear_plans", []() { g_plans.clear(); }, "drop the cached execution plans");
 
     m.def("build_part", &build_part, "forward neighbour groups (HIP)");
     m.def("build_back_part", &build_back_part, "compaction + group split in one call (HIP)");

@@ -27,6 +27,7 @@ class BackwardPath:
     num_parts: int
     valid_len: int
     valid_node: int
+    plan: object = None      # column-blocked execution plan of this path (speed only)
 
 
 @dataclasses.dataclass
@@ -38,6 +39,7 @@ class Workload:
     train_mask: torch.Tensor
     ngh_masks: List[torch.Tensor]
     paths: List[BackwardPath]     # paths[k] belongs to conv layer k (0-based), as edge_masks[k] does
+    plans: dict = None            # feature width -> execution plan of the forward groups
 
     @property
     def num_parts(self) -> int:
@@ -58,7 +60,7 @@ def choose_back_part_size(mode: str, constant: int, valid_node: int, valid_len: 
 
 def prepare(graph: graphs.Graph, num_layers: int = 2, train_ratio: float = 0.1, mask_seed: int = 2,
             part_size: int = None, backsize_mode: str = "constant", backsize: int = 32,
-            train_mask: torch.Tensor = None) -> Workload:
+            train_mask: torch.Tensor = None, widths=(16, 22), plan: bool = True) -> Workload:
     g = graph
     dev = g.column_index.device
     n, e = g.num_nodes, g.num_edges
@@ -89,9 +91,18 @@ def prepare(graph: graphs.Graph, num_layers: int = 2, train_ratio: float = 0.1, 
         bps = choose_back_part_size(backsize_mode, backsize, valid_node, valid_len)
         part_pointer, num_parts, v2 = capi.split_back_part(node_degs[k], e, bps)
         assert v2 == valid_len
+        width = widths[min(k, len(widths) - 1)]
+        # a heavily pruned path gathers from few distinct rows, which stay cached without a plan
+        path_plan = (capi.build_plan(part_pointer, edge_list, num_parts, valid_len, n, width, ids=ids)
+                     if plan and num_parts > 0 and 2 * valid_len >= e else None)
         paths.append(BackwardPath(k + 1, ids, edge_list, part_pointer, node_degs[k], bps, num_parts,
-                                  valid_len, valid_node))
-    return Workload(g, ps, part_ptr, part2node, train_mask, ngh_masks, paths)
+                                  valid_len, valid_node, path_plan))
+    # one plan of the forward groups serves every width (the column block is sized for the widest)
+    plans = {}
+    if plan and part2node.numel() > 0:
+        shared = capi.build_plan(part_ptr, g.column_index, part2node.numel(), e, n, max(widths), part2node=part2node)
+        plans = {w: shared for w in set(widths)}
+    return Workload(g, ps, part_ptr, part2node, train_mask, ngh_masks, paths, plans)
 
 
 # ------------------------------------------------------------------ algorithmic bytes (4-byte elements)

@@ -60,6 +60,24 @@ int eppgcn_abi_version(void);
 /* Floats a separate feature workspace must hold for [num_nodes, dim] features. */
 size_t eppgcn_feature_workspace_floats(int64_t num_nodes, int dim);
 
+/* Execution plan for the aggregation kernels: a copy of the groups (pointers, rows, adjacency
+ * flags, column ids) re-ordered by the column block (2^shift vertices, shift chosen from `dim`;
+ * pass the widest feature width the plan will be used with) of each group's first slot, original
+ * order inside a block.  The aggregation functions accept it as an optional argument (NULL = the
+ * groups as given): it changes no result, only which groups run together, so that the rows
+ * gathered at any moment come from one window of the table and are served from L2.  It is used
+ * when a feature workspace is given as well.  Build it once per graph and group array:
+ *   forward groups : part_pointers + column_index + part2node (ids = NULL)
+ *   backward path  : part_pointer + edge_list + ids (part2node = NULL)
+ * num_slots = number of slots the groups cover (num_edges, or the kept length).  The plan must
+ * be rebuilt when the groups change.  No counterpart in the reference. */
+size_t eppgcn_plan_bytes(int64_t num_parts, int64_t num_slots);
+size_t eppgcn_plan_workspace_bytes(int64_t num_parts);
+int eppgcn_build_plan(const int32_t* part_pointers, const int32_t* column_index,
+                      const int32_t* part2node, const int32_t* ids, int num_parts, int64_t num_slots,
+                      int num_nodes, int dim, void* plan, size_t plan_bytes,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
 /* Forward neighbour-group aggregation:
  *   out[r,:] = sum_{e in groups of r} fl32(degrees[r]*degrees[col[e]]) * in[col[e],:]
  * `out` ([num_nodes, dim]) is fully overwritten (rows without groups become 0).
@@ -73,7 +91,7 @@ int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers
                         const int32_t* part_pointers, const int32_t* part2node,
                         int num_nodes, int dim, int num_parts,
                         int part_size, int dim_worker, int warp_per_block,
-                        float* workspace, size_t workspace_floats, void* stream);
+                        float* workspace, size_t workspace_floats, const void* plan, void* stream);
 
 /* Unpruned backward aggregation: the same operator applied to d_output (valid
  * because the normalised adjacency is symmetric).  Stands in for
@@ -84,7 +102,7 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
                          const int32_t* part_pointers, const int32_t* part2node,
                          int num_nodes, int dim, int num_parts,
                          int part_size, int dim_worker, int warp_per_block,
-                         float* workspace, size_t workspace_floats, void* stream);
+                         float* workspace, size_t workspace_floats, const void* plan, void* stream);
 
 /* Pruned backward aggregation over the compacted execution path:
  *   d_input[id_p,:] += sum_{k in group p} fl32(degrees[id_p]*degrees[edge_list[k]]) * d_output[edge_list[k],:]
@@ -96,7 +114,7 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
 int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids,
                          const int32_t* part_pointer, const int32_t* edge_list, const float* degrees,
                          int num_nodes, int dim, int num_parts, int part_size, int layer,
-                         int blockx, int blocky, float* workspace, size_t workspace_floats, void* stream);
+                         int blockx, int blocky, float* workspace, size_t workspace_floats, const void* plan, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Execution-path preparation.
@@ -189,6 +207,11 @@ void eppgcn_set_team_size(int lanes);
 /* Forces the number of consecutive group rounds one wave processes (0 = choose from
  * the group size so that a wave gathers about 512 rows).  For tuning runs. */
 void eppgcn_set_rounds(int rounds);
+/* Forces the column block size of eppgcn_build_plan to 2^shift vertices (0 = choose from the
+ * feature width).  For tuning runs. */
+void eppgcn_set_plan_shift(int shift);
+/* Rows with at most this many groups stay together in a plan (default 8; 0 = block every group). */
+void eppgcn_set_plan_keep_rows(int groups);
 
 #ifdef __cplusplus
 }

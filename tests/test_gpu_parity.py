@@ -238,6 +238,99 @@ def test_forward_and_pruned_forced_rounds_exact_integer_sums(api, rounds, dim):
         api.set_rounds(0)
 
 
+@pytest.mark.parametrize("name", ["tiny", "small", "isolated", "hub", "medium"])
+@pytest.mark.parametrize("ps", [1, 5, 32])
+def test_plan_is_a_stable_column_block_reordering(api, name, ps):
+    """The execution plan must hold every group exactly once, ordered by the column block of its
+    first slot with the original order kept inside a block, with rows, column ids and adjacency
+    flags that describe the original groups."""
+    indptr, col = GRAPHS[name]()
+    n = indptr.size - 1
+    pp, p2n = co.build_part(ps, indptr)
+    P = p2n.size
+    for dim in (16, 256):
+        plan = api.build_plan(dev(pp), dev(col), P, col.size, n, dim, part2node=dev(p2n))
+        ptr, row, flags, pcol = [t.cpu().numpy() for t in plan.view()]
+        assert ptr[0] == 0 and ptr[-1] == col.size and np.all(np.diff(ptr) >= 1)
+        # identify every plan entry with its original group: same row, same size, same columns;
+        # the first column and the row identify a group uniquely
+        first = {(int(p2n[p]), int(col[pp[p]])): p for p in range(P)}
+        order = np.array([first[(int(row[q]), int(pcol[ptr[q]]))] for q in range(P)])
+        assert np.array_equal(np.sort(order), np.arange(P))
+        for q in (0, P // 3, P // 2, P - 1):
+            p = order[q]
+            assert np.array_equal(pcol[ptr[q]:ptr[q + 1]], col[pp[p]:pp[p + 1]])
+        sizes = np.diff(pp)[order]
+        assert np.array_equal(np.diff(ptr), sizes)
+        first_col = col[pp[:-1]][order]
+        ok = False
+        for shift in range(8, 14):
+            blocks = first_col >> shift
+            if np.all(np.diff(blocks) >= 0) and np.all((np.diff(blocks) > 0) | (np.diff(order) > 0)):
+                ok = True
+        assert ok, "not ordered by a power-of-two column block with stable ties"
+        prev = np.concatenate([[False], p2n[1:] == p2n[:-1]])[order]
+        nxt = np.concatenate([p2n[1:] == p2n[:-1], [False]])[order]
+        jl = prev & np.concatenate([[False], order[1:] == order[:-1] + 1])
+        jr = nxt & np.concatenate([order[1:] == order[:-1] + 1, [False]])
+        assert np.array_equal(flags & 1, prev) and np.array_equal((flags >> 1) & 1, nxt)
+        assert np.array_equal((flags >> 2) & 1, jl) and np.array_equal((flags >> 3) & 1, jr)
+
+
+@pytest.mark.parametrize("rounds", [0, 1, 3])
+@pytest.mark.parametrize("dim", [16, 22, 64, 256])
+@pytest.mark.parametrize("shift", [0, 3, 20])
+def test_planned_aggregation_exact_integer_sums(api, rounds, dim, shift):
+    """A plan only changes which groups run together.  With s == 1 and small integer features the
+    result must be exactly the neighbour sums, for tiny column blocks (every group alone in its
+    block order), the default, and one block (the original order)."""
+    indptr, col = hub_csr(3000, 2500, 23)
+    n = indptr.size - 1
+    x = np.random.default_rng(dim).integers(-8, 9, (n, dim)).astype(np.float32)
+    s = np.ones(n, np.float32)
+    want = np.zeros((n, dim), np.float64)
+    np.add.at(want, cf.row_index(indptr), x[col].astype(np.float64))
+    src = np.random.default_rng(5).random(n) < 0.4
+    keep = src[col]
+    want_b = np.zeros((n, dim), np.float64)
+    np.add.at(want_b, cf.row_index(indptr)[keep], (x * src[:, None])[col[keep]].astype(np.float64))
+    try:
+        api.set_rounds(rounds)
+        api.set_plan_shift(shift)
+        for ps in (1, 3, 32):
+            pp, p2n = co.build_part(ps, indptr)
+            dpp, dcol, dp2n = dev(pp), dev(col), dev(p2n)
+            plan = api.build_plan(dpp, dcol, p2n.size, col.size, n, dim, part2node=dp2n)
+            got = api.spmm_forward(dev(x), dcol, dev(s), dpp, dp2n, part_size=ps, plan=plan)
+            assert np.array_equal(got.cpu().numpy().astype(np.float64), want), f"forward ps={ps}"
+            oid, oedge, bpp, p = _gpu_path(api, indptr, col, src, 5, ps)
+            if p == 0:
+                continue
+            bplan = api.build_plan(bpp, oedge, p, int(keep.sum()), n, dim, ids=oid)
+            dy = dev((x * src[:, None]).astype(np.float32))
+            gb = api.ours_backward(dy, oid, bpp, oedge, dev(s), p, part_size=ps, plan=bplan)
+            assert np.array_equal(gb.cpu().numpy().astype(np.float64), want_b), f"pruned ps={ps}"
+    finally:
+        api.set_rounds(0)
+        api.set_plan_shift(0)
+
+
+@pytest.mark.parametrize("name", ["isolated", "hub", "medium"])
+@pytest.mark.parametrize("dim", [16, 22, 100])
+def test_planned_aggregation_within_tolerance(api, name, dim):
+    indptr, col = GRAPHS[name]()
+    n = indptr.size - 1
+    x = np.random.default_rng(dim).standard_normal((n, dim)).astype(np.float32)
+    s = scale_inv_sqrt(indptr)
+    want = co.spmm_f64(x, indptr, col, s)
+    bound = cf.abs_sum_bound(indptr, col, s, x)
+    for ps in (4, 32):
+        pp, p2n = co.build_part(ps, indptr)
+        plan = api.build_plan(dev(pp), dev(col), p2n.size, col.size, n, dim, part2node=dev(p2n))
+        got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp), dev(p2n), part_size=ps, plan=plan)
+        assert_close(got.cpu().numpy(), want, bound, f"{name} D={dim} ps={ps} planned")
+
+
 def test_forward_unit_scale_integer_features_bit_exact(api):
     """With s == 1 and small integer features every partial sum is exact in fp32, so any
     grouping, lane mapping or atomic order must give exactly the neighbour sum."""
@@ -355,6 +448,9 @@ def test_rmat20_exact_integer_sums_and_path_invariants(api, rmat20):
     got = api.spmm_forward(xi.float(), g.column_index, ones, pp, p2n, part_size=ps)
     want = torch.zeros(n, 16, dtype=torch.int64, device="cuda").index_add_(0, row, xi[g.column_index.long()])
     assert torch.equal(got.long(), want)
+    plan = api.build_plan(pp, g.column_index, p2n.numel(), e, n, 16, part2node=p2n)
+    got_p = api.spmm_forward(xi.float(), g.column_index, ones, pp, p2n, part_size=ps, plan=plan)
+    assert torch.equal(got_p.long(), want)
 
     train = graphs.bernoulli_mask(n, 0.1, 2, "cuda")
     bem = torch.full((e,), -1, dtype=torch.int32, device="cuda")
