@@ -171,7 +171,7 @@ def main():
     dominant = max(per_kernel, key=lambda k: per_kernel[k]["ms"])
     dk = per_kernel[dominant]
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": dk["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": round(dk["GBps"] / PEAK_HBM_GBS, 4), "traffic": None,
+                "frac": round(dk["GBps"] / PEAK_HBM_GBS, 4), "traffic": measured_traffic(args.config, dominant),
                 "kernel_ms": dk["ms"], "alg_bytes_per_launch": dk["alg_bytes"]}
 
     result = {
@@ -208,6 +208,19 @@ def main():
             except Exception as exc:
                 result["cpu_torch_sparse"] = {"error": repr(exc)}
     print(json.dumps(result), flush=True)
+
+
+def measured_traffic(config, kernel):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 counter summary (FETCH_SIZE +
+    WRITE_SIZE of the same bench command), or None when no summary covers this workload."""
+    import glob
+    import re
+    for path in glob.glob(os.path.join(ROOT, "profiles", "*.md")):
+        m = re.search(r"traffic_bytes %s %s = ([0-9.e+]+)" % (re.escape(config), re.escape(kernel)),
+                      open(path).read())
+        if m:
+            return float(m.group(1))
+    return None
 
 
 def cpu_baseline(args, g, wl, x16, x22, dy22, dy16, bytes_epoch):

@@ -262,10 +262,14 @@ def test_plan_is_a_stable_column_block_reordering(api, name, ps):
             assert np.array_equal(pcol[ptr[q]:ptr[q + 1]], col[pp[p]:pp[p + 1]])
         sizes = np.diff(pp)[order]
         assert np.array_equal(np.diff(ptr), sizes)
-        first_col = col[pp[:-1]][order]
+        # sort key: column block of the group's first slot; rows with at most 8 groups use the key
+        # of their first group so that they stay together
+        groups_per_row = np.bincount(p2n, minlength=n)
+        row_first_group = np.concatenate([[0], np.cumsum(groups_per_row)[:-1]])
+        key_col = np.where(groups_per_row[p2n] <= 8, col[pp[row_first_group[p2n]]], col[pp[:-1]])[order]
         ok = False
-        for shift in range(8, 14):
-            blocks = first_col >> shift
+        for shift in range(8, 17):
+            blocks = key_col >> shift
             if np.all(np.diff(blocks) >= 0) and np.all((np.diff(blocks) > 0) | (np.diff(order) > 0)):
                 ok = True
         assert ok, "not ordered by a power-of-two column block with stable ties"
