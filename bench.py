@@ -41,6 +41,7 @@ def parse():
     ap.add_argument("--rounds", type=int, default=0, help="force group rounds per wave (0 = automatic)")
     ap.add_argument("--plan_shift", type=int, default=0, help="force log2 of the plan's column block")
     ap.add_argument("--plan_keep", type=int, default=-1, help="rows with at most this many groups stay together")
+    ap.add_argument("--force_plan", action="store_true", help="use execution plans even for small feature tables")
     ap.add_argument("--no_plan", action="store_true",
                     help="process the groups in CSR order instead of the column-blocked execution plan")
     ap.add_argument("--no_workspace", action="store_true",
@@ -85,7 +86,7 @@ def main():
         capi.set_plan_keep_rows(args.plan_keep)
     t0 = time.perf_counter()
     wl = workload.prepare(g, 2, args.train_ratio, 2, args.part_size or None, args.backsize_mode, args.backsize,
-                          plan=not (args.no_plan or args.no_workspace))
+                          plan=False if (args.no_plan or args.no_workspace) else (True if args.force_plan else None))
     torch.cuda.synchronize()
     prep_s = time.perf_counter() - t0
     n, e = g.num_nodes, g.num_edges
@@ -185,7 +186,7 @@ def main():
                    "kept_edges": [p.valid_len for p in wl.paths],
                    "backward_groups": [p.num_parts for p in wl.paths], "max_degree": g.stats()["max_degree"],
                    "feature_workspace": not args.no_workspace,
-                   "column_blocked_plan": not (args.no_plan or args.no_workspace)},
+                   "column_blocked_plan": bool(wl.plans)},
         "agg_ms_per_epoch": round(ms_per_step, 4), "alg_bytes_per_epoch": bytes_epoch,
         "pct_of_peak_hbm": round(value / PEAK_HBM_GBS * 100, 2),
         "per_kernel": per_kernel, "path_preparation_s": round(prep_s, 3),

@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("EPPGCN_HIP_LIB") or os.path.join(_HERE, "lib", "libeppgcn_hip.so")
 
 EXPORTS = [
-    "eppgcn_last_error", "eppgcn_abi_version", "eppgcn_feature_workspace_floats", "eppgcn_plan_bytes",
+    "eppgcn_last_error", "eppgcn_abi_version", "eppgcn_feature_workspace_floats", "eppgcn_plan_recommended", "eppgcn_plan_bytes",
     "eppgcn_plan_workspace_bytes", "eppgcn_build_plan", "eppgcn_spmm_forward", "eppgcn_spmm_backward",
     "eppgcn_ours_backward", "eppgcn_mask_forward", "eppgcn_compact_workspace_bytes",
     "eppgcn_split_workspace_bytes", "eppgcn_compact_back_edge", "eppgcn_count_nonzero",
@@ -45,6 +45,8 @@ def load():
     lib.eppgcn_abi_version.restype = i
     lib.eppgcn_feature_workspace_floats.argtypes = [i64, i]
     lib.eppgcn_feature_workspace_floats.restype = sz
+    lib.eppgcn_plan_recommended.argtypes = [i64, i]
+    lib.eppgcn_plan_recommended.restype = i
     lib.eppgcn_plan_bytes.argtypes = [i64, i64]
     lib.eppgcn_plan_bytes.restype = sz
     lib.eppgcn_plan_workspace_bytes.argtypes = [i64]
@@ -184,6 +186,11 @@ def build_plan(part_ptr, column_index, num_parts: int, num_slots: int, num_nodes
                                  C.c_void_p(wbase), wbytes, _stream()))
     torch.cuda.current_stream().synchronize()      # the workspace is released on return
     return Plan(buf, base, int(num_parts), int(num_slots))
+
+
+def plan_recommended(num_nodes: int, dim: int) -> bool:
+    """True when the feature table is too large to stay cached by itself, so a plan pays off."""
+    return bool(load().eppgcn_plan_recommended(int(num_nodes), int(dim)))
 
 
 def _plan_ptr(plan, num_parts):

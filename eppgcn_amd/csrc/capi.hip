@@ -156,6 +156,11 @@ size_t eppgcn_feature_workspace_floats(int64_t num_nodes, int dim)
 {
     return (num_nodes <= 0 || dim <= 0) ? 0 : feature_workspace_floats(num_nodes, dim);
 }
+int eppgcn_plan_recommended(int64_t num_nodes, int dim)
+{
+    if (num_nodes <= 0 || dim <= 0) return 0;
+    return static_cast<double>(feature_workspace_floats(num_nodes, dim)) * 4.0 >= 192.0 * (1 << 20) ? 1 : 0;
+}
 size_t eppgcn_plan_bytes(int64_t num_parts, int64_t num_slots) { return plan_bytes(num_parts, num_slots); }
 size_t eppgcn_plan_workspace_bytes(int64_t num_parts) { return plan_workspace_bytes(num_parts); }
 

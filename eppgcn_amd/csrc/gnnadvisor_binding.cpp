@@ -81,6 +81,7 @@ struct PlanEntry {
 };
 std::list<PlanEntry> g_plans;
 constexpr size_t kMaxPlans = 8;
+int g_plan_policy = 0;   // 0: where eppgcn_plan_recommended says so, 1: always, -1: never
 
 int dim_class_of(int dim) { return dim <= 32 ? 0 : dim <= 128 ? 1 : 2; }
 int dim_of_class(int c) { return c == 0 ? 32 : c == 1 ? 128 : 256; }
@@ -97,7 +98,8 @@ Tensor aligned_bytes(size_t bytes, const Tensor& like, void** base)
 const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& rows, bool is_forward, int64_t num_parts,
                      int64_t num_slots, int num_nodes, int dim)
 {
-    if (num_parts <= 0) return nullptr;
+    if (num_parts <= 0 || g_plan_policy < 0) return nullptr;
+    if (g_plan_policy == 0 && !eppgcn_plan_recommended(num_nodes, dim)) return nullptr;
     const int dc = dim_class_of(dim);
     for (auto it = g_plans.begin(); it != g_plans.end(); ++it) {
         if (it->part_ptr == part_ptr.data_ptr() && it->col == col.data_ptr() && it->rows == rows.data_ptr() &&
@@ -147,7 +149,7 @@ const void* backward_plan(const Tensor& part_pointer, const Tensor& edge_list, c
         if (c.part_ptr == part_pointer.data_ptr() && c.num_parts == num_parts)
             return c.use_plan ? plan_for(part_pointer, edge_list, ids, false, num_parts, -1, num_nodes, dim) : nullptr;
     const int64_t valid_len = part_pointer[num_parts].item<int64_t>();
-    const bool use = 2 * valid_len >= edge_list.numel();
+    const bool use = g_plan_policy > 0 || 2 * valid_len >= edge_list.numel();
     if (g_path_choices.size() >= 64) g_path_choices.erase(g_path_choices.begin());
     g_path_choices.push_back({part_pointer.data_ptr(), num_parts, use});
     return use ? plan_for(part_pointer, edge_list, ids, false, num_parts, valid_len, num_nodes, dim) : nullptr;
@@ -392,7 +394,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("clear_time", &eppgcn_clear_time, "reset accumulated kernel times");
     m.def("set_timing", [](bool on) { eppgcn_set_timing(on ? 1 : 0); }, "enable per-call kernel timing");
     m.def("get_time_ms", &eppgcn_get_time_ms, "accumulated kernel time in ms");
-    m.def("clear_plans", []() { g_plans.clear(); }, "drop the cached execution plans");
+    m.def("clear_plans", []() { g_plans.clear(); g_path_choices.clear(); }, "drop the cached execution plans");
+    m.def("set_plan_policy", [](int policy) { g_plan_policy = policy; g_plans.clear(); g_path_choices.clear(); },
+          "execution plans: 0 = where the feature table outgrows the caches (default), 1 = always, -1 = never");
+    m.def("cached_plans", []() { return static_cast<int>(g_plans.size()); }, "number of execution plans held");
 
     m.def("build_part", &build_part, "forward neighbour groups (HIP)");
     m.def("build_back_part", &build_back_part, "compaction + group split in one call (HIP)");

@@ -60,10 +60,12 @@ def choose_back_part_size(mode: str, constant: int, valid_node: int, valid_len: 
 
 def prepare(graph: graphs.Graph, num_layers: int = 2, train_ratio: float = 0.1, mask_seed: int = 2,
             part_size: int = None, backsize_mode: str = "constant", backsize: int = 32,
-            train_mask: torch.Tensor = None, widths=(16, 22), plan: bool = True) -> Workload:
+            train_mask: torch.Tensor = None, widths=(16, 22), plan=None) -> Workload:
     g = graph
     dev = g.column_index.device
     n, e = g.num_nodes, g.num_edges
+    if plan is None:             # default: plans where the feature table outgrows the caches
+        plan = capi.plan_recommended(n, max(widths))
     ps = part_size or max(1, int(g.avg_degree))       # EPPGCN/param.py:80
     part_ptr, part2node = capi.build_part(ps, g.row_pointers, e)
     if train_mask is None:

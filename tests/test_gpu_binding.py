@@ -131,8 +131,12 @@ def _dense_model_grads(indptr, col, s, x, w0, w1, train, y):
     return float(loss), w0.grad.numpy(), w1.grad.numpy()
 
 
-def test_autograd_layer_gradients_vs_dense_float64(GNNA):
+@pytest.mark.parametrize("policy", [0, 1, -1])
+def test_autograd_layer_gradients_vs_dense_float64(GNNA, policy):
+    """policy 1 forces column-blocked execution plans (normally reserved for large graphs), so that
+    the module's plan cache and the planned kernels are exercised through autograd as well."""
     from eppgcn_amd import graphs, train
+    GNNA.set_plan_policy(policy)
     indptr, col = random_symmetric_csr(400, 1500, 3)
     n = indptr.size - 1
     g = graphs.Graph("t", n, dev(indptr), dev(col), dev(scale_inv_sqrt(indptr)))
@@ -155,6 +159,8 @@ def test_autograd_layer_gradients_vs_dense_float64(GNNA):
     # later iterations reuse the prepared path and give the same gradients
     tr.train_step(False)
     assert np.allclose(tr.model.convs[0].weights.grad.cpu().numpy(), g0, rtol=1e-4, atol=1e-7)
+    assert (GNNA.cached_plans() > 0) == (policy == 1)
+    GNNA.set_plan_policy(0)
 
 
 @pytest.mark.parametrize("cfg", ["cfg1_uniform", "cfg2_chunglu"])
