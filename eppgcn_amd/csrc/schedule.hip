@@ -180,6 +180,8 @@ size_t plan_workspace_bytes(long long num_parts)
            align256(temp) + 256;
 }
 
+int workspace_pitch(int dim);   // aggregate.hip
+
 static int g_force_shift = 0;
 static int g_keep_rows = 8;
 void set_schedule_shift(int shift) { g_force_shift = shift; }
@@ -191,7 +193,7 @@ int schedule_shift(int dim)
     // column blocks of about 4 MB of feature rows (65536 rows of 64 bytes), one XCD's L2: measured
     // at R-MAT scale 22, blocks of 8K..256K rows gather equally fast and larger blocks leave fewer
     // partial sums to combine
-    int row_bytes = 4 * (dim <= 8 ? (dim + 3) / 4 * 4 : (dim + 7) / 8 * 8);
+    const int row_bytes = 4 * workspace_pitch(dim);
     int shift = 16;
     while (shift > 8 && (static_cast<long long>(row_bytes) << shift) > (6ll << 20)) --shift;
     return shift;
