@@ -24,9 +24,10 @@
  *   - The aggregation functions take an optional feature workspace of
  *     eppgcn_feature_workspace_floats(num_nodes, dim) floats, 16-byte aligned
  *     (its size is passed as workspace_floats and checked).  With it the
- *     features are scaled by `degrees` once per call into rows padded to whole
- *     32-byte sectors and the kernel gathers pre-scaled rows, which removes one
- *     random memory request per edge; with NULL the kernel gathers the
+ *     features are scaled by `degrees` once per call into padded rows (to a
+ *     power of two up to 128 bytes, beyond that to whole 32-byte sectors) and
+ *     the kernel gathers pre-scaled rows, which removes one random memory
+ *     request per edge; with NULL the kernel gathers the
  *     neighbour's scale per edge and needs no scratch.  The workspace may be the
  *     input pointer itself when the caller no longer needs the unscaled input
  *     (it is then overwritten with degrees[r]*in[r,:], unpadded).  Results of the
