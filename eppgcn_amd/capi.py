@@ -22,6 +22,8 @@ EXPORTS = [
     "eppgcn_map_back_part_size", "eppgcn_threshold_back_part_size", "eppgcn_split_back_part",
     "eppgcn_build_part", "eppgcn_get_ginfo", "eppgcn_set_timing", "eppgcn_print_time",
     "eppgcn_clear_time", "eppgcn_get_time_ms", "eppgcn_set_team_size", "eppgcn_set_rounds", "eppgcn_set_plan_shift", "eppgcn_set_plan_keep_rows",
+    "eppgcn_feature_workspace_pitch", "eppgcn_update_forward", "eppgcn_update_backward_input",
+    "eppgcn_update_workspace_bytes", "eppgcn_update_backward_weight", "eppgcn_update_supported",
 ]
 
 _lib = None
@@ -82,6 +84,17 @@ def load():
     lib.eppgcn_set_plan_shift.restype = None
     lib.eppgcn_set_plan_keep_rows.argtypes = [i]
     lib.eppgcn_set_plan_keep_rows.restype = None
+    lib.eppgcn_feature_workspace_pitch.argtypes = [i]
+    lib.eppgcn_feature_workspace_pitch.restype = i
+    lib.eppgcn_update_supported.argtypes = [i, i]
+    lib.eppgcn_update_supported.restype = i
+    lib.eppgcn_update_forward.argtypes = [p, i, p, p, p, i, i64, i, i, p]
+    lib.eppgcn_update_backward_input.argtypes = [p, p, p, p, i64, i, i, p]
+    lib.eppgcn_update_workspace_bytes.argtypes = [i64, i, i]
+    lib.eppgcn_update_workspace_bytes.restype = sz
+    lib.eppgcn_update_backward_weight.argtypes = [p, p, p, i, i64, i, i, p, sz, p]
+    for name in ("eppgcn_update_forward", "eppgcn_update_backward_input", "eppgcn_update_backward_weight"):
+        getattr(lib, name).restype = i
     for name in ("eppgcn_spmm_forward", "eppgcn_spmm_backward", "eppgcn_ours_backward", "eppgcn_mask_forward",
                  "eppgcn_compact_back_edge", "eppgcn_count_nonzero", "eppgcn_map_back_part_size",
                  "eppgcn_threshold_back_part_size", "eppgcn_split_back_part", "eppgcn_build_part",
@@ -125,6 +138,66 @@ def _mask_bytes(t, name):
 
 
 # --------------------------------------------------------------------------- aggregation
+def feature_workspace_pitch(dim: int) -> int:
+    """Row pitch (floats) of the pre-scaled feature workspace for `dim`-wide features."""
+    return int(load().eppgcn_feature_workspace_pitch(int(dim)))
+
+
+def update_forward(x, w, scale=None, relu_input=False, ld_out=None, out=None):
+    """scale[r] * act(x) @ w as rows ``ld_out`` floats apart (zeros in the padding) -> [N, ld_out]."""
+    lib = load()
+    _dev(x, torch.float32, "x"); _dev(w, torch.float32, "w")
+    n, k = x.shape
+    if w.dim() != 2 or w.shape[0] != k:
+        raise EppgcnError("w must be [in_dim, out_dim]")
+    m = w.shape[1]
+    ld = int(ld_out) if ld_out else m
+    if scale is not None:
+        _dev(scale, torch.float32, "scale")
+        if scale.numel() != n:
+            raise EppgcnError("scale must have one entry per row")
+    if out is None:
+        out = torch.empty((n, ld), dtype=torch.float32, device=x.device)
+    elif out.numel() < n * ld:
+        raise EppgcnError("out is too small")
+    _check(lib.eppgcn_update_forward(_ptr(out), ld, _ptr(x), _ptr(w), _ptr(scale), int(bool(relu_input)), n, k, m,
+                                     _stream()))
+    return out
+
+
+def update_backward_input(g, w, relu_ref=None):
+    """(g @ w.T), zeroed where relu_ref <= 0 -> [N, in_dim]."""
+    lib = load()
+    _dev(g, torch.float32, "g"); _dev(w, torch.float32, "w")
+    n, m = g.shape
+    if w.dim() != 2 or w.shape[1] != m:
+        raise EppgcnError("w must be [in_dim, out_dim] with out_dim = g.shape[1]")
+    k = w.shape[0]
+    if relu_ref is not None:
+        _dev(relu_ref, torch.float32, "relu_ref")
+        if tuple(relu_ref.shape) != (n, k):
+            raise EppgcnError("relu_ref must be [N, in_dim]")
+    d_x = torch.empty((n, k), dtype=torch.float32, device=g.device)
+    _check(lib.eppgcn_update_backward_input(_ptr(d_x), _ptr(g), _ptr(w), _ptr(relu_ref), n, k, m, _stream()))
+    return d_x
+
+
+def update_backward_weight(x, g, relu_input=False):
+    """act(x).T @ g -> [in_dim, out_dim], summed in a fixed order."""
+    lib = load()
+    _dev(x, torch.float32, "x"); _dev(g, torch.float32, "g")
+    n, k = x.shape
+    if g.shape[0] != n:
+        raise EppgcnError("x and g must have the same number of rows")
+    m = g.shape[1]
+    d_w = torch.empty((k, m), dtype=torch.float32, device=x.device)
+    nbytes = lib.eppgcn_update_workspace_bytes(n, k, m)
+    ws = torch.empty(max(1, (nbytes + 3) // 4), dtype=torch.float32, device=x.device)
+    _check(lib.eppgcn_update_backward_weight(_ptr(d_w), _ptr(x), _ptr(g), int(bool(relu_input)), n, k, m, _ptr(ws),
+                                             nbytes, _stream()))
+    return d_w
+
+
 def _feature_workspace(workspace, feats):
     """None -> per-edge scale gather (no scratch); True -> allocate; a tensor -> use it (it may be
     `feats` itself, which is then overwritten with the scaled features)."""
@@ -202,14 +275,23 @@ def _plan_ptr(plan, num_parts):
 
 
 def spmm_forward(feats, column_index, degrees, part_ptr, part2node, part_size=32, dim_worker=32,
-                 warp_per_block=8, row_pointers=None, out=None, backward=False, workspace=True, plan=None):
+                 warp_per_block=8, row_pointers=None, out=None, backward=False, workspace=True, plan=None,
+                 prescaled_dim=None):
     """out[N, D] = neighbour-group aggregation of feats (``backward=True`` uses the unpruned
-    backward entry point; same operator)."""
+    backward entry point; same operator).  ``feats=None`` with ``prescaled_dim=D``: ``workspace``
+    already holds the scaled, padded rows (as ``update_forward(..., scale=degrees)`` writes them)."""
     lib = load()
-    _dev(feats, torch.float32, "feats"); _dev(column_index, torch.int32, "column_index")
+    _dev(column_index, torch.int32, "column_index")
     _dev(degrees, torch.float32, "degrees"); _dev(part_ptr, torch.int32, "part_ptr")
     _dev(part2node, torch.int32, "part2node")
-    n, dim = feats.shape
+    if feats is None:
+        _dev(workspace, torch.float32, "workspace")
+        n, dim = degrees.numel(), int(prescaled_dim)
+        if out is None:
+            out = torch.empty((n, dim), dtype=torch.float32, device=degrees.device)
+    else:
+        _dev(feats, torch.float32, "feats")
+        n, dim = feats.shape
     num_parts = part2node.numel()
     if part_ptr.numel() < num_parts + 1:
         raise EppgcnError("part_ptr needs num_parts + 1 entries")
@@ -218,7 +300,7 @@ def spmm_forward(feats, column_index, degrees, part_ptr, part2node, part_size=32
     if out is None:
         out = torch.empty_like(feats)
     fn = lib.eppgcn_spmm_backward if backward else lib.eppgcn_spmm_forward
-    ws = _feature_workspace(workspace, feats)
+    ws = workspace if feats is None else _feature_workspace(workspace, feats)
     _check(fn(_ptr(out), _ptr(feats), _ptr(row_pointers), _ptr(column_index), _ptr(degrees), _ptr(part_ptr),
               _ptr(part2node), n, dim, num_parts, part_size, dim_worker, warp_per_block, _ptr(ws),
               0 if ws is None else ws.numel(), _plan_ptr(plan, num_parts), _stream()))

@@ -551,8 +551,10 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
     EPPGCN_HIP(hipMemsetAsync(out, 0, static_cast<size_t>(num_nodes) * dim * sizeof(float), stream));
     if (num_parts == 0) return kOk;
     if (prescaled) {
+        // in == nullptr: the caller (the dense update) already wrote the scaled, padded rows
         ld_in = workspace == in ? dim : workspace_pitch(dim);
-        if (int rc = launch_scale_rows(workspace, in, scale, num_nodes, dim, ld_in, stream)) return rc;
+        if (in)
+            if (int rc = launch_scale_rows(workspace, in, scale, num_nodes, dim, ld_in, stream)) return rc;
         in = workspace;
     }
     KernelTimer timer(stream, sink, sink2);   // brackets the aggregation kernel alone

@@ -24,6 +24,11 @@ int launch_build_plan(const int*, const int*, const int*, const int*, int, long 
 void set_agg_force_team(int);
 void set_agg_force_rounds(int);
 size_t feature_workspace_floats(long long, int);
+int workspace_pitch(int);
+int launch_dense_rows(float*, int, int, const float*, int, const float*, long long, long long, const float*,
+                      const float*, int, int, long long, int, int, hipStream_t);
+size_t update_workspace_bytes(long long, int, int);
+int launch_dense_weight(float*, const float*, int, const float*, int, int, long long, int, int, void*, hipStream_t);
 size_t compact_workspace_bytes(long long);
 size_t split_workspace_bytes(long long);
 int launch_mask_forward(const int*, const int*, const int*, const uint8_t*, uint8_t*, int*, int*, int, long long, int,
@@ -70,7 +75,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 3; }
+int eppgcn_abi_version(void) { return 4; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -81,7 +86,7 @@ int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
     EPPGCN_REQUIRE(part_size > 0 && dim_worker > 0 && warp_per_block > 0, "launch hints must be positive");
     if (num_nodes == 0) return kOk;
-    EPPGCN_REQUIRE(out && in && degrees, "null feature or scale pointer");
+    EPPGCN_REQUIRE(out && (in || workspace) && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (column_index && part_pointers && part2node), "null index pointer");
     EPPGCN_REQUIRE(aligned(out, 4) && aligned(in, 4), "feature pointers must be 4-byte aligned");
     EPPGCN_REQUIRE(!plan || aligned(plan, 256), "plan must be 256-byte aligned");
@@ -102,7 +107,7 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
     EPPGCN_REQUIRE(part_size > 0 && dim_worker > 0 && warp_per_block > 0, "launch hints must be positive");
     if (num_nodes == 0) return kOk;
-    EPPGCN_REQUIRE(d_input && d_output && degrees, "null feature or scale pointer");
+    EPPGCN_REQUIRE(d_input && (d_output || workspace) && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (column_index && part_pointers && part2node), "null index pointer");
     EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
     EPPGCN_REQUIRE(!plan || aligned(plan, 256), "plan must be 256-byte aligned");
@@ -124,7 +129,7 @@ int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* i
     EPPGCN_REQUIRE(blockx > 0 && blocky > 0, "launch hints must be positive");
     EPPGCN_REQUIRE(layer >= 1, "layer is 1-based");
     if (num_nodes == 0) return kOk;
-    EPPGCN_REQUIRE(d_input && d_output && degrees, "null feature or scale pointer");
+    EPPGCN_REQUIRE(d_input && (d_output || workspace) && degrees, "null feature or scale pointer");
     EPPGCN_REQUIRE(num_parts == 0 || (ids && part_pointer && edge_list), "null index pointer");
     EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
     EPPGCN_REQUIRE(!plan || aligned(plan, 256), "plan must be 256-byte aligned");
@@ -350,5 +355,64 @@ void eppgcn_set_team_size(int lanes) { set_agg_force_team(lanes); }
 void eppgcn_set_rounds(int rounds) { set_agg_force_rounds(rounds); }
 void eppgcn_set_plan_shift(int shift) { set_schedule_shift(shift); }
 void eppgcn_set_plan_keep_rows(int groups) { set_plan_keep_rows(groups); }
+
+// ---- dense update
+int eppgcn_feature_workspace_pitch(int dim) { return dim > 0 ? workspace_pitch(dim) : 0; }
+
+int eppgcn_update_supported(int in_dim, int out_dim)
+{
+    if (in_dim <= 0 || out_dim <= 0) return 0;
+    int mask = 0;
+    if (in_dim <= 1024) mask |= 1;       // forward: reduction over in_dim
+    if (out_dim <= 1024) mask |= 2;      // backward_input: reduction over out_dim
+    if (out_dim <= 64) mask |= 4;        // backward_weight: gradient columns held in one block
+    return mask;
+}
+
+int eppgcn_update_forward(float* out, int ld_out, const float* x, const float* w, const float* scale,
+                          int relu_input, int64_t num_nodes, int in_dim, int out_dim, void* stream)
+{
+    EPPGCN_REQUIRE(num_nodes >= 0 && in_dim > 0 && out_dim > 0, "num_nodes >= 0, in_dim > 0, out_dim > 0 required");
+    EPPGCN_REQUIRE(ld_out >= out_dim, "ld_out must be at least out_dim");
+    if (num_nodes == 0) return kOk;
+    EPPGCN_REQUIRE(out && x && w, "null matrix pointer");
+    EPPGCN_REQUIRE(aligned(out, 4) && aligned(x, 4) && aligned(w, 4), "matrix pointers must be 4-byte aligned");
+    EPPGCN_REQUIRE(out != x, "the product cannot be written over its input");
+    return launch_dense_rows(out, ld_out, ld_out, x, in_dim, w, out_dim, 1, scale, nullptr, 0, relu_input ? 1 : 0,
+                             num_nodes, in_dim, out_dim, static_cast<hipStream_t>(stream));
+}
+
+int eppgcn_update_backward_input(float* d_x, const float* g, const float* w, const float* relu_ref,
+                                 int64_t num_nodes, int in_dim, int out_dim, void* stream)
+{
+    EPPGCN_REQUIRE(num_nodes >= 0 && in_dim > 0 && out_dim > 0, "num_nodes >= 0, in_dim > 0, out_dim > 0 required");
+    if (num_nodes == 0) return kOk;
+    EPPGCN_REQUIRE(d_x && g && w, "null matrix pointer");
+    EPPGCN_REQUIRE(aligned(d_x, 4) && aligned(g, 4) && aligned(w, 4) && aligned(relu_ref, 4),
+                   "matrix pointers must be 4-byte aligned");
+    EPPGCN_REQUIRE(d_x != g, "the product cannot be written over its input");
+    // reduction over the out_dim columns of g; operand element (d, k) is w[k, d]
+    return launch_dense_rows(d_x, in_dim, in_dim, g, out_dim, w, 1, out_dim, nullptr, relu_ref, in_dim, 0, num_nodes,
+                             out_dim, in_dim, static_cast<hipStream_t>(stream));
+}
+
+size_t eppgcn_update_workspace_bytes(int64_t num_nodes, int in_dim, int out_dim)
+{
+    return update_workspace_bytes(num_nodes, in_dim, out_dim);
+}
+
+int eppgcn_update_backward_weight(float* d_w, const float* x, const float* g, int relu_input, int64_t num_nodes,
+                                  int in_dim, int out_dim, void* workspace, size_t workspace_bytes, void* stream)
+{
+    EPPGCN_REQUIRE(num_nodes >= 0 && in_dim > 0 && out_dim > 0, "num_nodes >= 0, in_dim > 0, out_dim > 0 required");
+    EPPGCN_REQUIRE(d_w, "null output pointer");
+    EPPGCN_REQUIRE(num_nodes == 0 || (x && g), "null matrix pointer");
+    EPPGCN_REQUIRE(aligned(d_w, 4) && aligned(x, 4) && aligned(g, 4), "matrix pointers must be 4-byte aligned");
+    EPPGCN_REQUIRE(num_nodes == 0 || (workspace && aligned(workspace, 4) &&
+                                      workspace_bytes >= update_workspace_bytes(num_nodes, in_dim, out_dim)),
+                   "workspace smaller than eppgcn_update_workspace_bytes(num_nodes, in_dim, out_dim)");
+    return launch_dense_weight(d_w, x, in_dim, g, out_dim, relu_input ? 1 : 0, num_nodes, in_dim, out_dim, workspace,
+                               static_cast<hipStream_t>(stream));
+}
 
 }  // extern "C"

@@ -1,8 +1,9 @@
 // Python extension module `GNNAdvisor` for PyTorch-ROCm: the twelve functions the
 // reference's Python calls (EPPGCN/GCNConv/EPPGCN.cpp:388-403), same positional
 // signatures, implemented over the C ABI of libeppgcn_hip.so.  torch supplies the
-// tensors, the dense X*W products and the current HIP stream; everything else
-// happens in the HIP library.  Host C++ only: no device code in this file.
+// tensors and the current HIP stream (and torch::mm for dense products whose shapes
+// the library's tall-and-skinny kernels do not cover); everything else happens in
+// the HIP library.  Host C++ only: no device code in this file.
 //
 // Differences from the reference binding, all deliberate:
 //   - errors raise (RuntimeError in Python) instead of printf + exit(-1);
@@ -161,57 +162,125 @@ Tensor feature_scratch(const Tensor& feats)
     return torch::empty({static_cast<int64_t>(n)}, feats.options());
 }
 
+// ---------------------------------------------------------------- dense update helpers
+// The three products around the aggregation run in the library's tall-and-skinny kernels when the
+// shapes fit them (eppgcn_update_supported) and in torch::mm otherwise; g_dense_policy -1 forces mm.
+int g_dense_policy = 0;
+
+int dense_support(const Tensor& X, const Tensor& W)
+{
+    if (g_dense_policy < 0) return 0;
+    return eppgcn_update_supported(static_cast<int>(X.size(1)), static_cast<int>(W.size(1)));
+}
+
+// scale[r] * act(X) * W as the padded, pre-scaled feature table the aggregation gathers from
+Tensor scaled_product(const Tensor& X, const Tensor& W, const Tensor& degrees, bool relu_input, size_t* ws_floats)
+{
+    const int64_t n = X.size(0);
+    const int dim = static_cast<int>(W.size(1));
+    const int pitch = eppgcn_feature_workspace_pitch(dim);
+    *ws_floats = eppgcn_feature_workspace_floats(n, dim);
+    auto scaled = torch::empty({static_cast<int64_t>(*ws_floats)}, X.options());
+    check(eppgcn_update_forward(scaled.data_ptr<float>(), pitch, X.data_ptr<float>(), W.data_ptr<float>(),
+                                f32(degrees), relu_input ? 1 : 0, n, static_cast<int>(X.size(1)), dim, stream_of(X)),
+          "update_forward");
+    return scaled;
+}
+
+// {dX or an empty tensor, dW} from the aggregated gradient G
+std::vector<Tensor> dense_backward(const Tensor& G, const Tensor& X, const Tensor& W, bool need_dx, bool relu_input)
+{
+    const int64_t n = X.size(0);
+    const int in_dim = static_cast<int>(X.size(1)), out_dim = static_cast<int>(W.size(1));
+    const int sup = dense_support(X, W);
+    Tensor d_weight, d_input;
+    if (sup & 4) {
+        d_weight = torch::empty({in_dim, out_dim}, X.options());
+        const size_t nbytes = eppgcn_update_workspace_bytes(n, in_dim, out_dim);
+        auto ws = torch::empty({static_cast<int64_t>((nbytes + 3) / 4) + 1}, X.options());
+        check(eppgcn_update_backward_weight(d_weight.data_ptr<float>(), f32(X), f32(G), relu_input ? 1 : 0, n, in_dim,
+                                            out_dim, ws.data_ptr<float>(), nbytes, stream_of(X)),
+              "update_backward_weight");
+    } else {
+        d_weight = torch::mm((relu_input ? torch::relu(X) : X).transpose(0, 1), G);
+    }
+    if (!need_dx) {
+        d_input = torch::empty({0}, X.options());
+    } else if (sup & 2) {
+        d_input = torch::empty({n, in_dim}, X.options());
+        check(eppgcn_update_backward_input(d_input.data_ptr<float>(), f32(G), f32(W), relu_input ? f32(X) : nullptr, n,
+                                           in_dim, out_dim, stream_of(X)),
+              "update_backward_input");
+    } else {
+        d_input = torch::mm(G, W.transpose(0, 1));
+        if (relu_input) d_input = d_input * (X > 0);
+    }
+    return {d_input, d_weight};
+}
+
 // ---------------------------------------------------------------- forward / backward
 std::vector<Tensor> forward(Tensor input, Tensor weight, Tensor row_pointers, Tensor column_index, Tensor degrees,
-                            Tensor part_pointers, Tensor part2Node, int partSize, int dimWorker, int warpPerBlock)
+                            Tensor part_pointers, Tensor part2Node, int partSize, int dimWorker, int warpPerBlock,
+                            bool relu_input)
 {
     CHECK_F32(input); CHECK_F32(weight); CHECK_I32(row_pointers); CHECK_I32(column_index);
     CHECK_F32(degrees); CHECK_I32(part_pointers); CHECK_I32(part2Node);
     TORCH_CHECK(input.dim() == 2 && weight.dim() == 2 && input.size(1) == weight.size(0), "shape mismatch");
     TORCH_CHECK(degrees.numel() == input.size(0), "degrees must have one entry per vertex");
     TORCH_CHECK(part_pointers.numel() >= part2Node.numel() + 1, "part_pointers needs num_parts + 1 entries");
-    auto tmp = torch::mm(input, weight);
-    auto output = torch::empty_like(tmp);
+    const int64_t n = input.size(0);
+    const int dim = static_cast<int>(weight.size(1));
+    auto output = torch::empty({n, dim}, input.options());
+    const void* plan = plan_for(part_pointers, column_index, part2Node, true, part2Node.numel(), column_index.numel(),
+                                static_cast<int>(n), dim);
+    if (n > 0 && (dense_support(input, weight) & 1)) {
+        // the product is written scaled and padded, ready to be gathered: no separate scaling pass
+        size_t ws_floats = 0;
+        auto scaled = scaled_product(input, weight, degrees, relu_input, &ws_floats);
+        check(eppgcn_spmm_forward(output.data_ptr<float>(), nullptr, i32(row_pointers), i32(column_index),
+                                  f32(degrees), i32(part_pointers), i32(part2Node), static_cast<int>(n), dim,
+                                  static_cast<int>(part2Node.numel()), partSize, dimWorker, warpPerBlock,
+                                  scaled.data_ptr<float>(), ws_floats, plan, stream_of(input)),
+              "forward");
+        return {output};
+    }
+    auto tmp = torch::mm(relu_input ? torch::relu(input) : input, weight);
     // tmp is ours: when its rows need no padding it is scaled in place, otherwise into scratch
-    const size_t ws_floats = eppgcn_feature_workspace_floats(tmp.size(0), static_cast<int>(tmp.size(1)));
+    const size_t ws_floats = eppgcn_feature_workspace_floats(tmp.size(0), dim);
     auto scaled = ws_floats == static_cast<size_t>(tmp.numel())
                       ? tmp
                       : torch::empty({static_cast<int64_t>(ws_floats)}, tmp.options());
-    check(eppgcn_spmm_forward(output.data_ptr<float>(), tmp.data_ptr<float>(), i32(row_pointers), i32(column_index),
-                              f32(degrees), i32(part_pointers), i32(part2Node), static_cast<int>(tmp.size(0)),
-                              static_cast<int>(tmp.size(1)), static_cast<int>(part2Node.numel()), partSize, dimWorker,
-                              warpPerBlock, scaled.data_ptr<float>(), ws_floats,
-                              plan_for(part_pointers, column_index, part2Node, true, part2Node.numel(),
-                                       column_index.numel(), static_cast<int>(tmp.size(0)),
-                                       static_cast<int>(tmp.size(1))),
-                              stream_of(input)),
+    check(eppgcn_spmm_forward(output.data_ptr<float>(), f32(tmp), i32(row_pointers), i32(column_index),
+                              f32(degrees), i32(part_pointers), i32(part2Node), static_cast<int>(n), dim,
+                              static_cast<int>(part2Node.numel()), partSize, dimWorker, warpPerBlock,
+                              scaled.numel() ? scaled.data_ptr<float>() : nullptr, ws_floats, plan, stream_of(input)),
           "forward");
     return {output};
 }
 
 std::vector<Tensor> backward(Tensor d_output, Tensor X, Tensor W, Tensor row_pointers, Tensor column_index,
                              Tensor degrees, Tensor part_pointers, Tensor part2Node, int partSize, int dimWorker,
-                             int warpPerBlock)
+                             int warpPerBlock, bool need_dx, bool relu_input)
 {
     CHECK_F32(d_output); CHECK_F32(X); CHECK_F32(W); CHECK_I32(row_pointers); CHECK_I32(column_index);
     CHECK_F32(degrees); CHECK_I32(part_pointers); CHECK_I32(part2Node);
     TORCH_CHECK(d_output.dim() == 2 && degrees.numel() == d_output.size(0), "shape mismatch");
+    TORCH_CHECK(X.dim() == 2 && W.dim() == 2 && X.size(0) == d_output.size(0) && X.size(1) == W.size(0) &&
+                    W.size(1) == d_output.size(1), "X, W and d_output do not fit together");
     TORCH_CHECK(part_pointers.numel() >= part2Node.numel() + 1, "part_pointers needs num_parts + 1 entries");
     auto d_input_prime = torch::empty_like(d_output);
     auto scaled = feature_scratch(d_output);     // d_output belongs to autograd: scale into scratch
-    check(eppgcn_spmm_backward(d_input_prime.data_ptr<float>(), d_output.data_ptr<float>(), i32(row_pointers),
+    check(eppgcn_spmm_backward(d_input_prime.data_ptr<float>(), f32(d_output), i32(row_pointers),
                                i32(column_index), f32(degrees), i32(part_pointers), i32(part2Node),
                                static_cast<int>(d_output.size(0)), static_cast<int>(d_output.size(1)),
                                static_cast<int>(part2Node.numel()), partSize, dimWorker, warpPerBlock,
-                               scaled.data_ptr<float>(), static_cast<size_t>(scaled.numel()),
+                               scaled.numel() ? scaled.data_ptr<float>() : nullptr, static_cast<size_t>(scaled.numel()),
                                plan_for(part_pointers, column_index, part2Node, true, part2Node.numel(),
                                         column_index.numel(), static_cast<int>(d_output.size(0)),
                                         static_cast<int>(d_output.size(1))),
                                stream_of(d_output)),
           "backward");
-    auto d_input = torch::mm(d_input_prime, W.transpose(0, 1));
-    auto d_weight = torch::mm(X.transpose(0, 1), d_input_prime);
-    return {d_input, d_weight};
+    return dense_backward(d_input_prime, X, W, need_dx, relu_input);
 }
 
 void mask_forward(Tensor id, Tensor partPointer, Tensor edgeList, Tensor src_mask, Tensor ngh_mask,
@@ -234,26 +303,28 @@ void mask_forward(Tensor id, Tensor partPointer, Tensor edgeList, Tensor src_mas
 }
 
 std::vector<Tensor> ours_backward(Tensor d_output, Tensor X, Tensor W, Tensor id, Tensor partPointer, Tensor edgeList,
-                                  Tensor degrees, int partSize, int numParts, int layer, int blockx, int blocky)
+                                  Tensor degrees, int partSize, int numParts, int layer, int blockx, int blocky,
+                                  bool need_dx, bool relu_input)
 {
     CHECK_F32(d_output); CHECK_F32(X); CHECK_F32(W); CHECK_I32(id); CHECK_I32(partPointer); CHECK_I32(edgeList);
     CHECK_F32(degrees);
     TORCH_CHECK(d_output.dim() == 2 && degrees.numel() == d_output.size(0), "shape mismatch");
+    TORCH_CHECK(X.dim() == 2 && W.dim() == 2 && X.size(0) == d_output.size(0) && X.size(1) == W.size(0) &&
+                    W.size(1) == d_output.size(1), "X, W and d_output do not fit together");
     TORCH_CHECK(numParts >= 0 && partPointer.numel() >= static_cast<int64_t>(numParts) + 1,
                 "partPointer needs numParts + 1 entries");
     auto d_input_prime = torch::empty_like(d_output);
     auto scaled = feature_scratch(d_output);     // d_output belongs to autograd: scale into scratch
-    check(eppgcn_ours_backward(d_input_prime.data_ptr<float>(), d_output.data_ptr<float>(), i32(id), i32(partPointer),
+    check(eppgcn_ours_backward(d_input_prime.data_ptr<float>(), f32(d_output), i32(id), i32(partPointer),
                                i32(edgeList), f32(degrees), static_cast<int>(d_output.size(0)),
                                static_cast<int>(d_output.size(1)), numParts, partSize > 0 ? partSize : 1, layer, blockx,
-                               blocky, scaled.data_ptr<float>(), static_cast<size_t>(scaled.numel()),
+                               blocky, scaled.numel() ? scaled.data_ptr<float>() : nullptr,
+                               static_cast<size_t>(scaled.numel()),
                                backward_plan(partPointer, edgeList, id, numParts, static_cast<int>(d_output.size(0)),
                                              static_cast<int>(d_output.size(1))),
                                stream_of(d_output)),
           "ours_backward");
-    auto d_input = torch::mm(d_input_prime, W.transpose(0, 1));
-    auto d_weight = torch::mm(X.transpose(0, 1), d_input_prime);
-    return {d_input, d_weight};
+    return dense_backward(d_input_prime, X, W, need_dx, relu_input);
 }
 
 // ---------------------------------------------------------------- path preparation
@@ -386,10 +457,24 @@ Tensor get_ginfo(Tensor node_deg, int valid_len)
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
-    m.def("forward", &forward, "neighbour-group forward: mm + aggregation (HIP)");
-    m.def("backward", &backward, "unpruned backward: aggregation + 2 mm (HIP)");
+    namespace py = pybind11;
+    // the trailing keyword arguments are additions: relu_input applies max(x, 0) to the layer input
+    // inside the product (and masks dX accordingly); need_dx=False skips dX (an empty tensor is returned)
+    m.def("forward", &forward, "neighbour-group forward: X*W + aggregation (HIP)", py::arg("input"), py::arg("weight"),
+          py::arg("row_pointers"), py::arg("column_index"), py::arg("degrees"), py::arg("part_pointers"),
+          py::arg("part2Node"), py::arg("partSize"), py::arg("dimWorker"), py::arg("warpPerBlock"),
+          py::arg("relu_input") = false);
+    m.def("backward", &backward, "unpruned backward: aggregation + dX, dW (HIP)", py::arg("d_output"), py::arg("X"),
+          py::arg("W"), py::arg("row_pointers"), py::arg("column_index"), py::arg("degrees"), py::arg("part_pointers"),
+          py::arg("part2Node"), py::arg("partSize"), py::arg("dimWorker"), py::arg("warpPerBlock"),
+          py::arg("need_dx") = true, py::arg("relu_input") = false);
     m.def("mask_forward", &mask_forward, "mark the backward execution path of one layer (HIP)");
-    m.def("ours_backward", &ours_backward, "pruned backward over the compacted path: aggregation + 2 mm (HIP)");
+    m.def("ours_backward", &ours_backward, "pruned backward over the compacted path: aggregation + dX, dW (HIP)",
+          py::arg("d_output"), py::arg("X"), py::arg("W"), py::arg("id"), py::arg("partPointer"), py::arg("edgeList"),
+          py::arg("degrees"), py::arg("partSize"), py::arg("numParts"), py::arg("layer"), py::arg("blockx"),
+          py::arg("blocky"), py::arg("need_dx") = true, py::arg("relu_input") = false);
+    m.def("set_dense_policy", [](int policy) { g_dense_policy = policy; },
+          "dense products: 0 = library kernels where the shapes fit (default), -1 = always torch::mm");
     m.def("print_time", &eppgcn_print_time, "print accumulated kernel times");
     m.def("clear_time", &eppgcn_clear_time, "reset accumulated kernel times");
     m.def("set_timing", [](bool on) { eppgcn_set_timing(on ? 1 : 0); }, "enable per-call kernel timing");

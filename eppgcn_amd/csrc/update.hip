@@ -1,0 +1,393 @@
+// Dense update of a GCN layer: the three matrix products the reference computes with torch::mm
+// around the aggregation (EPPGCN/GCNConv/EPPGCN_kernel.cu:142 X*W, :614 dX = G*W^T,
+// :615 dW = X^T*G), written for tall-and-skinny shapes (millions of rows, tens of columns)
+// where the work is bound by streaming the tall operand from HBM once.
+//
+// All three run on the fp32 matrix cores with v_mfma_f32_16x16x4_f32 (one wave computes a
+// 16x16 tile of C += A[16x4] * B[4x16]; lane l supplies A[l%16][l/16] and B[l/16][l%16] and
+// holds C[4*(l/16) + v][l%16] in accumulator register v).  The tall operand is read straight
+// from global memory in the operand layout, so no staging through LDS is needed:
+//
+//   rows kernel    out[r, m] = f(r, m) * sum_k act(X[r, k]) * Wop(k, m)      (X*W and G*W^T)
+//                  tile: 16 output columns (MFMA rows) x 16 matrix rows (MFMA columns); a lane
+//                  reads VW consecutive floats of "its" row per step, the small operand sits in
+//                  LDS in operand order; epilogues fuse the per-row scale of the aggregation
+//                  weights, the zero padding of the pre-scaled feature table, the ReLU of the
+//                  layer input and the ReLU mask of the gradient.
+//   weight kernel  dW[k, d] = sum_r act(X[r, k]) * G[r, d]
+//                  tile: 16 k x 16 d, reduction over 4 rows per instruction; every wave owns a
+//                  contiguous range of rows, block partial sums go to a workspace and a second
+//                  kernel adds them in a fixed order (deterministic, no float atomics).
+#include "common.hpp"
+
+namespace eppgcn {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kUpdateThreads = 256;
+constexpr int kUpdateWaves = kUpdateThreads / kWave;
+constexpr int kTileRows = 16;
+constexpr int kMaxWeightBlocks = 1024;
+constexpr size_t kMaxOperandLds = 64 * 1024;
+
+__device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+// ---------------------------------------------------------------- rows kernel
+// Reduction index of lane (i = l%16, j = l/16), step t, component v:  k = (4*t + j)*VW + v.
+// Any assignment of k to (step, slot) is valid as long as both operands use the same one; this
+// one lets a lane fetch VW consecutive floats of its row with one load.
+template <int VW>
+__device__ __forceinline__ void load_row_piece(float (&x)[VW], const float* __restrict__ row, int k, int K,
+                                               bool relu)
+{
+    if (k + VW <= K) {
+        if constexpr (VW == 4) {
+            const float4 t = *reinterpret_cast<const float4*>(row + k);
+            x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
+        } else if constexpr (VW == 2) {
+            const float2 t = *reinterpret_cast<const float2*>(row + k);
+            x[0] = t.x; x[1] = t.y;
+        } else {
+            x[0] = row[k];
+        }
+    } else {
+#pragma unroll
+        for (int v = 0; v < VW; ++v) x[v] = k + v < K ? row[k + v] : 0.f;
+    }
+    if (relu) {
+#pragma unroll
+        for (int v = 0; v < VW; ++v) x[v] = fmaxf(x[v], 0.f);
+    }
+}
+
+struct RowsArgs {
+    float* out;              // [N, ld_out]; columns [0, out_cols) are written, [M, out_cols) with zeros
+    const float* x;          // [N, ld_x], K valid columns
+    const float* w;          // small operand: element (k, m) at w[k*sk + m*sm]
+    const float* scale;      // per-row factor or nullptr
+    const float* relu_ref;   // [N, ld_ref] or nullptr: out[r, m] is zeroed where relu_ref[r, m] <= 0
+    long long n;
+    long long sk, sm;
+    int ld_out, out_cols, ld_x, ld_ref;
+    int K, M;
+    int relu_in;             // apply max(x, 0) to X on load
+    int vec_store;           // rows of out are 16-byte aligned
+};
+
+template <int VW, int MT, int CU>
+__global__ __launch_bounds__(kUpdateThreads) void dense_rows_kernel(RowsArgs a)
+{
+    extern __shared__ __align__(16) float w_lds[];   // [MT][chunks_p][64 lanes][VW]
+    const int chunks = (a.K + 4 * VW - 1) / (4 * VW);
+    const int chunks_p = (chunks + CU - 1) / CU * CU;
+    for (int idx = threadIdx.x; idx < MT * chunks_p * kWave * VW; idx += kUpdateThreads) {
+        const int v = idx % VW;
+        const int l = (idx / VW) % kWave;
+        const int t = (idx / (VW * kWave)) % chunks_p;
+        const int mt = idx / (VW * kWave * chunks_p);
+        const int k = (4 * t + l / 16) * VW + v;
+        const int m = mt * 16 + l % 16;
+        w_lds[idx] = (k < a.K && m < a.M) ? a.w[k * a.sk + m * a.sm] : 0.f;
+    }
+    __syncthreads();
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x / kWave;
+    const int i = lane % 16, j = lane / 16;
+    const long long tiles = (a.n + kTileRows - 1) / kTileRows;
+    for (long long tile = static_cast<long long>(blockIdx.x) * kUpdateWaves + wave; tile < tiles;
+         tile += static_cast<long long>(gridDim.x) * kUpdateWaves) {
+        const long long r = tile * kTileRows + i;
+        const bool row_ok = r < a.n;
+        const long long rc = row_ok ? r : a.n - 1;      // rows past the end read the last row, store nothing
+        const float* __restrict__ xrow = a.x + rc * a.ld_x;
+        floatx4 acc[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+        for (int t0 = 0; t0 < chunks_p; t0 += CU) {
+            float x[CU][VW];
+#pragma unroll
+            for (int u = 0; u < CU; ++u) load_row_piece<VW>(x[u], xrow, (4 * (t0 + u) + j) * VW, a.K, a.relu_in != 0);
+#pragma unroll
+            for (int u = 0; u < CU; ++u) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const float* wp = w_lds + ((mt * chunks_p + t0 + u) * kWave + lane) * VW;
+                    float wv[VW];
+                    if constexpr (VW == 4) {
+                        const float4 t = *reinterpret_cast<const float4*>(wp);
+                        wv[0] = t.x; wv[1] = t.y; wv[2] = t.z; wv[3] = t.w;
+                    } else if constexpr (VW == 2) {
+                        const float2 t = *reinterpret_cast<const float2*>(wp);
+                        wv[0] = t.x; wv[1] = t.y;
+                    } else {
+                        wv[0] = wp[0];
+                    }
+#pragma unroll
+                    for (int v = 0; v < VW; ++v) acc[mt] = mfma16(wv[v], x[u][v], acc[mt]);
+                }
+            }
+        }
+
+        if (!row_ok) continue;
+        const float s = a.scale ? a.scale[r] : 1.f;
+        float* __restrict__ orow = a.out + r * a.ld_out;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m0 = mt * 16 + 4 * j;
+            if (m0 >= a.out_cols) continue;
+            float y[4] = {acc[mt][0] * s, acc[mt][1] * s, acc[mt][2] * s, acc[mt][3] * s};
+            if (a.relu_ref) {
+                const float* __restrict__ ref = a.relu_ref + r * a.ld_ref;
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (m0 + v < a.M && !(ref[m0 + v] > 0.f)) y[v] = 0.f;
+            }
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (m0 + v >= a.M) y[v] = 0.f;        // padding columns hold exact zeros
+            if (a.vec_store && m0 + 4 <= a.out_cols) {
+                *reinterpret_cast<float4*>(orow + m0) = make_float4(y[0], y[1], y[2], y[3]);
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (m0 + v < a.out_cols) orow[m0 + v] = y[v];
+            }
+        }
+    }
+}
+
+template <int VW, int MT>
+static hipError_t launch_rows_cu(const RowsArgs& a, int cu, unsigned blocks, size_t lds, hipStream_t stream)
+{
+    if (cu == 4) hipLaunchKernelGGL((dense_rows_kernel<VW, MT, 4>), dim3(blocks), dim3(kUpdateThreads), lds, stream, a);
+    else if (cu == 2) hipLaunchKernelGGL((dense_rows_kernel<VW, MT, 2>), dim3(blocks), dim3(kUpdateThreads), lds, stream, a);
+    else hipLaunchKernelGGL((dense_rows_kernel<VW, MT, 1>), dim3(blocks), dim3(kUpdateThreads), lds, stream, a);
+    return hipGetLastError();
+}
+
+template <int VW>
+static hipError_t launch_rows_mt(const RowsArgs& a, int mt, int cu, unsigned blocks, size_t lds, hipStream_t stream)
+{
+    switch (mt) {
+        case 1: return launch_rows_cu<VW, 1>(a, cu, blocks, lds, stream);
+        case 2: return launch_rows_cu<VW, 2>(a, cu, blocks, lds, stream);
+        case 4: return launch_rows_cu<VW, 4>(a, cu, blocks, lds, stream);
+        default: return launch_rows_cu<VW, 8>(a, cu, blocks, lds, stream);
+    }
+}
+
+// out[r, 0:out_cols] = scale[r] * (act(X[r, 0:K]) * Wop)[0:M] (zero beyond M), optionally masked by
+// relu_ref.  Wop(k, m) = w[k*sk + m*sm].  Returns kErrInvalidArgument when K is too large for the
+// operand to fit the LDS (the caller then has to use a general GEMM).
+int launch_dense_rows(float* out, int ld_out, int out_cols, const float* x, int ld_x, const float* w, long long sk,
+                      long long sm, const float* scale, const float* relu_ref, int ld_ref, int relu_in,
+                      long long n, int K, int M, hipStream_t stream)
+{
+    if (n == 0 || out_cols == 0) return kOk;
+    const uintptr_t xa = reinterpret_cast<uintptr_t>(x);
+    const int vw = (ld_x % 4 == 0 && xa % 16 == 0) ? 4 : (ld_x % 2 == 0 && xa % 8 == 0) ? 2 : 1;
+    const int chunks = (K + 4 * vw - 1) / (4 * vw);
+    const int cu = chunks >= 3 ? 4 : chunks;
+    const int chunks_p = (chunks + cu - 1) / cu * cu;
+    const size_t lds_per_tile = static_cast<size_t>(chunks_p) * kWave * vw * sizeof(float);
+    if (lds_per_tile > kMaxOperandLds) {
+        set_error("dense update: inner dimension too large for the on-chip operand buffer");
+        return kErrInvalidArgument;
+    }
+    int mt_cap = 8;                                     // 16-column tiles one launch covers
+    while (mt_cap > 1 && lds_per_tile * mt_cap > kMaxOperandLds) mt_cap /= 2;
+    const long long tiles = (n + kTileRows - 1) / kTileRows;
+    long long blocks = (tiles + kUpdateWaves - 1) / kUpdateWaves;
+    if (blocks > 256 * 8) blocks = 256 * 8;
+    for (int c0 = 0; c0 < out_cols; c0 += 16 * mt_cap) {
+        const int cols = out_cols - c0 < 16 * mt_cap ? out_cols - c0 : 16 * mt_cap;
+        int mt = 1;
+        while (16 * mt < cols) mt *= 2;
+        RowsArgs a;
+        a.out = out + c0;
+        a.x = x;
+        a.w = w + c0 * sm;
+        a.scale = scale;
+        a.relu_ref = relu_ref ? relu_ref + c0 : nullptr;
+        a.n = n;
+        a.sk = sk;
+        a.sm = sm;
+        a.ld_out = ld_out;
+        a.out_cols = cols;
+        a.ld_x = ld_x;
+        a.ld_ref = ld_ref;
+        a.K = K;
+        a.M = M - c0 > 0 ? (M - c0 < cols ? M - c0 : cols) : 0;
+        a.relu_in = relu_in;
+        a.vec_store = (ld_out % 4 == 0 && reinterpret_cast<uintptr_t>(a.out) % 16 == 0) ? 1 : 0;
+        const size_t lds = lds_per_tile * mt;
+        hipError_t e;
+        if (vw == 4) e = launch_rows_mt<4>(a, mt, cu, static_cast<unsigned>(blocks), lds, stream);
+        else if (vw == 2) e = launch_rows_mt<2>(a, mt, cu, static_cast<unsigned>(blocks), lds, stream);
+        else e = launch_rows_mt<1>(a, mt, cu, static_cast<unsigned>(blocks), lds, stream);
+        if (e != hipSuccess) return hip_fail(e, "dense rows kernel launch");
+    }
+    return kOk;
+}
+
+// ---------------------------------------------------------------- weight kernel
+// partial[blockIdx.x][k][d] = sum over the block's rows of act(X[r, k]) * G[r, d]
+template <int KTB, int DT>
+__global__ __launch_bounds__(kUpdateThreads) void dense_weight_kernel(float* __restrict__ partial,
+                                                                      const float* __restrict__ x, int ld_x,
+                                                                      const float* __restrict__ g, int ld_g,
+                                                                      int relu_in, long long n, int K, int D,
+                                                                      long long rows_per_wave)
+{
+    __shared__ float red[kUpdateWaves][KTB * DT * 4 * kWave];
+    const int lane = lane_id();
+    const int wave = threadIdx.x / kWave;
+    const int i = lane % 16, j = lane / 16;
+    const int k0 = blockIdx.y * KTB * 16;
+    floatx4 acc[KTB][DT];
+#pragma unroll
+    for (int kt = 0; kt < KTB; ++kt)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[kt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const long long wave_id = static_cast<long long>(blockIdx.x) * kUpdateWaves + wave;
+    const long long r_begin = wave_id * rows_per_wave;
+    long long r_end = r_begin + rows_per_wave;
+    if (r_end > n) r_end = n;
+    for (long long r0 = r_begin; r0 < r_end; r0 += 16) {
+        float av[4][KTB], bv[4][DT];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const long long row = r0 + 4 * s + j;
+            const bool ok = row < r_end;
+            const float* __restrict__ xr = x + (ok ? row : r_begin) * ld_x;
+            const float* __restrict__ gr = g + (ok ? row : r_begin) * ld_g;
+#pragma unroll
+            for (int kt = 0; kt < KTB; ++kt) {
+                const int k = k0 + kt * 16 + i;
+                float t = (ok && k < K) ? xr[k] : 0.f;
+                av[s][kt] = relu_in ? fmaxf(t, 0.f) : t;
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int d = dt * 16 + i;
+                bv[s][dt] = (ok && d < D) ? gr[d] : 0.f;
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int kt = 0; kt < KTB; ++kt)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) acc[kt][dt] = mfma16(av[s][kt], bv[s][dt], acc[kt][dt]);
+    }
+
+#pragma unroll
+    for (int kt = 0; kt < KTB; ++kt)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[wave][((kt * DT + dt) * 4 + v) * kWave + lane] = acc[kt][dt][v];
+    __syncthreads();
+    float* __restrict__ mine = partial + static_cast<size_t>(blockIdx.x) * K * D;
+    for (int e = threadIdx.x; e < KTB * DT * 4 * kWave; e += kUpdateThreads) {
+        float sum = red[0][e];
+#pragma unroll
+        for (int w = 1; w < kUpdateWaves; ++w) sum += red[w][e];
+        const int l = e % kWave;
+        const int v = (e / kWave) % 4;
+        const int dt = (e / (4 * kWave)) % DT;
+        const int kt = e / (4 * kWave * DT);
+        const int k = k0 + kt * 16 + 4 * (l / 16) + v;
+        const int d = dt * 16 + l % 16;
+        if (k < K && d < D) mine[static_cast<size_t>(k) * D + d] = sum;
+    }
+}
+
+// dw[e] = sum over blocks of partial[b][e], added in a fixed order
+__global__ __launch_bounds__(256) void reduce_partials_kernel(float* __restrict__ dw,
+                                                              const float* __restrict__ partial, int num_blocks,
+                                                              int count)
+{
+    __shared__ float red[4][64];
+    const int e = blockIdx.x * 64 + threadIdx.x % 64;
+    const int slice = threadIdx.x / 64;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (e < count) {
+        int b = slice;
+        for (; b + 12 < num_blocks; b += 16) {
+            s0 += partial[static_cast<size_t>(b) * count + e];
+            s1 += partial[static_cast<size_t>(b + 4) * count + e];
+            s2 += partial[static_cast<size_t>(b + 8) * count + e];
+            s3 += partial[static_cast<size_t>(b + 12) * count + e];
+        }
+        for (; b < num_blocks; b += 4) s0 += partial[static_cast<size_t>(b) * count + e];
+    }
+    red[slice][threadIdx.x % 64] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (slice == 0 && e < count) dw[e] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+}
+
+static int weight_blocks(long long n)
+{
+    long long b = (n + 63) / 64;                         // at least 16 rows per wave
+    if (b > kMaxWeightBlocks) b = kMaxWeightBlocks;
+    return static_cast<int>(b < 1 ? 1 : b);
+}
+
+size_t update_workspace_bytes(long long n, int K, int D)
+{
+    if (n <= 0 || K <= 0 || D <= 0) return 0;
+    return static_cast<size_t>(weight_blocks(n)) * K * D * sizeof(float);
+}
+
+template <int KTB, int DT>
+static hipError_t launch_weight(float* partial, const float* x, int ld_x, const float* g, int ld_g, int relu_in,
+                                long long n, int K, int D, long long rows_per_wave, int blocks, hipStream_t stream)
+{
+    const int ktiles = (K + 15) / 16;
+    hipLaunchKernelGGL((dense_weight_kernel<KTB, DT>), dim3(blocks, (ktiles + KTB - 1) / KTB), dim3(kUpdateThreads), 0,
+                       stream, partial, x, ld_x, g, ld_g, relu_in, n, K, D, rows_per_wave);
+    return hipGetLastError();
+}
+
+// dw[K, D] = act(X[N, K])^T * G[N, D]; D <= 64.
+int launch_dense_weight(float* dw, const float* x, int ld_x, const float* g, int ld_g, int relu_in, long long n,
+                        int K, int D, void* workspace, hipStream_t stream)
+{
+    if (K == 0 || D == 0) return kOk;
+    if (n == 0) {
+        EPPGCN_HIP(hipMemsetAsync(dw, 0, static_cast<size_t>(K) * D * sizeof(float), stream));
+        return kOk;
+    }
+    if (D > 64) {
+        set_error("dense update: more than 64 gradient columns are not supported by the weight kernel");
+        return kErrInvalidArgument;
+    }
+    const int blocks = weight_blocks(n);
+    const long long waves = static_cast<long long>(blocks) * kUpdateWaves;
+    const long long rows_per_wave = ((n + waves - 1) / waves + 15) / 16 * 16;
+    float* partial = static_cast<float*>(workspace);
+    const int dt = D <= 16 ? 1 : D <= 32 ? 2 : 4;
+    const int ktiles = (K + 15) / 16;
+    int ktb = 8 / dt;
+    while (ktb > 1 && ktb / 2 >= ktiles) ktb /= 2;
+    hipError_t e;
+#define EPPGCN_W(KTB_, DT_) launch_weight<KTB_, DT_>(partial, x, ld_x, g, ld_g, relu_in, n, K, D, rows_per_wave, blocks, stream)
+    if (dt == 1) e = ktb == 8 ? EPPGCN_W(8, 1) : ktb == 4 ? EPPGCN_W(4, 1) : ktb == 2 ? EPPGCN_W(2, 1) : EPPGCN_W(1, 1);
+    else if (dt == 2) e = ktb == 4 ? EPPGCN_W(4, 2) : ktb == 2 ? EPPGCN_W(2, 2) : EPPGCN_W(1, 2);
+    else e = ktb == 2 ? EPPGCN_W(2, 4) : EPPGCN_W(1, 4);
+#undef EPPGCN_W
+    if (e != hipSuccess) return hip_fail(e, "dense weight kernel launch");
+    const int count = K * D;
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3((count + 63) / 64), dim3(256), 0, stream, dw, partial, blocks, count);
+    EPPGCN_HIP(hipGetLastError());
+    return kOk;
+}
+
+}  // namespace eppgcn

@@ -43,14 +43,21 @@ class GraphDataset:
 
 
 class Net(torch.nn.Module):
-    def __init__(self, dataset: GraphDataset, hidden: int, num_layers: int, weight_seed: int = None):
+    """The reference's model (EPPGCN/gcn_main.py:190-208): conv -> relu -> ... -> conv.  With
+    ``fuse_relu`` (default) the activation between two layers is applied by the consuming layer
+    while it loads its input instead of by a separate F.relu pass; the function computed is the
+    same."""
+
+    def __init__(self, dataset: GraphDataset, hidden: int, num_layers: int, weight_seed: int = None,
+                 fuse_relu: bool = True):
         super().__init__()
         self.num_layers = num_layers
+        self.fuse_relu = fuse_relu
         self.convs = torch.nn.ModuleList()
         for i in range(num_layers):
             fan_in = hidden if i != 0 else dataset.num_features
             fan_out = hidden if i < num_layers - 1 else dataset.num_classes
-            conv = GCNConv(fan_in, fan_out)
+            conv = GCNConv(fan_in, fan_out, relu_input=fuse_relu and i != 0)
             if weight_seed is not None:
                 with torch.no_grad():
                     conv.weights.copy_(graphs.uniform_weights(weight_seed + i, fan_in, fan_out))
@@ -60,7 +67,7 @@ class Net(torch.nn.Module):
         for i in range(self.num_layers):
             info = inputInfo.set_input() if i == 0 else inputInfo.set_hidden()
             x = self.convs[i](x, info, mask_props[i], back_props[i], isFirstIter, isBackModeNet)
-            if i < self.num_layers - 1:
+            if i < self.num_layers - 1 and not self.fuse_relu:
                 x = F.relu(x)
         return x
 
@@ -69,7 +76,8 @@ class Trainer:
     """Wiring of EPPGCN/gcn_main.py: decider -> build_part -> mask/back records -> Net -> Adam."""
 
     def __init__(self, graph: graphs.Graph, dim=96, hidden=16, num_classes=22, num_layers=2, train_ratio=0.1,
-                 train_mask=None, backsize_mode="constant", backsize=32, labels="ones", weight_seed=3, lr=0.01):
+                 train_mask=None, backsize_mode="constant", backsize=32, labels="ones", weight_seed=3, lr=0.01,
+                 fuse_relu=True):
         self.GNNA = gnnadvisor()
         self.backsize_mode, self.backsize = backsize_mode, backsize
         self.dataset = ds = GraphDataset(graph, dim, num_classes, num_layers, train_mask, train_ratio, labels)
@@ -89,7 +97,7 @@ class Trainer:
             self.mask_props.append(maskInputProperty(src, dst, ds.edge_masks[num_layers - 1 - i],
                                                      ds.node_degs[num_layers - 1 - i], num_layers, i + 1, width))
             self.back_props.append(backInputProperty(degrees=ds.degrees, dim=width, layer=i + 1))
-        self.model = Net(ds, hidden, num_layers, weight_seed).to(ds.x.device)
+        self.model = Net(ds, hidden, num_layers, weight_seed, fuse_relu).to(ds.x.device)
         self.optimizer = torch.optim.Adam(self.model.parameters(), lr=lr)
         self.for_time = self.loss_time = self.back_time = self.build_time = 0.0
         self.losses: List[float] = []

@@ -30,8 +30,12 @@
  *     request per edge; with NULL the kernel gathers the
  *     neighbour's scale per edge and needs no scratch.  The workspace may be the
  *     input pointer itself when the caller no longer needs the unscaled input
- *     (it is then overwritten with degrees[r]*in[r,:], unpadded).  Results of the
- *     modes agree to rounding (a few ulp per term).
+ *     (it is then overwritten with degrees[r]*in[r,:], unpadded).  With a NULL
+ *     input and a workspace, the workspace must already hold the scaled rows
+ *     degrees[r]*in[r,:] at a pitch of eppgcn_feature_workspace_pitch(dim) floats
+ *     with zeros in the padding (eppgcn_update_forward writes exactly that) and
+ *     the scaling pass is skipped.  Results of the modes agree to rounding (a few
+ *     ulp per term).
  */
 #ifndef EPPGCN_HIP_H_
 #define EPPGCN_HIP_H_
@@ -60,6 +64,8 @@ int eppgcn_abi_version(void);
 
 /* Floats a separate feature workspace must hold for [num_nodes, dim] features. */
 size_t eppgcn_feature_workspace_floats(int64_t num_nodes, int dim);
+/* Row pitch (floats) of that workspace. */
+int eppgcn_feature_workspace_pitch(int dim);
 
 /* Execution plan for the aggregation kernels: a copy of the groups (pointers, rows, adjacency
  * flags, column ids) re-ordered by the column block (2^shift vertices, shift chosen from `dim`;
@@ -192,6 +198,43 @@ int eppgcn_build_part(const int32_t* row_pointers, int num_nodes, int part_size,
  * on the host; d_hist: ten device ints of scratch.  Synchronises. */
 int eppgcn_get_ginfo(const int32_t* node_deg, int64_t num_nodes, int64_t valid_len,
                      int32_t* d_hist, float* h_out, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Dense update of a layer: the matrix products the reference computes with torch::mm around
+ * the aggregation, for tall-and-skinny shapes (num_nodes rows, tens of columns), on the fp32
+ * matrix cores.  All matrices are fp32 row-major and contiguous unless a pitch is given.
+ * A call fails with EPPGCN_ERR_INVALID_ARGUMENT (and a message) for shapes outside what the
+ * kernels cover (reduction length beyond 1024, more than 64 gradient columns for the weight
+ * gradient); callers then use a general GEMM.
+ * ------------------------------------------------------------------------- */
+
+/* Bit mask of the update functions that cover [*, in_dim] x [in_dim, out_dim] layers:
+ * 1 eppgcn_update_forward, 2 eppgcn_update_backward_input, 4 eppgcn_update_backward_weight. */
+int eppgcn_update_supported(int in_dim, int out_dim);
+
+/* out[r, 0:out_dim] = scale[r] * act(x[r, :]) * w, columns out_dim..ld_out-1 = 0.
+ * x [num_nodes, in_dim], w [in_dim, out_dim], out rows ld_out floats apart; scale may be NULL
+ * (factor 1); relu_input != 0 applies max(x, 0) on load.  With scale = degrees and
+ * ld_out = eppgcn_feature_workspace_pitch(out_dim) the result is the pre-scaled feature
+ * workspace the aggregation functions accept with a NULL input.
+ * Replaces `tmp = torch::mm(input, weight)`, EPPGCN_kernel.cu:142 (spmm_forward_cuda). */
+int eppgcn_update_forward(float* out, int ld_out, const float* x, const float* w, const float* scale,
+                          int relu_input, int64_t num_nodes, int in_dim, int out_dim, void* stream);
+
+/* d_x[num_nodes, in_dim] = g[num_nodes, out_dim] * w^T, w [in_dim, out_dim]; with relu_ref
+ * ([num_nodes, in_dim], may be NULL) entries where relu_ref <= 0 are zeroed (gradient of a
+ * ReLU applied to the layer input).
+ * Replaces `d_input = torch::mm(d_input_prime, W.transpose(0,1))`, EPPGCN_kernel.cu:461,614. */
+int eppgcn_update_backward_input(float* d_x, const float* g, const float* w, const float* relu_ref,
+                                 int64_t num_nodes, int in_dim, int out_dim, void* stream);
+
+/* d_w[in_dim, out_dim] = act(x)^T * g, x [num_nodes, in_dim], g [num_nodes, out_dim], out_dim <= 64.
+ * Sums are formed in a fixed order (bitwise reproducible).  workspace: at least
+ * eppgcn_update_workspace_bytes(num_nodes, in_dim, out_dim) bytes, 4-byte aligned.
+ * Replaces `d_weight = torch::mm(X.transpose(0,1), d_input_prime)`, EPPGCN_kernel.cu:462,615. */
+size_t eppgcn_update_workspace_bytes(int64_t num_nodes, int in_dim, int out_dim);
+int eppgcn_update_backward_weight(float* d_w, const float* x, const float* g, int relu_input, int64_t num_nodes,
+                                  int in_dim, int out_dim, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Timers (print_time / clear_time, EPPGCN_kernel.cu:89-116; EPPGCN.cpp:394-395).

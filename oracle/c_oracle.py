@@ -62,6 +62,12 @@ def load():
     lib.oracle_threshold_back_part_size.argtypes = [C.c_int, C.c_int]
     lib.oracle_get_ginfo.restype = None
     lib.oracle_get_ginfo.argtypes = [_i32p, C.c_int, C.c_int, _f32p]
+    lib.oracle_update_forward.restype = None
+    lib.oracle_update_forward.argtypes = [_f32p, C.c_int, _f32p, _f32p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_int]
+    lib.oracle_update_backward_input.restype = None
+    lib.oracle_update_backward_input.argtypes = [_f32p, _f32p, _f32p, C.c_void_p, C.c_int64, C.c_int, C.c_int]
+    lib.oracle_update_backward_weight.restype = None
+    lib.oracle_update_backward_weight.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int64, C.c_int, C.c_int]
     lib.oracle_num_threads.restype = C.c_int
     _lib = lib
     return lib
@@ -182,3 +188,39 @@ def get_ginfo(node_deg, valid_len: int):
     re = np.zeros(10, np.float32)
     load().oracle_get_ginfo(node_deg, node_deg.size, valid_len, re)
     return re
+
+
+def update_forward(x, w, scale=None, relu_input: bool = False, ld_out: int = None):
+    """scale[r] * act(x) @ w with rows ld_out floats apart (zero padded) -> float32 [N, ld_out]."""
+    lib = load()
+    x, w = _f32(x), _f32(w)
+    n, k = x.shape
+    m = w.shape[1]
+    ld = ld_out or m
+    out = np.empty((n, ld), np.float32)
+    sc = _f32(scale) if scale is not None else None
+    lib.oracle_update_forward(out, ld, x, w, sc.ctypes.data if sc is not None else None, int(relu_input), n, k, m)
+    return out
+
+
+def update_backward_input(g, w, relu_ref=None):
+    """(g @ w.T) masked where relu_ref <= 0 -> float32 [N, in_dim]."""
+    lib = load()
+    g, w = _f32(g), _f32(w)
+    n, m = g.shape
+    k = w.shape[0]
+    d_x = np.empty((n, k), np.float32)
+    ref = _f32(relu_ref) if relu_ref is not None else None
+    lib.oracle_update_backward_input(d_x, g, w, ref.ctypes.data if ref is not None else None, n, k, m)
+    return d_x
+
+
+def update_backward_weight(x, g, relu_input: bool = False):
+    """act(x).T @ g -> float32 [in_dim, out_dim]."""
+    lib = load()
+    x, g = _f32(x), _f32(g)
+    n, k = x.shape
+    m = g.shape[1]
+    d_w = np.empty((k, m), np.float32)
+    lib.oracle_update_backward_weight(d_w, x, g, int(relu_input), n, k, m)
+    return d_w

@@ -365,6 +365,69 @@ void oracle_get_ginfo(const int32_t *node_deg, int num_nodes, int valid_len, flo
     for (int i = 3; i < 10; i++) re[i] = (float)(ginfo[i] * 1.0 / valid_node);
 }
 
+/* ------------------------------------------------------------------------
+ * Dense update of a layer: the three torch::mm calls around the aggregation.
+ *   tmp      = mm(input, weight)                EPPGCN/GCNConv/EPPGCN_kernel.cu:142
+ *   d_input  = mm(d_input_prime, W^T)           EPPGCN/GCNConv/EPPGCN_kernel.cu:461,614
+ *   d_weight = mm(X^T, d_input_prime)           EPPGCN/GCNConv/EPPGCN_kernel.cu:462,615
+ * torch::mm leaves the order of the fp32 additions to the BLAS behind it, so
+ * the restatement accumulates every dot product in double and rounds once;
+ * comparisons carry the fp32 tolerance.  The optional pieces the HIP kernels
+ * fuse are restated as the reference's driver composes them: relu on the layer
+ * input (F.relu between the layers, EPPGCN/gcn_main.py:203-205), its gradient
+ * mask, and the per-row factor of the aggregation weights (applied here to the
+ * product so that the aggregation can gather scaled rows).
+ * ---------------------------------------------------------------------- */
+void oracle_update_forward(float *out, int ld_out, const float *x, const float *w, const float *scale,
+                           int relu_input, int64_t num_nodes, int in_dim, int out_dim)
+{
+    for (int64_t r = 0; r < num_nodes; r++) {
+        for (int m = 0; m < ld_out; m++) {
+            double acc = 0.0;
+            if (m < out_dim) {
+                for (int k = 0; k < in_dim; k++) {
+                    float xv = x[r * in_dim + k];
+                    if (relu_input && !(xv > 0.f)) xv = 0.f;
+                    acc += (double)xv * (double)w[(int64_t)k * out_dim + m];
+                }
+                if (scale) acc = (double)(float)acc * (double)scale[r];
+            }
+            out[r * ld_out + m] = (float)acc;
+        }
+    }
+}
+
+void oracle_update_backward_input(float *d_x, const float *g, const float *w, const float *relu_ref,
+                                  int64_t num_nodes, int in_dim, int out_dim)
+{
+    for (int64_t r = 0; r < num_nodes; r++) {
+        for (int k = 0; k < in_dim; k++) {
+            double acc = 0.0;
+            for (int d = 0; d < out_dim; d++)
+                acc += (double)g[r * out_dim + d] * (double)w[(int64_t)k * out_dim + d];
+            if (relu_ref && !(relu_ref[r * in_dim + k] > 0.f)) acc = 0.0;
+            d_x[r * in_dim + k] = (float)acc;
+        }
+    }
+}
+
+void oracle_update_backward_weight(float *d_w, const float *x, const float *g, int relu_input,
+                                   int64_t num_nodes, int in_dim, int out_dim)
+{
+    double *acc = (double *)calloc((size_t)in_dim * out_dim, sizeof(double));
+    for (int64_t r = 0; r < num_nodes; r++) {
+        for (int k = 0; k < in_dim; k++) {
+            float xv = x[r * in_dim + k];
+            if (relu_input && !(xv > 0.f)) xv = 0.f;
+            if (xv == 0.f) continue;
+            for (int d = 0; d < out_dim; d++)
+                acc[(size_t)k * out_dim + d] += (double)xv * (double)g[r * out_dim + d];
+        }
+    }
+    for (size_t e = 0; e < (size_t)in_dim * out_dim; e++) d_w[e] = (float)acc[e];
+    free(acc);
+}
+
 int oracle_num_threads(void)
 {
 #ifdef _OPENMP

@@ -209,3 +209,54 @@ def test_print_time_lines(GNNA, capfd):
     out = capfd.readouterr().out
     for key in ("for_agg_time:", "back_agg_time:", "l1_back_agg_time:", "l2_back_agg_time:", "mask_time:"):
         assert key in out
+
+
+@pytest.mark.parametrize("fuse_relu", [True, False])
+@pytest.mark.parametrize("dense", [0, -1])
+def test_gradients_with_fused_relu_and_with_torch_products(GNNA, fuse_relu, dense):
+    """The activation applied inside the consuming layer's product, and the library's own dense
+    products versus torch::mm (dense = -1), all give the float64 dense model's gradients."""
+    from eppgcn_amd import graphs, train
+    GNNA.set_dense_policy(dense)
+    try:
+        indptr, col = random_symmetric_csr(700, 2500, 8)
+        n = indptr.size - 1
+        g = graphs.Graph("t", n, dev(indptr), dev(col), dev(scale_inv_sqrt(indptr)))
+        mask = np.random.default_rng(2).random(n) < 0.2
+        tr = train.Trainer(g, dim=24, hidden=16, num_classes=22, train_mask=torch.from_numpy(mask), backsize=4,
+                           labels="uniform", fuse_relu=fuse_relu)
+        x, y = tr.dataset.x.cpu().numpy(), tr.dataset.y.cpu().numpy()
+        w0 = tr.model.convs[0].weights.detach().cpu().numpy()
+        w1 = tr.model.convs[1].weights.detach().cpu().numpy()
+        want_loss, want_g0, want_g1 = _dense_model_grads(indptr, col, scale_inv_sqrt(indptr), x, w0, w1, mask, y)
+        tr.optimizer = torch.optim.SGD(tr.model.parameters(), lr=0.0)
+        loss = tr.train_step(True)
+        assert abs(float(loss) - want_loss) < 1e-5 * max(1.0, abs(want_loss))
+        g0 = tr.model.convs[0].weights.grad.cpu().numpy()
+        g1 = tr.model.convs[1].weights.grad.cpu().numpy()
+        assert np.linalg.norm(g0 - want_g0) / np.linalg.norm(want_g0) < 1e-4
+        assert np.linalg.norm(g1 - want_g1) / np.linalg.norm(want_g1) < 1e-4
+    finally:
+        GNNA.set_dense_policy(0)
+
+
+def test_keyword_additions_of_the_layer_ops(GNNA):
+    """relu_input and need_dx, the two keyword arguments this build adds to the reference's calls."""
+    indptr, col = random_symmetric_csr(900, 4000, 17)
+    n = indptr.size - 1
+    s = scale_inv_sqrt(indptr)
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((n, 16)).astype(np.float32)
+    w = rng.uniform(-0.3, 0.3, (16, 22)).astype(np.float32)
+    dy = rng.standard_normal((n, 22)).astype(np.float32)
+    pp, p2n = GNNA.build_part(6, dev(indptr))
+    args = (dev(indptr), dev(col), dev(s), pp.int(), p2n.int(), 6, 32, 8)
+    plain = GNNA.forward(torch.relu(dev(x)), dev(w), *args)[0]
+    fused = GNNA.forward(dev(x), dev(w), *args, relu_input=True)[0]
+    assert torch.allclose(plain, fused, rtol=1e-5, atol=1e-6)
+    dx, dw = GNNA.backward(dev(dy), torch.relu(dev(x)), dev(w), *args)
+    dx_f, dw_f = GNNA.backward(dev(dy), dev(x), dev(w), *args, relu_input=True)
+    assert torch.allclose(dw, dw_f, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(dx * (dev(x) > 0), dx_f, rtol=1e-5, atol=1e-6)
+    none, dw_only = GNNA.backward(dev(dy), dev(x), dev(w), *args, need_dx=False, relu_input=True)
+    assert none.numel() == 0 and torch.equal(dw_only, dw_f)

@@ -1,0 +1,129 @@
+"""GPU parity of the dense layer update (X*W, G*W^T, X^T*G on the matrix cores) through the
+C ABI against the CPU checker.  fp32 bar: |got - want| <= 1e-5 * sum_k |a_k b_k| per output
+element (the checker accumulates in float64, so only summation order and product rounding of
+the fp32 kernel remain)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from tests.helpers import random_symmetric_csr, scale_inv_sqrt
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def api():
+    from eppgcn_amd import capi
+    capi.load()
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return capi
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def assert_close(got, want, bound, what=""):
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    lim = RTOL * bound + 1e-30
+    worst = float(np.max(err / lim)) if err.size else 0.0
+    assert worst <= 1.0, f"{what}: max err/limit = {worst:.3f}"
+
+
+def data(n, k, m, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((n, k)).astype(np.float32)
+    w = rng.uniform(-0.5, 0.5, (k, m)).astype(np.float32)
+    g = rng.standard_normal((n, m)).astype(np.float32)
+    s = rng.uniform(0.1, 2.0, n).astype(np.float32)
+    return x, w, g, s
+
+
+# rows x reduction length x output columns: tile edges (16 rows, 16 columns, 4*VW reduction
+# steps), odd sizes (scalar loads), the benchmark's layer shapes, column slabs (> 128 columns)
+SHAPES = [(1, 1, 1), (5, 3, 2), (16, 16, 16), (17, 96, 16), (1000, 16, 22), (1000, 22, 16), (4097, 96, 16),
+          (300, 33, 40), (123, 130, 70), (64, 8, 150), (50, 257, 5), (40000, 96, 16)]
+
+
+@pytest.mark.parametrize("n,k,m", SHAPES)
+@pytest.mark.parametrize("relu", [False, True])
+def test_update_forward_matches_checker(api, n, k, m, relu):
+    x, w, _, s = data(n, k, m, 1)
+    xa = np.maximum(x, 0) if relu else x
+    bound = np.abs(xa).astype(np.float64) @ np.abs(w).astype(np.float64)
+    got = api.update_forward(dev(x), dev(w), relu_input=relu).cpu().numpy()
+    assert_close(got, co.update_forward(x, w, relu_input=relu), bound, "plain product")
+    ld = api.feature_workspace_pitch(m)
+    got = api.update_forward(dev(x), dev(w), scale=dev(s), relu_input=relu, ld_out=ld).cpu().numpy()
+    assert got.shape == (n, ld) and not got[:, m:].any()
+    assert_close(got[:, :m], co.update_forward(x, w, scale=s, relu_input=relu), bound * s[:, None], "scaled, padded")
+
+
+@pytest.mark.parametrize("n,k,m", SHAPES)
+def test_update_backward_input_matches_checker(api, n, k, m):
+    x, w, g, _ = data(n, k, m, 2)
+    bound = np.abs(g).astype(np.float64) @ np.abs(w).astype(np.float64).T
+    got = api.update_backward_input(dev(g), dev(w)).cpu().numpy()
+    assert_close(got, co.update_backward_input(g, w), bound, "no mask")
+    got = api.update_backward_input(dev(g), dev(w), relu_ref=dev(x)).cpu().numpy()
+    assert_close(got, co.update_backward_input(g, w, relu_ref=x), bound, "relu mask")
+    assert not got[x <= 0].any()
+
+
+@pytest.mark.parametrize("n,k,m", [(1, 1, 1), (5, 3, 2), (63, 16, 16), (1000, 16, 22), (1000, 22, 16),
+                                   (4097, 96, 16), (300, 33, 40), (123, 130, 64), (70000, 96, 16), (300000, 16, 22)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_update_backward_weight_matches_checker(api, n, k, m, relu):
+    x, _, g, _ = data(n, k, m, 3)
+    xa = np.maximum(x, 0) if relu else x
+    bound = np.abs(xa).astype(np.float64).T @ np.abs(g).astype(np.float64)
+    a = api.update_backward_weight(dev(x), dev(g), relu_input=relu)
+    b = api.update_backward_weight(dev(x), dev(g), relu_input=relu)
+    assert torch.equal(a, b), "the weight gradient must be bitwise reproducible"
+    assert_close(a.cpu().numpy(), co.update_backward_weight(x, g, relu_input=relu), bound, "weight gradient")
+
+
+def test_update_handles_unaligned_views(api):
+    """Operands that start 4 bytes into an allocation take the narrower load paths."""
+    n, k, m = 777, 22, 16
+    x, w, g, _ = data(n, k, m, 4)
+    flat = torch.empty(n * k + 1, dtype=torch.float32, device="cuda")
+    xv = flat[1:].view(n, k)
+    xv.copy_(dev(x))
+    bound = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64)
+    assert_close(api.update_forward(xv, dev(w)).cpu().numpy(), co.update_forward(x, w), bound, "forward")
+    bw = np.abs(x).astype(np.float64).T @ np.abs(g).astype(np.float64)
+    assert_close(api.update_backward_weight(xv, dev(g)).cpu().numpy(), co.update_backward_weight(x, g), bw, "weight")
+
+
+def test_update_rejects_unsupported_shapes(api):
+    x = torch.zeros((4, 5000), device="cuda")
+    w = torch.zeros((5000, 3), device="cuda")
+    with pytest.raises(api.EppgcnError, match="inner dimension"):
+        api.update_forward(x, w)
+    with pytest.raises(api.EppgcnError, match="64 gradient columns"):
+        api.update_backward_weight(torch.zeros((4, 3), device="cuda"), torch.zeros((4, 65), device="cuda"))
+    with pytest.raises(api.EppgcnError):
+        api.update_forward(torch.zeros((4, 3), device="cuda"), torch.zeros((4, 3), device="cuda"))
+
+
+@pytest.mark.parametrize("dim", [16, 22, 7, 40])
+def test_aggregation_accepts_the_prescaled_product(api, dim):
+    """update_forward(scale=degrees, pitch of the workspace) followed by the aggregation with a
+    NULL input equals the aggregation of the unscaled product."""
+    indptr, col = random_symmetric_csr(5000, 30000, 21)
+    n = indptr.size - 1
+    s = scale_inv_sqrt(indptr)
+    x, w, _, _ = data(n, 24, dim, 6)
+    pp, p2n = api.build_part(8, dev(indptr), col.size)
+    ws = api.update_forward(dev(x), dev(w), scale=dev(s), ld_out=api.feature_workspace_pitch(dim))
+    got = api.spmm_forward(None, dev(col), dev(s), pp, p2n, part_size=8, workspace=ws.view(-1), prescaled_dim=dim)
+    t = co.update_forward(x, w)
+    want = co.spmm_f64(t, indptr, col, s)
+    bound = co.spmm_f64(np.abs(t), indptr, col, s) + 1e-30
+    # two fp32 stages: the product (relative to |x||w|) and the aggregation of its result
+    tb = (np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64)).astype(np.float32)
+    bound = bound + co.spmm_f64(tb, indptr, col, s)
+    assert_close(got.cpu().numpy(), want, bound, f"prescaled aggregation, width {dim}")
