@@ -32,49 +32,78 @@ __global__ void scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles)
 }
 
 // ================================================================ path marking
-// A team of TS lanes owns one forward group and strides over its slots.
-template <int TS>
-__global__ __launch_bounds__(256) void mask_forward_kernel(
+// A wave owns 64 consecutive forward groups (one per lane) and walks the contiguous slot range
+// they cover 64 slots at a time, so that the column ids are read and the edge marks written
+// with full-width coalesced accesses whatever the group lengths are.  The group (hence the
+// row) of a slot is found by a 6-step search over the 64 group starts kept in LDS.  Kept
+// slots are counted per group from the wave ballot, the counts of adjacent groups of one row
+// are added across lanes, and one atomic per (wave, row) updates node_degs.
+constexpr int kMaskBlock = 256;
+constexpr int kMaskWaves = kMaskBlock / kWave;
+
+__global__ __launch_bounds__(kMaskBlock) void mask_forward_kernel(
     const int* __restrict__ part2node, const int* __restrict__ part_ptr, const int* __restrict__ col,
     const uint8_t* __restrict__ src_mask, uint8_t* __restrict__ ngh_mask, int* __restrict__ back_edge_mask,
     int* __restrict__ node_degs, int num_parts, int is_last)
 {
-    constexpr int TPW = kWave / TS;
+    __shared__ int s_beg[kMaskWaves][kWave + 1];
     const int lane = threadIdx.x & (kWave - 1);
-    const int team = lane / TS;
-    const int tl = lane % TS;
-    const long long wave_global = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
-    const long long p = wave_global * TPW + team;
-    int beg = 0, end = 0, row = 0;
+    const int wave = threadIdx.x >> 6;
+    const long long g0 = (static_cast<long long>(blockIdx.x) * kMaskWaves + wave) * kWave;
+    if (g0 >= num_parts) return;                       // wave-uniform; the LDS rows are wave-private
+    const int ng = static_cast<int>(min(static_cast<long long>(kWave), num_parts - g0));
+
+    int beg = 0, end = 0, row = -1;
     bool row_in_src = false;
-    if (p < num_parts) {
-        beg = part_ptr[p];
-        end = part_ptr[p + 1];
-        row = part2node[p];
+    if (lane < ng) {
+        beg = part_ptr[g0 + lane];
+        end = part_ptr[g0 + lane + 1];
+        row = part2node[g0 + lane];
         row_in_src = !is_last && end > beg && src_mask[row] != 0;
+        if (row_in_src) ngh_mask[row] = 1;
     }
-    if (row_in_src && tl == 0) ngh_mask[row] = 1;
+    int* begs = s_beg[wave];
+    begs[lane] = lane < ng ? beg : 0x7fffffff;
+    if (lane == 0) begs[kWave] = 0x7fffffff;
+    __builtin_amdgcn_wave_barrier();
+    const int first = __shfl(beg, 0, kWave);
+    const int last = __shfl(end, ng - 1, kWave);
+
     int kept = 0;
-    // all lanes of the wave iterate together so that the ballot below is wave-uniform
-    const int span = end - beg;
-    int max_span = span;
+    for (int base = first; base < last; base += kWave) {
+        const int e = base + lane;
+        const bool in_range = e < last;
+        int owner = 0;
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) max_span = max(max_span, __shfl_xor(max_span, off, kWave));
-    for (int i = tl; i - tl < max_span; i += TS) {
-        const bool in_range = i < span;
+        for (int step = kWave / 2; step > 0; step >>= 1)
+            if (begs[owner + step] <= e) owner += step;          // last group starting at or before e
+        const int e_row = __shfl(row, owner, kWave);
+        const bool e_src = __shfl(static_cast<int>(row_in_src), owner, kWave) != 0;
         bool keep = false;
         if (in_range) {
-            const int e = beg + i;
             const int end_id = col[e];
             keep = src_mask[end_id] != 0;
-            if (keep) back_edge_mask[e] = row;
-            if (row_in_src) ngh_mask[end_id] = 1;
+            if (keep) back_edge_mask[e] = e_row;
+            if (e_src) ngh_mask[end_id] = 1;
         }
         const uint64_t ballot = __ballot(keep);
-        const uint64_t team_bits = (TS == 64) ? ballot : ((ballot >> (team * TS)) & ((1ull << (TS % 64)) - 1ull));
-        kept += __popcll(team_bits);
+        // this lane's group covers wave slots [lo, hi) of the current 64
+        const int lo = min(max(beg - base, 0), kWave);
+        const int hi = min(max(end - base, 0), kWave);
+        if (hi > lo) {
+            const uint64_t below_hi = hi == kWave ? ~0ull : (1ull << hi) - 1ull;
+            kept += __popcll(ballot & below_hi & ~((1ull << lo) - 1ull));
+        }
     }
-    if (tl == 0 && kept > 0) atomicAdd(node_degs + row, kept);
+    // groups of one row sit in adjacent lanes: suffix sums within a run of equal rows
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const int other = __shfl_down(kept, off, kWave);
+        const int other_row = __shfl_down(row, off, kWave);
+        if (lane + off < kWave && other_row == row) kept += other;
+    }
+    const int prev_row = __shfl_up(row, 1, kWave);
+    if (lane < ng && (lane == 0 || prev_row != row) && kept > 0) atomicAdd(node_degs + row, kept);
 }
 
 // ================================================================ compaction
@@ -315,23 +344,12 @@ int launch_mask_forward(const int* part2node, const int* part_ptr, const int* co
                         uint8_t* ngh_mask, int* back_edge_mask, int* node_degs, int num_parts,
                         long long num_edges, int is_last, hipStream_t stream)
 {
+    (void)num_edges;
     if (num_parts == 0) return kOk;
-    const double avg = static_cast<double>(num_edges) / num_parts;
-    int ts = 4;
-    while (ts < 64 && ts < avg) ts <<= 1;
-    const long long groups_per_block = (kWave / ts) * 4;
+    const long long groups_per_block = static_cast<long long>(kWave) * kMaskWaves;
     const unsigned grid = static_cast<unsigned>((num_parts + groups_per_block - 1) / groups_per_block);
-#define EPPGCN_MASK(TS_)                                                                                 \
-    hipLaunchKernelGGL((mask_forward_kernel<TS_>), dim3(grid), dim3(256), 0, stream, part2node, part_ptr, \
-                       col, src_mask, ngh_mask, back_edge_mask, node_degs, num_parts, is_last)
-    switch (ts) {
-        case 4: EPPGCN_MASK(4); break;
-        case 8: EPPGCN_MASK(8); break;
-        case 16: EPPGCN_MASK(16); break;
-        case 32: EPPGCN_MASK(32); break;
-        default: EPPGCN_MASK(64); break;
-    }
-#undef EPPGCN_MASK
+    hipLaunchKernelGGL(mask_forward_kernel, dim3(grid), dim3(kMaskBlock), 0, stream, part2node, part_ptr, col, src_mask,
+                       ngh_mask, back_edge_mask, node_degs, num_parts, is_last);
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }

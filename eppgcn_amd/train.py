@@ -101,6 +101,7 @@ class Trainer:
         self.optimizer = torch.optim.Adam(self.model.parameters(), lr=lr)
         self.for_time = self.loss_time = self.back_time = self.build_time = 0.0
         self.losses: List[float] = []
+        self.train_idx = self.train_y = None
 
     def build_back_part(self):
         """EPPGCN/gcn_main.py:151-168 ('net' mode, which needs an unpublished predictor, is not offered)."""
@@ -130,8 +131,13 @@ class Trainer:
             torch.cuda.synchronize()
             self.build_time += time.perf_counter() - t
         t = time.perf_counter()
-        logp = F.log_softmax(out, dim=1)
-        loss = F.nll_loss(logp[ds.train_mask], ds.y[ds.train_mask])
+        # EPPGCN/gcn_main.py:252-253 takes log_softmax of every row and then selects the training
+        # rows with the boolean mask (a device-to-host round trip per epoch); selecting the rows
+        # first, through indices computed once, is the same function of `out`
+        if self.train_idx is None:
+            self.train_idx = ds.train_mask.nonzero().squeeze(1)
+            self.train_y = ds.y[self.train_idx]
+        loss = F.nll_loss(F.log_softmax(out.index_select(0, self.train_idx), dim=1), self.train_y)
         torch.cuda.synchronize()
         self.loss_time += time.perf_counter() - t
         t = time.perf_counter()
