@@ -77,10 +77,17 @@ class Trainer:
 
     def __init__(self, graph: graphs.Graph, dim=96, hidden=16, num_classes=22, num_layers=2, train_ratio=0.1,
                  train_mask=None, backsize_mode="constant", backsize=32, labels="ones", weight_seed=3, lr=0.01,
-                 fuse_relu=True):
+                 fuse_relu=True, dataset=None):
+        """``dataset``: a loaded ``eppgcn_amd.dataset.custom_dataset`` (or any object with the same
+        attributes) to train on instead of synthetic features over ``graph``."""
         self.GNNA = gnnadvisor()
         self.backsize_mode, self.backsize = backsize_mode, backsize
-        self.dataset = ds = GraphDataset(graph, dim, num_classes, num_layers, train_mask, train_ratio, labels)
+        if dataset is not None:
+            ds = dataset
+            dim, num_classes, num_layers = ds.num_features, ds.num_classes, ds.num_layers
+        else:
+            ds = GraphDataset(graph, dim, num_classes, num_layers, train_mask, train_ratio, labels)
+        self.dataset = ds
         self.num_layers = num_layers
         info = inputProperty(ds.row_pointers, ds.column_index, ds.degrees, 32, 32, 8, 100, hiddenDim=hidden,
                              dataset_obj=ds, manual_mode=False)

@@ -260,3 +260,29 @@ def test_keyword_additions_of_the_layer_ops(GNNA):
     assert torch.allclose(dx * (dev(x) > 0), dx_f, rtol=1e-5, atol=1e-6)
     none, dw_only = GNNA.backward(dev(dy), dev(x), dev(w), *args, need_dx=False, relu_input=True)
     assert none.numel() == 0 and torch.equal(dw_only, dw_f)
+
+
+def test_training_from_a_dataset_file(GNNA, tmp_path):
+    """Reference-format files -> loader -> the same Trainer; the first-iteration gradients equal
+    the float64 dense model's on the loaded graph (scale = the loader's sqrt(deg) filling would
+    blow up a 2-layer model, so the symmetric normalisation is asked for)."""
+    from eppgcn_amd import dataset as dsmod, train
+    indptr, col = random_symmetric_csr(300, 1200, 31)
+    n = indptr.size - 1
+    rows = np.repeat(np.arange(n), np.diff(indptr))
+    np.savez(str(tmp_path / "g.npz"), src_li=rows, dst_li=col, num_nodes=n)
+    mask = np.random.default_rng(9).random(n) < 0.25
+    dsmod.write_train_mask(str(tmp_path), 0.25, mask)
+    d = dsmod.custom_dataset(str(tmp_path / "g.npz"), str(tmp_path), 0.25, 12, 7, 2, load_from_txt=False,
+                             scale_mode="inv_sqrt", feature_seed=5)
+    assert np.array_equal(d.row_pointers.cpu().numpy(), indptr) and np.array_equal(d.column_index.cpu().numpy(), col)
+    tr = train.Trainer(None, hidden=16, dataset=d, backsize=4)
+    w0 = tr.model.convs[0].weights.detach().cpu().numpy()
+    w1 = tr.model.convs[1].weights.detach().cpu().numpy()
+    want_loss, want_g0, want_g1 = _dense_model_grads(indptr, col, scale_inv_sqrt(indptr), d.x.cpu().numpy(), w0, w1,
+                                                     mask, d.y.cpu().numpy())
+    tr.optimizer = torch.optim.SGD(tr.model.parameters(), lr=0.0)
+    loss = tr.train_step(True)
+    assert abs(float(loss) - want_loss) < 1e-5 * max(1.0, abs(want_loss))
+    assert np.linalg.norm(tr.model.convs[0].weights.grad.cpu().numpy() - want_g0) / np.linalg.norm(want_g0) < 1e-4
+    assert np.linalg.norm(tr.model.convs[1].weights.grad.cpu().numpy() - want_g1) / np.linalg.norm(want_g1) < 1e-4
