@@ -190,12 +190,13 @@ void set_plan_keep_rows(int keep) { g_keep_rows = keep < 0 ? 0 : keep; }
 int schedule_shift(int dim)
 {
     if (g_force_shift > 0) return g_force_shift;
-    // column blocks of about 4 MB of feature rows (65536 rows of 64 bytes), one XCD's L2: measured
-    // at R-MAT scale 22, blocks of 8K..256K rows gather equally fast and larger blocks leave fewer
-    // partial sums to combine
+    // column blocks of at most 128K rows and 16 MB of feature rows.  Measured at R-MAT scale 22
+    // (ms per epoch, 64- and 128-byte rows): 2^14 5.95, 2^15 5.74, 2^16 5.63, 2^17 5.60, 2^18 5.65,
+    // 2^19 5.83 - the window all waves gather from has to stay resident in the memory-side cache,
+    // not in one XCD's L2, and larger blocks leave fewer partial sums to combine
     const int row_bytes = 4 * workspace_pitch(dim);
-    int shift = 16;
-    while (shift > 8 && (static_cast<long long>(row_bytes) << shift) > (6ll << 20)) --shift;
+    int shift = 17;
+    while (shift > 8 && (static_cast<long long>(row_bytes) << shift) > (16ll << 20)) --shift;
     return shift;
 }
 

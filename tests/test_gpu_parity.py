@@ -248,8 +248,13 @@ def test_plan_is_a_stable_column_block_reordering(api, name, ps):
     n = indptr.size - 1
     pp, p2n = co.build_part(ps, indptr)
     P = p2n.size
-    for dim in (16, 256):
-        plan = api.build_plan(dev(pp), dev(col), P, col.size, n, dim, part2node=dev(p2n))
+    # default block sizes (one block for these small graphs at width 16) and forced small blocks
+    for dim, forced in ((16, 0), (256, 0), (16, 9), (16, 12)):
+        api.set_plan_shift(forced)
+        try:
+            plan = api.build_plan(dev(pp), dev(col), P, col.size, n, dim, part2node=dev(p2n))
+        finally:
+            api.set_plan_shift(0)
         ptr, row, flags, pcol = [t.cpu().numpy() for t in plan.view()]
         assert ptr[0] == 0 and ptr[-1] == col.size and np.all(np.diff(ptr) >= 1)
         # identify every plan entry with its original group: same row, same size, same columns;
@@ -268,7 +273,7 @@ def test_plan_is_a_stable_column_block_reordering(api, name, ps):
         row_first_group = np.concatenate([[0], np.cumsum(groups_per_row)[:-1]])
         key_col = np.where(groups_per_row[p2n] <= 8, col[pp[row_first_group[p2n]]], col[pp[:-1]])[order]
         ok = False
-        for shift in range(8, 17):
+        for shift in ([forced] if forced else range(8, 18)):
             blocks = key_col >> shift
             if np.all(np.diff(blocks) >= 0) and np.all((np.diff(blocks) > 0) | (np.diff(order) > 0)):
                 ok = True
