@@ -286,3 +286,39 @@ def test_training_from_a_dataset_file(GNNA, tmp_path):
     assert abs(float(loss) - want_loss) < 1e-5 * max(1.0, abs(want_loss))
     assert np.linalg.norm(tr.model.convs[0].weights.grad.cpu().numpy() - want_g0) / np.linalg.norm(want_g0) < 1e-4
     assert np.linalg.norm(tr.model.convs[1].weights.grad.cpu().numpy() - want_g1) / np.linalg.norm(want_g1) < 1e-4
+
+
+@pytest.mark.parametrize("num_layers", [3, 4])
+def test_deeper_models_follow_the_mask_chain(GNNA, num_layers):
+    """3 and 4 layers (the reference sweeps 3-6): the marking of layer i feeds layer i+1's source
+    mask and edge_masks[L-1-i]; gradients of every weight equal the float64 dense model's."""
+    from eppgcn_amd import graphs, train
+    indptr, col = random_symmetric_csr(500, 1400, 41)
+    n = indptr.size - 1
+    s = scale_inv_sqrt(indptr)
+    g = graphs.Graph("t", n, dev(indptr), dev(col), dev(s))
+    mask = np.random.default_rng(4).random(n) < 0.1
+    tr = train.Trainer(g, dim=20, hidden=16, num_classes=9, num_layers=num_layers, train_mask=torch.from_numpy(mask),
+                       backsize=4, labels="uniform")
+    ws = [c.weights.detach().cpu().numpy() for c in tr.model.convs]
+    a = torch.zeros(n, n, dtype=torch.float64)
+    a[torch.from_numpy(cf.row_index(indptr)), torch.from_numpy(col.astype(np.int64))] = 1.0
+    a = a * (torch.from_numpy(s)[:, None] * torch.from_numpy(s)[None, :]).double()
+    w64 = [torch.tensor(w, dtype=torch.float64, requires_grad=True) for w in ws]
+    h = tr.dataset.x.cpu().double()
+    for i, w in enumerate(w64):
+        h = a @ (h @ w)
+        if i < num_layers - 1:
+            h = torch.relu(h)
+    tm = torch.from_numpy(mask)
+    want = torch.nn.functional.nll_loss(torch.log_softmax(h, 1)[tm], tr.dataset.y.cpu()[tm])
+    want.backward()
+    tr.optimizer = torch.optim.SGD(tr.model.parameters(), lr=0.0)
+    loss = tr.train_step(True)
+    assert abs(float(loss) - float(want)) < 1e-5 * max(1.0, abs(float(want)))
+    for c, w in zip(tr.model.convs, w64):
+        got, ref = c.weights.grad.cpu().numpy(), w.grad.numpy()
+        assert np.linalg.norm(got - ref) / np.linalg.norm(ref) < 1e-4
+    # the kept path grows from the last layer (train rows only) towards the first
+    kept = [b.numParts for b in tr.back_props]
+    assert all(kept[i] >= kept[i + 1] for i in range(num_layers - 1))
