@@ -411,7 +411,7 @@ struct AggTuning {
 static AggTuning g_tuning;
 void set_agg_force_team(int ts) { g_tuning.force_team = ts; }
 void set_agg_force_rounds(int r) { g_tuning.force_rounds = r; }
-constexpr int kEdgesPerWave = 400;
+constexpr int kEdgesPerWave = 800;
 constexpr int kGroupsPerWave = 64;
 constexpr int kMinWaves = 256 * 24 * 4;
 constexpr int kMaxRounds = 64;
@@ -431,8 +431,8 @@ static hipError_t launch_one(float* out, const float* in, const int* col, const 
     constexpr int TPW = kWave / TS;
     // rounds per wave: at least kEdgesPerWave gathered rows per wave, judged by the caller's
     // group size (an upper bound of the real group length), and at least kGroupsPerWave groups
-    // when a round holds fewer than 16 (measured at R-MAT scale 22: width 16, 16 groups a round,
-    // is fastest with one round of 496 edges; width 22, 8 groups a round, gains 9 % from 8 rounds
+    // when a round holds fewer than 16 (measured at R-MAT scale 22 with execution plans: width 16, 16
+    // groups a round, 1 / 2 / 4 / 8 rounds -> 1.36 / 1.32 / 1.35 / 1.45 ms; width 22, 8 groups a round, gains 9 % from 8 rounds
     // because a long row is then flushed once per 64 groups instead of once per 8)
     int rounds = g_tuning.force_rounds;
     if (rounds <= 0) {
