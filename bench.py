@@ -6,7 +6,7 @@ A step is one epoch's worth of aggregation for the 2-layer GCN of the reference'
 at width 22 (last layer) and 16 (first layer), launched back to back through the C ABI with
 every input resident in HBM.  The dense X*W products are not part of the metric.
 
-Prints ONE JSON line:  metric = BASELINE.json's, value = algorithmic GB/s of the epoch's
+Prints ONE JSON line:  metric = the headline metric below, value = algorithmic GB/s of the epoch's
 aggregation, ms_per_step = aggregation ms per epoch, plus `roofline` for the dominant kernel
 (HIP-event time of the kernel alone) and `cpu_baseline` (the CPU checker's OpenMP restatement
 timed on the host cores on one epoch of the same workload).
