@@ -42,6 +42,8 @@ def parse():
     ap.add_argument("--plan_shift", type=int, default=0, help="force log2 of the plan's column block")
     ap.add_argument("--plan_keep", type=int, default=-1, help="rows with at most this many groups stay together")
     ap.add_argument("--force_plan", action="store_true", help="use execution plans even for small feature tables")
+    ap.add_argument("--stepwise_prep", action="store_true",
+                    help="prepare the backward paths with the reference's separate marking and compaction steps")
     ap.add_argument("--no_plan", action="store_true",
                     help="process the groups in CSR order instead of the column-blocked execution plan")
     ap.add_argument("--no_workspace", action="store_true",
@@ -140,7 +142,8 @@ def main():
         capi.set_plan_keep_rows(args.plan_keep)
     t0 = time.perf_counter()
     wl = workload.prepare(g, 2, args.train_ratio, 2, args.part_size or None, args.backsize_mode, args.backsize,
-                          plan=False if (args.no_plan or args.no_workspace) else (True if args.force_plan else None))
+                          plan=False if (args.no_plan or args.no_workspace) else (True if args.force_plan else None),
+                          fused=not args.stepwise_prep)
     torch.cuda.synchronize()
     prep_s = time.perf_counter() - t0
     n, e = g.num_nodes, g.num_edges

@@ -24,6 +24,7 @@ EXPORTS = [
     "eppgcn_clear_time", "eppgcn_get_time_ms", "eppgcn_set_team_size", "eppgcn_set_rounds", "eppgcn_set_plan_shift", "eppgcn_set_plan_keep_rows",
     "eppgcn_feature_workspace_pitch", "eppgcn_update_forward", "eppgcn_update_backward_input",
     "eppgcn_update_workspace_bytes", "eppgcn_update_backward_weight", "eppgcn_update_supported",
+    "eppgcn_mark_compact_workspace_bytes", "eppgcn_mark_compact",
 ]
 
 _lib = None
@@ -84,6 +85,10 @@ def load():
     lib.eppgcn_set_plan_shift.restype = None
     lib.eppgcn_set_plan_keep_rows.argtypes = [i]
     lib.eppgcn_set_plan_keep_rows.restype = None
+    lib.eppgcn_mark_compact_workspace_bytes.argtypes = [i64]
+    lib.eppgcn_mark_compact_workspace_bytes.restype = sz
+    lib.eppgcn_mark_compact.argtypes = [p, p, p, p, p, p, p, p, i, i64, i, p, sz, p, C.POINTER(i64), p]
+    lib.eppgcn_mark_compact.restype = i
     lib.eppgcn_feature_workspace_pitch.argtypes = [i]
     lib.eppgcn_feature_workspace_pitch.restype = i
     lib.eppgcn_update_supported.argtypes = [i, i]
@@ -360,6 +365,30 @@ def compact_back_edge(edge_mask, column_index):
     v = C.c_int64(0)
     _check(lib.eppgcn_compact_back_edge(_ptr(edge_mask), _ptr(column_index), _ptr(out_id), _ptr(out_edge), length,
                                         _ptr(ws), nbytes, None, C.byref(v), _stream()))
+    return out_id, out_edge, int(v.value)
+
+
+def mark_compact(part2node, part_ptr, column_index, src_mask, ngh_mask, node_degs, is_last_layer: bool):
+    """Marking and compaction of one layer in one pass -> (id int32[E], edge_list int32[E],
+    valid_len); ngh_mask and node_degs are updated in place."""
+    lib = load()
+    _dev(part2node, torch.int32, "part2node"); _dev(part_ptr, torch.int32, "part_ptr")
+    _dev(column_index, torch.int32, "column_index"); _dev(node_degs, torch.int32, "node_degs")
+    src = _mask_bytes(src_mask, "src_mask")
+    ngh = _mask_bytes(ngh_mask, "ngh_mask")
+    if src is None:
+        raise EppgcnError("src_mask must not be empty")
+    if part_ptr.numel() < part2node.numel() + 1:
+        raise EppgcnError("part_ptr needs num_parts + 1 entries")
+    length = column_index.numel()
+    out_id = torch.empty(length, dtype=torch.int32, device=column_index.device)
+    out_edge = torch.empty(length, dtype=torch.int32, device=column_index.device)
+    nbytes = lib.eppgcn_mark_compact_workspace_bytes(length)
+    ws = _workspace(nbytes, column_index.device)
+    v = C.c_int64(0)
+    _check(lib.eppgcn_mark_compact(_ptr(part2node), _ptr(part_ptr), _ptr(column_index), _ptr(src), _ptr(ngh),
+                                   _ptr(node_degs), _ptr(out_id), _ptr(out_edge), part2node.numel(), length,
+                                   int(bool(is_last_layer)), _ptr(ws), nbytes, None, C.byref(v), _stream()))
     return out_id, out_edge, int(v.value)
 
 

@@ -34,6 +34,9 @@ size_t split_workspace_bytes(long long);
 int launch_mask_forward(const int*, const int*, const int*, const uint8_t*, uint8_t*, int*, int*, int, long long, int,
                         hipStream_t);
 int launch_compact_mask(const int*, int*, const int*, int*, long long, void*, hipStream_t);
+size_t mark_compact_workspace_bytes(long long);
+int launch_mark_compact(const int*, const int*, const int*, const uint8_t*, uint8_t*, int*, int*, int*, int, long long,
+                        int, void*, hipStream_t);
 int launch_split(bool, const int*, int, int, int*, int*, long long, bool, void*, hipStream_t);
 int launch_count_nonzero(const int*, long long, int*, hipStream_t);
 int launch_ginfo_hist(const int*, long long, int*, hipStream_t);
@@ -196,6 +199,38 @@ int eppgcn_compact_back_edge(const int32_t* edge_mask, const int32_t* column_ind
     EPPGCN_REQUIRE(length == 0 || (edge_mask && column_index && out_id && out_edge), "null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (int rc = launch_compact_mask(edge_mask, out_id, column_index, out_edge, length, workspace, s)) return rc;
+    ScanState* st = static_cast<ScanState*>(workspace);
+    if (d_valid_len)
+        EPPGCN_HIP(hipMemcpyAsync(d_valid_len, st->counts, sizeof(int), hipMemcpyDeviceToDevice, s));
+    if (h_valid_len) {
+        ScanState host;
+        if (int rc = read_state(workspace, s, &host)) return rc;
+        *h_valid_len = host.counts[0];
+    }
+    return kOk;
+}
+
+size_t eppgcn_mark_compact_workspace_bytes(int64_t num_edges) { return mark_compact_workspace_bytes(num_edges); }
+
+int eppgcn_mark_compact(const int32_t* part2node, const int32_t* part_pointers, const int32_t* column_index,
+                        const uint8_t* src_mask, uint8_t* ngh_mask, int32_t* node_degs, int32_t* out_id,
+                        int32_t* out_edge, int num_parts, int64_t num_edges, int is_last, void* workspace,
+                        size_t workspace_bytes, int32_t* d_valid_len, int64_t* h_valid_len, void* stream)
+{
+    EPPGCN_REQUIRE(num_parts >= 0 && num_edges >= 0 && num_edges < (1ll << 31), "num_parts >= 0 and 0 <= num_edges < 2^31 required");
+    EPPGCN_REQUIRE(workspace && aligned(workspace, 8), "workspace must be 8-byte aligned");
+    EPPGCN_REQUIRE(workspace_bytes >= mark_compact_workspace_bytes(num_edges), "workspace too small");
+    EPPGCN_REQUIRE(num_edges == 0 || (out_id && out_edge), "null output pointer");
+    EPPGCN_REQUIRE(num_parts == 0 || (part2node && part_pointers && column_index && src_mask && node_degs),
+                   "null pointer");
+    EPPGCN_REQUIRE(is_last || num_parts == 0 || ngh_mask, "ngh_mask is required unless this is the last layer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    {
+        KernelTimer timer(s, &g_mask_ms);
+        if (int rc = launch_mark_compact(part2node, part_pointers, column_index, src_mask, ngh_mask, node_degs, out_id,
+                                         out_edge, num_parts, num_edges, is_last ? 1 : 0, workspace, s))
+            return rc;
+    }
     ScanState* st = static_cast<ScanState*>(workspace);
     if (d_valid_len)
         EPPGCN_HIP(hipMemcpyAsync(d_valid_len, st->counts, sizeof(int), hipMemcpyDeviceToDevice, s));

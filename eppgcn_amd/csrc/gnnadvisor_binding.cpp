@@ -407,6 +407,34 @@ std::vector<Tensor> compact_back_edge(Tensor edge_mask, Tensor column_index)
     return {c.id, c.edge_list, info};
 }
 
+// Addition: mask_forward and compact_back_edge of one layer in one pass, same arguments as
+// mask_forward minus the edge mask and the launch hints; returns what compact_back_edge returns.
+std::vector<Tensor> mark_compact(Tensor id, Tensor partPointer, Tensor edgeList, Tensor src_mask, Tensor ngh_mask,
+                                 Tensor node_degs, int num_layers, int layer)
+{
+    CHECK_I32(id); CHECK_I32(partPointer); CHECK_I32(edgeList); CHECK_MASK(src_mask); CHECK_MASK(ngh_mask);
+    CHECK_I32(node_degs);
+    const bool is_last = layer == num_layers;
+    TORCH_CHECK(partPointer.numel() >= id.numel() + 1, "partPointer needs num_parts + 1 entries");
+    TORCH_CHECK(src_mask.numel() == node_degs.numel(), "src_mask and node_degs must have one entry per vertex");
+    TORCH_CHECK(is_last || ngh_mask.numel() == node_degs.numel(), "ngh_mask must have one entry per vertex");
+    const int64_t length = edgeList.numel();
+    auto out_id = torch::empty({length}, edgeList.options());
+    auto out_edge = torch::empty({length}, edgeList.options());
+    const size_t nbytes = eppgcn_mark_compact_workspace_bytes(length);
+    auto ws = torch::empty({static_cast<int64_t>((nbytes + 7) / 8)}, edgeList.options().dtype(torch::kInt64));
+    int64_t valid_len = 0;
+    check(eppgcn_mark_compact(i32(id), i32(partPointer), i32(edgeList), static_cast<const uint8_t*>(src_mask.data_ptr()),
+                              ngh_mask.numel() ? static_cast<uint8_t*>(ngh_mask.data_ptr()) : nullptr,
+                              node_degs.data_ptr<int32_t>(), length ? out_id.data_ptr<int32_t>() : nullptr,
+                              length ? out_edge.data_ptr<int32_t>() : nullptr, static_cast<int>(id.numel()), length,
+                              is_last ? 1 : 0, ws.data_ptr(), nbytes, nullptr, &valid_len, stream_of(id)),
+          "mark_compact");
+    auto info = torch::zeros({1}, torch::kFloat64);
+    info[0] = static_cast<double>(valid_len);
+    return {out_id, out_edge, info};
+}
+
 int get_map_back_part_size(Tensor node_deg, int valid_len)
 {
     int clamped = 0;
@@ -487,6 +515,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("build_part", &build_part, "forward neighbour groups (HIP)");
     m.def("build_back_part", &build_back_part, "compaction + group split in one call (HIP)");
     m.def("compact_back_edge", &compact_back_edge, "compact the kept edges of one layer (HIP)");
+    m.def("mark_compact", &mark_compact, "marking + compaction of one layer in one pass (HIP)");
     m.def("get_map_back_part_size", &get_map_back_part_size, "backward group size from the fitted regression");
     m.def("split_back_part", &split_back_part, "split kept edges into backward groups (HIP)");
     m.def("get_ginfo", &get_ginfo, "degree-distribution features of the kept path");

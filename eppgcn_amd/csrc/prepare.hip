@@ -163,6 +163,165 @@ __global__ __launch_bounds__(kCompactBlock) void compact_mask_kernel(
     }
 }
 
+// ================================================================ fused marking + compaction
+// One pass over the slots does what mask_forward_kernel followed by compact_mask_kernel do, without
+// the E-entry edge mask between them: a tile of 4096 consecutive slots finds the group (hence the
+// row) of every slot from a bit map of the group starts inside the tile (prefix population count;
+// tile_groups_kernel finds each tile's first group beforehand), decides keep = src_mask[col],
+// marks the neighbour masks, counts kept slots per row from wave ballots (one atomic per run of
+// equal rows in a wave), and compacts (row, col) of the kept slots with the same ballot ranks and
+// look-back prefix as compact_mask_kernel.
+
+// first[t] = last group starting at or before slot t * kCompactTile; first[num_tiles] = last group
+__global__ void tile_groups_kernel(const int* __restrict__ part_ptr, int num_parts, int num_tiles,
+                                   int* __restrict__ first)
+{
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t > num_tiles) return;
+    if (t == num_tiles) {
+        first[t] = num_parts - 1;
+        return;
+    }
+    const long long slot = static_cast<long long>(t) * kCompactTile;
+    int a = 0, b = num_parts;                 // part_ptr[a] <= slot is assumed for a = 0
+    while (b - a > 1) {
+        const int mid = a + (b - a) / 2;
+        if (part_ptr[mid] <= slot) a = mid; else b = mid;
+    }
+    first[t] = a;
+}
+
+__global__ __launch_bounds__(kCompactBlock) void mark_compact_kernel(
+    const int* __restrict__ part2node, const int* __restrict__ part_ptr, const int* __restrict__ col,
+    const uint8_t* __restrict__ src_mask, uint8_t* __restrict__ ngh_mask, int* __restrict__ node_degs,
+    int* __restrict__ out_id, int* __restrict__ out_edge, int num_parts, int length, int num_tiles, int is_last,
+    const int* __restrict__ tile_first, ScanState* st, uint64_t* desc)
+{
+    __shared__ int s_tile;
+    __shared__ int s_count[kWave];
+    __shared__ int s_prefix;
+    __shared__ unsigned long long s_bits[kCompactTile / 64];   // bit p: a group starts at slot base + p
+    __shared__ int s_word_prefix[kCompactTile / 64];     // group starts before each 64-slot word
+    __shared__ int s_starts_in_tile;
+    if (threadIdx.x < kCompactTile / 64) s_bits[threadIdx.x] = 0ull;
+    if (threadIdx.x == 0) s_starts_in_tile = 0;
+    const int tile = acquire_tile(st, &s_tile);          // contains the barrier that publishes the zeros
+    if (tile >= num_tiles) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const long long base = static_cast<long long>(tile) * kCompactTile;
+    const int g_lo = tile_first[tile];
+    const int g_cnt = tile_first[tile + 1] - g_lo + 1;
+    // slots outside [part_ptr[0], part_ptr[num_parts]) belong to no group and are never kept
+    const int owned_lo = part_ptr[0];
+    const int owned_hi = part_ptr[num_parts];
+    // The owner of slot e is g_lo - 1 + (number of groups of the tile that start at or before e).
+    // When no two groups start at the same slot (no empty groups, as build_part guarantees) that
+    // number is a prefix population count over a 4096-bit map of group starts; otherwise every
+    // slot does a binary search over the group starts in global memory.
+    {
+        int mine = 0;
+        for (int i = threadIdx.x; i < g_cnt; i += kCompactBlock) {
+            const long long p = part_ptr[g_lo + i] - base;
+            if (p >= 0 && p < kCompactTile) {
+                atomicOr(&s_bits[p >> 6], 1ull << (p & 63));
+                ++mine;
+            }
+        }
+        if (mine) atomicAdd(&s_starts_in_tile, mine);
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const int pc = __popcll(s_bits[lane]);
+        const int incl = wave_inclusive_scan(pc);
+        s_word_prefix[lane] = incl - pc;
+        if (lane == kWave - 1 && incl != s_starts_in_tile) s_starts_in_tile = -1;   // duplicate starts
+    }
+    __syncthreads();
+    const bool by_bits = s_starts_in_tile >= 0;
+    const int before = part_ptr[g_lo] < base ? 1 : 0;    // g_lo itself starts before the tile
+
+    // phases with all loads of one kind issued together: a ballot inside the item loop would make
+    // every item wait for its own gather (16 dependent memory round trips per tile)
+    int v[kCompactItems], c[kCompactItems], rows[kCompactItems];
+    bool ok[kCompactItems], keep[kCompactItems], row_src[kCompactItems];
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k) {
+        const long long idx = base + k * kCompactBlock + threadIdx.x;
+        ok[k] = idx < length && idx >= owned_lo && idx < owned_hi;
+        c[k] = ok[k] ? col[idx] : 0;
+    }
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k) {
+        rows[k] = -1;
+        if (ok[k]) {
+            const int e = static_cast<int>(base + k * kCompactBlock + threadIdx.x);
+            int a = 0, b = g_cnt;
+            if (by_bits) {
+                const int p = k * kCompactBlock + threadIdx.x;
+                const unsigned long long upto = (p & 63) == 63 ? ~0ull : (2ull << (p & 63)) - 1ull;
+                a = before + s_word_prefix[p >> 6] + __popcll(s_bits[p >> 6] & upto) - 1;
+            } else {
+                while (b - a > 1) {
+                    const int mid = (a + b) >> 1;
+                    if (part_ptr[g_lo + mid] <= e) a = mid; else b = mid;
+                }
+            }
+            rows[k] = part2node[g_lo + a];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k) {
+        keep[k] = ok[k] && src_mask[c[k]] != 0;
+        row_src[k] = ok[k] && !is_last && src_mask[rows[k]] != 0;
+    }
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k) {
+        if (row_src[k]) {
+            ngh_mask[rows[k]] = 1;
+            ngh_mask[c[k]] = 1;
+        }
+        v[k] = keep[k] ? rows[k] : -1;
+        // kept slots per row: the lanes of a wave hold 64 consecutive slots of item k
+        const int row = rows[k];
+        const int prev_row = __shfl_up(row, 1, kWave);
+        const uint64_t heads = __ballot(lane == 0 || prev_row != row);
+        const uint64_t kept = __ballot(keep[k]);
+        if ((heads >> lane) & 1ull) {
+            const uint64_t above = lane == kWave - 1 ? 0ull : heads & ~((2ull << lane) - 1ull);
+            const int next = above ? __builtin_ctzll(above) : kWave;
+            const uint64_t upto = next == kWave ? ~0ull : (1ull << next) - 1ull;
+            const int n = __popcll(kept & upto & ~((1ull << lane) - 1ull));
+            if (n > 0) atomicAdd(node_degs + row, n);
+        }
+        if (lane == 0) s_count[k * (kCompactBlock / kWave) + wave] = __popcll(kept);
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const int cnt = s_count[lane];
+        const int incl = wave_inclusive_scan(cnt);
+        const int total = __shfl(incl, kWave - 1, kWave);
+        s_count[lane] = incl - cnt;
+        const uint64_t excl = tile_lookback(desc, st, tile, static_cast<uint64_t>(total));
+        if (lane == 0) {
+            s_prefix = static_cast<int>(excl);
+            if (tile == num_tiles - 1) st->counts[0] = static_cast<int>(excl) + total;
+        }
+    }
+    __syncthreads();
+    const int prefix = s_prefix;
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k) {
+        const bool pred = v[k] != -1;
+        const uint64_t ballot = __ballot(pred);
+        if (pred) {
+            const int dst = prefix + s_count[k * (kCompactBlock / kWave) + wave] + ballot_rank(ballot);
+            out_id[dst] = v[k];
+            out_edge[dst] = c[k];
+        }
+    }
+}
+
 // Zero both outputs from the compacted length (read on the device) to the end.
 __global__ void zero_tail2_kernel(int* __restrict__ a, int* __restrict__ b, const int* __restrict__ d_start, int length)
 {
@@ -372,6 +531,44 @@ int launch_compact_mask(const int* in_id, int* out_id, const int* in_edge, int* 
                            out_edge, st->counts, static_cast<int>(length));
         EPPGCN_HIP(hipGetLastError());
     }
+    return kOk;
+}
+
+size_t mark_compact_workspace_bytes(long long length)
+{
+    const long long tiles = (length + kCompactTile - 1) / kCompactTile;
+    return compact_workspace_bytes(length) + static_cast<size_t>(tiles + 2) * sizeof(int);
+}
+
+// Results land in the ScanState at the head of the workspace: counts[0] = kept length.
+int launch_mark_compact(const int* part2node, const int* part_ptr, const int* col, const uint8_t* src_mask,
+                        uint8_t* ngh_mask, int* node_degs, int* out_id, int* out_edge, int num_parts,
+                        long long length, int is_last, void* workspace, hipStream_t stream)
+{
+    ScanState* st = static_cast<ScanState*>(workspace);
+    uint64_t* desc = reinterpret_cast<uint64_t*>(st + 1);
+    const int num_tiles = num_parts > 0 ? static_cast<int>((length + kCompactTile - 1) / kCompactTile) : 0;
+    if (int rc = init_scan(workspace, num_tiles, stream)) return rc;
+    if (num_tiles == 0) {
+        if (length > 0) {
+            EPPGCN_HIP(hipMemsetAsync(out_id, 0, sizeof(int) * length, stream));
+            EPPGCN_HIP(hipMemsetAsync(out_edge, 0, sizeof(int) * length, stream));
+        }
+        return kOk;
+    }
+    int* tile_first = reinterpret_cast<int*>(static_cast<char*>(workspace) + compact_workspace_bytes(length));
+    hipLaunchKernelGGL(tile_groups_kernel, dim3((num_tiles + 1 + 255) / 256), dim3(256), 0, stream, part_ptr, num_parts,
+                       num_tiles, tile_first);
+    EPPGCN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(mark_compact_kernel, dim3(num_tiles), dim3(kCompactBlock), 0, stream, part2node, part_ptr, col,
+                       src_mask, ngh_mask, node_degs, out_id, out_edge, num_parts, static_cast<int>(length), num_tiles,
+                       is_last, tile_first, st, desc);
+    EPPGCN_HIP(hipGetLastError());
+    long long blocks = (length + 1023) / 1024;
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL(zero_tail2_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, out_id, out_edge,
+                       st->counts, static_cast<int>(length));
+    EPPGCN_HIP(hipGetLastError());
     return kOk;
 }
 

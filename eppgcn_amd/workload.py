@@ -60,7 +60,9 @@ def choose_back_part_size(mode: str, constant: int, valid_node: int, valid_len: 
 
 def prepare(graph: graphs.Graph, num_layers: int = 2, train_ratio: float = 0.1, mask_seed: int = 2,
             part_size: int = None, backsize_mode: str = "constant", backsize: int = 32,
-            train_mask: torch.Tensor = None, widths=(16, 22), plan=None) -> Workload:
+            train_mask: torch.Tensor = None, widths=(16, 22), plan=None, fused: bool = True) -> Workload:
+    """``fused``: mark and compact every layer in one pass (no E-entry edge masks); False runs the
+    reference's separate steps.  The results are identical."""
     g = graph
     dev = g.column_index.device
     n, e = g.num_nodes, g.num_edges
@@ -73,7 +75,8 @@ def prepare(graph: graphs.Graph, num_layers: int = 2, train_ratio: float = 0.1, 
 
     # per-run state, EPPGCN/dataset.py:135-156
     ngh_masks = [torch.zeros(n, dtype=torch.bool, device=dev) for _ in range(num_layers - 1)]
-    edge_masks = [torch.full((e,), -1, dtype=torch.int32, device=dev) for _ in range(num_layers)]
+    edge_masks = ([None] * num_layers if fused else
+                  [torch.full((e,), -1, dtype=torch.int32, device=dev) for _ in range(num_layers)])
     node_degs = [torch.zeros(n, dtype=torch.int32, device=dev) for _ in range(num_layers)]
 
     # mask chain, EPPGCN/gcn_main.py:130-139: step i runs in the forward of conv i
@@ -82,12 +85,16 @@ def prepare(graph: graphs.Graph, num_layers: int = 2, train_ratio: float = 0.1, 
         last = i == num_layers - 1
         dst = None if last else ngh_masks[i]
         k = num_layers - 1 - i
-        capi.mask_forward(part2node, part_ptr, g.column_index, src, dst, edge_masks[k], node_degs[k], last)
+        if fused:
+            edge_masks[k] = capi.mark_compact(part2node, part_ptr, g.column_index, src, dst, node_degs[k], last)
+        else:
+            capi.mask_forward(part2node, part_ptr, g.column_index, src, dst, edge_masks[k], node_degs[k], last)
 
     # buildBackPart, EPPGCN/gcn_main.py:151-168
     paths = []
     for k in range(num_layers):
-        ids, edge_list, valid_len = capi.compact_back_edge(edge_masks[k], g.column_index)
+        ids, edge_list, valid_len = (edge_masks[k] if fused else
+                                     capi.compact_back_edge(edge_masks[k], g.column_index))
         edge_masks[k] = None
         valid_node = capi.count_nonzero(node_degs[k])
         bps = choose_back_part_size(backsize_mode, backsize, valid_node, valid_len)

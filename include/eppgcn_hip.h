@@ -158,6 +158,21 @@ int eppgcn_compact_back_edge(const int32_t* edge_mask, const int32_t* column_ind
                              void* workspace, size_t workspace_bytes,
                              int32_t* d_valid_len, int64_t* h_valid_len, void* stream);
 
+/* Path marking and compaction of one layer in one pass over the slots: exactly the results of
+ * eppgcn_mask_forward on a -1-filled edge mask followed by eppgcn_compact_back_edge (ngh_mask and
+ * node_degs updated in place, out_id / out_edge with zero tails, V at d_valid_len / h_valid_len),
+ * without the num_edges-entry edge mask in between.  The reference runs the two steps separately
+ * (mask_forward_cuda, EPPGCN_kernel.cu:297-388, inside the first forward; compact_mask,
+ * cuCompactor.cu:328-465, from gcn_main.py:154); this call is for drivers that prepare the path
+ * before training.  The groups must tile the slots in order, as build_part produces them.
+ * workspace: eppgcn_mark_compact_workspace_bytes(num_edges) bytes, 8-byte aligned. */
+size_t eppgcn_mark_compact_workspace_bytes(int64_t num_edges);
+int eppgcn_mark_compact(const int32_t* part2node, const int32_t* part_pointers,
+                        const int32_t* column_index, const uint8_t* src_mask, uint8_t* ngh_mask,
+                        int32_t* node_degs, int32_t* out_id, int32_t* out_edge, int num_parts,
+                        int64_t num_edges, int is_last_layer, void* workspace, size_t workspace_bytes,
+                        int32_t* d_valid_len, int64_t* h_valid_len, void* stream);
+
 /* Number of entries != 0 (valid_node of the group-size heuristics).  Stands in for
  * compact_count (cuCompactor.cu:694-696 over :623-680).  d_count: one device int. */
 int eppgcn_count_nonzero(const int32_t* node_deg, int64_t length, int32_t* d_count,

@@ -322,3 +322,19 @@ def test_deeper_models_follow_the_mask_chain(GNNA, num_layers):
     # the kept path grows from the last layer (train rows only) towards the first
     kept = [b.numParts for b in tr.back_props]
     assert all(kept[i] >= kept[i + 1] for i in range(num_layers - 1))
+
+
+def test_module_mark_compact_equals_the_two_reference_steps(GNNA):
+    indptr, col = random_symmetric_csr(2000, 9000, 23)
+    n, e = indptr.size - 1, col.size
+    src = np.random.default_rng(6).random(n) < 0.2
+    pp, p2n = GNNA.build_part(7, dev(indptr))
+    pp, p2n = pp.int(), p2n.int()
+    ngh_a = torch.zeros(n, dtype=torch.bool, device="cuda"); ngh_b = ngh_a.clone()
+    degs_a = torch.zeros(n, dtype=torch.int32, device="cuda"); degs_b = degs_a.clone()
+    bem = torch.full((e,), -1, dtype=torch.int32, device="cuda")
+    GNNA.mask_forward(p2n, pp, dev(col), dev(src), ngh_a, bem, degs_a, 2, 1, 4, 16)
+    id_a, el_a, info_a = GNNA.compact_back_edge(bem, dev(col))
+    id_b, el_b, info_b = GNNA.mark_compact(p2n, pp, dev(col), dev(src), ngh_b, degs_b, 2, 1)
+    assert torch.equal(id_a, id_b) and torch.equal(el_a, el_b) and float(info_a[0]) == float(info_b[0])
+    assert torch.equal(ngh_a, ngh_b) and torch.equal(degs_a, degs_b)

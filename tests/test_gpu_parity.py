@@ -501,3 +501,48 @@ def test_rmat20_linearity_and_tolerance(api, rmat20):
             0, row, w.abs()[:, None] * x[g.column_index.long()].double().abs())
         worst = ((got.double() - want).abs() / (RTOL * bound + 1e-30)).max().item()
         assert worst <= 1.0, f"D={dim}: max err/limit {worst:.3f}"
+
+
+# ----------------------------------------------------------------------------- fused marking + compaction
+@pytest.mark.parametrize("name", list(GRAPHS))
+@pytest.mark.parametrize("ratio", [0.0, 0.1, 0.6, 1.0])
+@pytest.mark.parametrize("ps", [1, 3, 32, 5000])
+def test_mark_compact_equals_marking_then_compaction(api, name, ratio, ps):
+    """One pass must leave exactly what the checker's mask_forward followed by its compaction
+    leave: compacted rows and columns with zero tails, kept length, kept degrees (added to what
+    node_degs held), neighbour mask (or-ed into what it held); for a middle and a last layer."""
+    indptr, col = GRAPHS[name]()
+    n = indptr.size - 1
+    rng = np.random.default_rng(5)
+    src = rng.random(n) < ratio
+    pp, p2n = co.build_part(ps, indptr)
+    for is_last in (False, True):
+        ngh0 = rng.random(n) < 0.05
+        degs0 = rng.integers(0, 3, n).astype(np.int32)
+        want_ngh = ngh0.copy()
+        want_bem = np.full(col.size, -1, np.int32)
+        want_degs = degs0.copy()
+        co.mask_forward(p2n, pp, col, src, None if is_last else want_ngh, want_bem, want_degs, is_last)
+        want_id, want_edge, want_v = co.compact_mask(want_bem, col)
+        ngh = None if is_last else dev(ngh0)
+        degs = dev(degs0)
+        out_id, out_edge, v = api.mark_compact(dev(p2n), dev(pp), dev(col), dev(src), ngh, degs, is_last)
+        assert v == want_v
+        assert np.array_equal(out_id.cpu().numpy(), want_id) and np.array_equal(out_edge.cpu().numpy(), want_edge)
+        assert np.array_equal(degs.cpu().numpy(), want_degs)
+        if not is_last:
+            assert np.array_equal(ngh.cpu().numpy(), want_ngh)
+
+
+def test_fused_and_stepwise_path_preparation_agree_at_scale(api):
+    """R-MAT scale 20: the whole mask chain and both layers' backward paths, fused versus the
+    reference's separate steps, bit for bit."""
+    from eppgcn_amd import graphs, workload
+    g = graphs.make_graph("cfg3_rmat20", device="cuda")
+    a = workload.prepare(g, 2, 0.1, 2, fused=True, plan=False)
+    b = workload.prepare(g, 2, 0.1, 2, fused=False, plan=False)
+    assert torch.equal(a.ngh_masks[0], b.ngh_masks[0])
+    for pa, pb in zip(a.paths, b.paths):
+        assert (pa.valid_len, pa.num_parts, pa.valid_node) == (pb.valid_len, pb.num_parts, pb.valid_node)
+        assert torch.equal(pa.ids, pb.ids) and torch.equal(pa.edge_list, pb.edge_list)
+        assert torch.equal(pa.part_pointer, pb.part_pointer) and torch.equal(pa.node_degs, pb.node_degs)
