@@ -548,7 +548,7 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
 {
     const bool prescaled = workspace != nullptr;
     int ld_in = dim;
-    EPPGCN_HIP(hipMemsetAsync(out, 0, static_cast<size_t>(num_nodes) * dim * sizeof(float), stream));
+    if (int rc = launch_zero_words(out, static_cast<size_t>(num_nodes) * dim, stream)) return rc;
     if (num_parts == 0) return kOk;
     if (prescaled) {
         // in == nullptr: the caller (the dense update) already wrote the scaled, padded rows

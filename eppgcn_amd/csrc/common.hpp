@@ -40,6 +40,11 @@ int hip_fail(hipError_t e, const char* what);
         }                                                       \
     } while (0)
 
+// Zeroes `words` 32-bit words at p (4-byte aligned) with a fill kernel.  Used instead of
+// hipMemsetAsync everywhere so that every call of the library can be captured into a HIP graph
+// (memset nodes are the one node kind callers are told to avoid on this platform).
+int launch_zero_words(void* p, size_t words, hipStream_t stream);
+
 // ---------------------------------------------------------------- execution plan layout
 // One caller-owned buffer: ptr[P+1] | row[P] | flags[P] | col[S], each part 256-byte aligned
 // (contents described in schedule.hip).  Offsets depend on the group count alone.

@@ -480,6 +480,34 @@ __global__ __launch_bounds__(kSplitBlock) void split_groups_kernel(
 }
 
 // ================================================================ host launchers
+__global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* __restrict__ p, size_t head, size_t vecs, size_t words)
+{
+    // [0, head) scalar words up to the first 16-byte boundary, then `vecs` uint4, then the rest
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    uint4* v = reinterpret_cast<uint4*>(p + head);
+    for (size_t i = tid; i < vecs; i += stride) v[i] = make_uint4(0u, 0u, 0u, 0u);
+    const size_t tail = head + 4 * vecs;
+    if (tid < head) p[tid] = 0u;
+    if (tid < words - tail) p[tail + tid] = 0u;
+}
+
+int launch_zero_words(void* p, size_t words, hipStream_t stream)
+{
+    if (words == 0) return kOk;
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+    size_t head = ((16 - a % 16) % 16) / 4;
+    if (head > words) head = words;
+    const size_t vecs = (words - head) / 4;
+    size_t blocks = (vecs + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(zero_words_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
+                       static_cast<uint32_t*>(p), head, vecs, words);
+    EPPGCN_HIP(hipGetLastError());
+    return kOk;
+}
+
 size_t scan_workspace_bytes(long long length, int tile)
 {
     const long long tiles = (length + tile - 1) / tile;
@@ -551,8 +579,8 @@ int launch_mark_compact(const int* part2node, const int* part_ptr, const int* co
     if (int rc = init_scan(workspace, num_tiles, stream)) return rc;
     if (num_tiles == 0) {
         if (length > 0) {
-            EPPGCN_HIP(hipMemsetAsync(out_id, 0, sizeof(int) * length, stream));
-            EPPGCN_HIP(hipMemsetAsync(out_edge, 0, sizeof(int) * length, stream));
+            if (int rc = launch_zero_words(out_id, static_cast<size_t>(length), stream)) return rc;
+            if (int rc = launch_zero_words(out_edge, static_cast<size_t>(length), stream)) return rc;
         }
         return kOk;
     }
@@ -581,7 +609,8 @@ int launch_split(bool from_row_ptr, const int* src, int num_nodes, int part_size
     const int num_tiles = (num_nodes + kSplitTile - 1) / kSplitTile;
     if (int rc = init_scan(workspace, num_tiles, stream)) return rc;
     if (num_tiles == 0) {
-        if (capacity > 0) EPPGCN_HIP(hipMemsetAsync(part_ptr_out, 0, sizeof(int) * (zero_tail ? capacity : 1), stream));
+        if (capacity > 0)
+            if (int rc = launch_zero_words(part_ptr_out, static_cast<size_t>(zero_tail ? capacity : 1), stream)) return rc;
         return kOk;
     }
     if (from_row_ptr)
@@ -604,7 +633,7 @@ int launch_split(bool from_row_ptr, const int* src, int num_nodes, int part_size
 
 int launch_count_nonzero(const int* in, long long length, int* d_count, hipStream_t stream)
 {
-    EPPGCN_HIP(hipMemsetAsync(d_count, 0, sizeof(int), stream));
+    if (int rc = launch_zero_words(d_count, 1, stream)) return rc;
     if (length == 0) return kOk;
     long long blocks = (length + 1023) / 1024;
     if (blocks > 1024) blocks = 1024;
@@ -616,7 +645,7 @@ int launch_count_nonzero(const int* in, long long length, int* d_count, hipStrea
 
 int launch_ginfo_hist(const int* node_deg, long long length, int* d_hist10, hipStream_t stream)
 {
-    EPPGCN_HIP(hipMemsetAsync(d_hist10, 0, sizeof(int) * 10, stream));
+    if (int rc = launch_zero_words(d_hist10, 10, stream)) return rc;
     if (length == 0) return kOk;
     long long blocks = (length + 1023) / 1024;
     if (blocks > 1024) blocks = 1024;

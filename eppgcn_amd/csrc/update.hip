@@ -362,8 +362,7 @@ int launch_dense_weight(float* dw, const float* x, int ld_x, const float* g, int
 {
     if (K == 0 || D == 0) return kOk;
     if (n == 0) {
-        EPPGCN_HIP(hipMemsetAsync(dw, 0, static_cast<size_t>(K) * D * sizeof(float), stream));
-        return kOk;
+        return launch_zero_words(dw, static_cast<size_t>(K) * D, stream);
     }
     if (D > 64) {
         set_error("dense update: more than 64 gradient columns are not supported by the weight kernel");

@@ -546,3 +546,47 @@ def test_fused_and_stepwise_path_preparation_agree_at_scale(api):
         assert (pa.valid_len, pa.num_parts, pa.valid_node) == (pb.valid_len, pb.num_parts, pb.valid_node)
         assert torch.equal(pa.ids, pb.ids) and torch.equal(pa.edge_list, pb.edge_list)
         assert torch.equal(pa.part_pointer, pb.part_pointer) and torch.equal(pa.node_degs, pb.node_degs)
+
+
+# ----------------------------------------------------------------------------- HIP graph capture
+def test_aggregation_calls_replay_from_a_hip_graph(api):
+    """The library allocates nothing and clears its outputs with a fill kernel (no memset nodes),
+    so a caller can capture the calls into a HIP graph.  Every replay, with eager work and
+    synchronisations in between and fresh inputs each time, must equal the eager result."""
+    indptr, col = random_symmetric_csr(6000, 40000, 77)
+    n = indptr.size - 1
+    s = scale_inv_sqrt(indptr)
+    rng = np.random.default_rng(8)
+    src = rng.random(n) < 0.3
+    pp, p2n = api.build_part(8, dev(indptr), col.size)
+    d_col, d_s = dev(col), dev(s)
+    ids, edge_list, v = api.mark_compact(p2n, pp, d_col, dev(src), None, torch.zeros(n, dtype=torch.int32, device="cuda"), True)
+    degs = torch.zeros(n, dtype=torch.int32, device="cuda")
+    api.mark_compact(p2n, pp, d_col, dev(src), None, degs, True)
+    part_pointer, num_parts, _ = api.split_back_part(degs, col.size, 8)
+    x = torch.zeros((n, 22), device="cuda")
+    y_fwd, y_bwd = torch.empty_like(x), torch.empty_like(x)
+    ws = api.feature_workspace(n, 22, "cuda")
+
+    def both():
+        api.spmm_forward(x, d_col, d_s, pp, p2n, 8, out=y_fwd, workspace=ws)
+        api.ours_backward(x, ids, part_pointer, edge_list, d_s, num_parts, 8, out=y_bwd, workspace=ws)
+
+    both()                                    # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        both()
+    for rep in range(4):
+        x.copy_(dev(rng.standard_normal((n, 22)).astype(np.float32)))
+        y_fwd.fill_(7.0); y_bwd.fill_(7.0)    # stale contents the replay has to clear itself
+        graph.replay()
+        torch.cuda.synchronize()
+        got_f, got_b = y_fwd.clone(), y_bwd.clone()
+        both()                                # eager, same inputs
+        torch.cuda.synchronize()
+        xn = x.cpu().numpy()
+        bound = co.spmm_f64(np.abs(xn), indptr, col, s) + 1e-30
+        assert_close(got_f.cpu().numpy(), y_fwd.cpu().numpy().astype(np.float64), 2 * bound, f"forward replay {rep}")
+        assert_close(got_b.cpu().numpy(), y_bwd.cpu().numpy().astype(np.float64), 2 * bound, f"backward replay {rep}")
+        assert_close(got_f.cpu().numpy(), co.spmm_f64(xn, indptr, col, s), bound, f"forward replay {rep} vs checker")
