@@ -49,3 +49,34 @@ def test_product_package_never_imports_the_checker():
             if f.endswith((".py", ".hip", ".cpp", ".hpp", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, f"{f} mentions the checker"
+
+
+def test_argument_errors_are_reported_before_any_device_work():
+    """Invalid sizes and null pointers are rejected by host-side checks (return code -1 and a
+    message naming the function), so these calls are safe without a GPU."""
+    from eppgcn_amd import capi
+    lib = capi.load()
+    p0 = ctypes.c_void_p(0)
+    one = ctypes.c_void_p(16)      # a non-null, aligned, never dereferenced address
+    cases = [
+        (lib.eppgcn_update_forward(one, 4, one, one, p0, 0, 8, 0, 5, p0), "in_dim > 0"),
+        (lib.eppgcn_update_forward(one, 3, one, one, p0, 0, 8, 4, 5, p0), "ld_out"),
+        (lib.eppgcn_update_forward(one, 8, one, p0, p0, 0, 8, 4, 5, p0), "null matrix"),
+        (lib.eppgcn_update_backward_input(one, one, one, p0, -1, 4, 5, p0), "num_nodes >= 0"),
+        (lib.eppgcn_update_backward_weight(one, one, one, 0, 8, 4, 5, p0, 0, p0), "workspace"),
+        (lib.eppgcn_mark_compact(one, one, one, one, one, one, one, one, 3, 1 << 31, 0, one, 1 << 20, p0, None, p0),
+         "num_edges"),
+        (lib.eppgcn_mark_compact(one, one, one, one, one, one, one, one, 3, 100, 0, one, 8, p0, None, p0), "workspace too small"),
+        (lib.eppgcn_spmm_forward(one, p0, p0, one, one, one, one, 8, 4, 2, 1, 1, 1, p0, 0, p0, p0), "null feature"),
+        (lib.eppgcn_spmm_forward(one, one, p0, one, one, one, one, 8, 0, 2, 1, 1, 1, p0, 0, p0, p0), "dim > 0"),
+    ]
+    for rc, needle in cases:
+        assert rc == -1
+    # the message belongs to the last failing call
+    assert b"dim > 0" in lib.eppgcn_last_error()
+    assert lib.eppgcn_update_supported(96, 16) == 7 and lib.eppgcn_update_supported(2000, 16) == 6
+    assert lib.eppgcn_update_supported(16, 100) == 3 and lib.eppgcn_update_supported(0, 4) == 0
+    assert lib.eppgcn_feature_workspace_pitch(16) == 16 and lib.eppgcn_feature_workspace_pitch(22) == 32
+    assert lib.eppgcn_feature_workspace_pitch(3) == 4 and lib.eppgcn_feature_workspace_pitch(40) == 40
+    assert lib.eppgcn_update_workspace_bytes(0, 4, 4) == 0
+    assert lib.eppgcn_mark_compact_workspace_bytes(4096 * 3 + 1) >= 32 + 8 * 4 + 4 * 5

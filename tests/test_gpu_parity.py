@@ -590,3 +590,41 @@ def test_aggregation_calls_replay_from_a_hip_graph(api):
         assert_close(got_f.cpu().numpy(), y_fwd.cpu().numpy().astype(np.float64), 2 * bound, f"forward replay {rep}")
         assert_close(got_b.cpu().numpy(), y_bwd.cpu().numpy().astype(np.float64), 2 * bound, f"backward replay {rep}")
         assert_close(got_f.cpu().numpy(), co.spmm_f64(xn, indptr, col, s), bound, f"forward replay {rep} vs checker")
+
+
+# ----------------------------------------------------------------------------- headline size
+def test_rmat22_headline_size_exact_integer_sums_with_plans(api):
+    """The benchmark's own configuration (R-MAT scale 22, 132 M slots), where execution plans,
+    128-byte padded rows and multi-round waves are what runs by default.  Integer-valued inputs
+    with unit scale make every partial sum exact in fp32 (|sum| <= 8 * max degree < 2^24), so the
+    results must equal torch's index_add bit for bit whatever the summation order; the pruned
+    backward must equal the unpruned backward of the masked gradient."""
+    from eppgcn_amd import graphs, workload
+    g = graphs.make_graph("cfg4_rmat22", device="cuda")
+    n, e = g.num_nodes, g.num_edges
+    wl = workload.prepare(g, 2, 0.1, 2)
+    assert wl.plans and wl.paths[0].plan is not None, "plans are expected at this size"
+    assert int(g.row_pointers[1:].sub(g.row_pointers[:-1]).max()) * 8 < (1 << 24)
+    ones = torch.ones(n, device="cuda")
+    row = g.row_index()
+    col = g.column_index.long()
+    for dim in (16, 22):
+        xi = (graphs.uniform32(6, torch.arange(n * dim, device="cuda")) % 17 - 8).reshape(n, dim).float()
+        want = torch.zeros(n, dim, device="cuda").index_add_(0, row, xi[col])
+        got = api.spmm_forward(xi, g.column_index, ones, wl.part_ptr, wl.part2node, wl.part_size, plan=wl.plans[dim])
+        assert torch.equal(got, want), f"planned forward, width {dim}"
+        del want
+        path = wl.paths[0] if dim == 16 else wl.paths[1]
+        src = wl.ngh_masks[0] if dim == 16 else wl.train_mask
+        dy = xi * src[:, None]
+        pruned = api.ours_backward(dy, path.ids, path.part_pointer, path.edge_list, ones, path.num_parts,
+                                   path.part_size, plan=path.plan)
+        unpruned = api.spmm_forward(dy, g.column_index, ones, wl.part_ptr, wl.part2node, wl.part_size, backward=True,
+                                    plan=wl.plans[dim])
+        assert torch.equal(pruned, unpruned), f"pruned vs unpruned backward, width {dim}"
+        # the kept path is exactly the slots whose column is in the source mask, in CSR order
+        keep = src[col]
+        assert path.valid_len == int(keep.sum())
+        assert torch.equal(path.edge_list[:path.valid_len], g.column_index[keep])
+        assert torch.equal(path.ids[:path.valid_len].long(), row[keep])
+        del keep, dy, pruned, unpruned, xi
