@@ -131,7 +131,7 @@ struct PlanGroups {
 // loads for widths such as 22 whose rows are only 8-byte aligned in the caller's layout.
 __global__ __launch_bounds__(256) void scale_rows_kernel(float* __restrict__ dst, const float* __restrict__ src,
                                                          const float* __restrict__ scale, long long total_vecs,
-                                                         int vecs_per_row, int dim)
+                                                         int vecs_per_row, int dim, bool pairs)
 {
     const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
     for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs; i += stride) {
@@ -140,10 +140,16 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(float* __restrict__ dst
         const float s = scale[r];
         const float* row = src + r * dim;
         float4 v;
-        v.x = c0 + 0 < dim ? s * row[c0 + 0] : 0.f;
-        v.y = c0 + 1 < dim ? s * row[c0 + 1] : 0.f;
-        v.z = c0 + 2 < dim ? s * row[c0 + 2] : 0.f;
-        v.w = c0 + 3 < dim ? s * row[c0 + 3] : 0.f;
+        if (pairs) {                 // even width, 8-byte aligned source: a pair is all in or all out
+            const float2 lo = c0 < dim ? *reinterpret_cast<const float2*>(row + c0) : make_float2(0.f, 0.f);
+            const float2 hi = c0 + 2 < dim ? *reinterpret_cast<const float2*>(row + c0 + 2) : make_float2(0.f, 0.f);
+            v = make_float4(s * lo.x, s * lo.y, s * hi.x, s * hi.y);
+        } else {
+            v.x = c0 + 0 < dim ? s * row[c0 + 0] : 0.f;
+            v.y = c0 + 1 < dim ? s * row[c0 + 1] : 0.f;
+            v.z = c0 + 2 < dim ? s * row[c0 + 2] : 0.f;
+            v.w = c0 + 3 < dim ? s * row[c0 + 3] : 0.f;
+        }
         *reinterpret_cast<float4*>(dst + i * 4) = v;
     }
 }
@@ -155,6 +161,20 @@ __global__ __launch_bounds__(256) void scale_rows_flat_kernel(float* __restrict_
     const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
     for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride)
         dst[i] = scale[i / dim] * src[i];
+}
+
+// Same for rows of a multiple of 4 floats and 16-byte aligned buffers: one float4 per thread.
+__global__ __launch_bounds__(256) void scale_rows_flat4_kernel(float4* dst, const float4* src,
+                                                               const float* __restrict__ scale, long long total_vecs,
+                                                               int vecs_per_row)
+{
+    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+    for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs; i += stride) {
+        const float s = scale[i / vecs_per_row];
+        float4 v = src[i];
+        v.x *= s; v.y *= s; v.z *= s; v.w *= s;
+        dst[i] = v;
+    }
 }
 
 // ---------------------------------------------------------------- kernel
@@ -516,6 +536,15 @@ static int launch_scale_rows(float* dst, const float* src, const float* scale, i
     if (static_cast<long long>(num_nodes) * dim == 0) return kOk;
     if (dst == src || ld_dst == dim) {
         const long long total = static_cast<long long>(num_nodes) * dim;
+        if (dim % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0) {
+            long long blocks = (total / 4 + 255) / 256;
+            if (blocks > 256 * 32) blocks = 256 * 32;
+            hipLaunchKernelGGL(scale_rows_flat4_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
+                               reinterpret_cast<float4*>(dst), reinterpret_cast<const float4*>(src), scale, total / 4,
+                               dim / 4);
+            EPPGCN_HIP(hipGetLastError());
+            return kOk;
+        }
         long long blocks = (total + 255) / 256;
         if (blocks > 256 * 32) blocks = 256 * 32;
         hipLaunchKernelGGL(scale_rows_flat_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, dst, src,
@@ -525,7 +554,7 @@ static int launch_scale_rows(float* dst, const float* src, const float* scale, i
         long long blocks = (vecs + 255) / 256;
         if (blocks > 256 * 32) blocks = 256 * 32;
         hipLaunchKernelGGL(scale_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, dst, src, scale,
-                           vecs, ld_dst / 4, dim);
+                           vecs, ld_dst / 4, dim, dim % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 8 == 0);
     }
     EPPGCN_HIP(hipGetLastError());
     return kOk;
