@@ -11,6 +11,24 @@ from . import gnnadvisor
 from .param import *  # noqa: F401,F403  (the reference's module re-exports its parameter records)
 
 
+def _graph_args(info):
+    """Positional tail of GNNA.forward after (X, W): graph, groups and the three launch hints."""
+    return (info.row_pointers, info.column_index, info.degrees, info.partPtr, info.part2Node, info.partSize,
+            info.dimWorker, info.warpPerBlock)
+
+
+def _marking_args(info, mask):
+    """Arguments of GNNA.mask_forward for one layer."""
+    return (info.part2Node, info.partPtr, info.column_index, mask.src_mask, mask.ngh_mask, mask.backEdgeMask,
+            mask.node_degs, mask.num_layers, mask.layer, mask.blockx, mask.blocky)
+
+
+def _path_args(back):
+    """Positional tail of GNNA.ours_backward after (dY, X, W): the compacted path of the layer."""
+    return (back.id, back.partPointer, back.edgeList, back.degrees, back.partSize, back.numParts, back.layer,
+            back.blockx, back.blocky)
+
+
 class GNNAFunction(torch.autograd.Function):
     """forward: X*W then neighbour-group aggregation; on the first iteration also marks this
     layer's share of the backward path.  backward: pruned aggregation over the compacted path,
@@ -23,31 +41,24 @@ class GNNAFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, X, weight, inputInfo, maskInfo, backInfo, isFirstIter, isBackModeNet, reluInput=False):
-        GNNA = gnnadvisor()
+        ops = gnnadvisor()
         ctx.save_for_backward(X, weight)
-        ctx.inputInfo = inputInfo
-        ctx.backInfo = backInfo
-        ctx.reluInput = bool(reluInput)
+        # the reference keeps these on ctx as well; backward only needs the path record
+        ctx.inputInfo, ctx.backInfo, ctx.reluInput = inputInfo, backInfo, bool(reluInput)
         ctx.partSize, ctx.dimWorker, ctx.warpPerBlock = inputInfo.partSize, inputInfo.dimWorker, inputInfo.warpPerBlock
-        X_prime = GNNA.forward(X, weight, inputInfo.row_pointers, inputInfo.column_index, inputInfo.degrees,
-                               inputInfo.partPtr, inputInfo.part2Node, inputInfo.partSize, inputInfo.dimWorker,
-                               inputInfo.warpPerBlock, relu_input=ctx.reluInput)[0]
+        (aggregated,) = ops.forward(X, weight, *_graph_args(inputInfo), relu_input=ctx.reluInput)
         if isFirstIter and not isBackModeNet:
-            GNNA.mask_forward(inputInfo.part2Node, inputInfo.partPtr, inputInfo.column_index, maskInfo.src_mask,
-                              maskInfo.ngh_mask, maskInfo.backEdgeMask, maskInfo.node_degs, maskInfo.num_layers,
-                              maskInfo.layer, maskInfo.blockx, maskInfo.blocky)
-        return X_prime
+            ops.mask_forward(*_marking_args(inputInfo, maskInfo))
+        return aggregated
 
     @staticmethod
     def backward(ctx, d_output):
-        GNNA = gnnadvisor()
         X, weight = ctx.saved_tensors
-        b = ctx.backInfo
-        need_dx = bool(ctx.needs_input_grad[0])
-        d_input, d_weight = GNNA.ours_backward(d_output.contiguous(), X, weight, b.id, b.partPointer, b.edgeList,
-                                               b.degrees, b.partSize, b.numParts, b.layer, b.blockx, b.blocky,
-                                               need_dx=need_dx, relu_input=ctx.reluInput)
-        return (d_input if need_dx else None), d_weight, None, None, None, None, None, None
+        wants_dx = bool(ctx.needs_input_grad[0])
+        d_input, d_weight = gnnadvisor().ours_backward(d_output.contiguous(), X, weight, *_path_args(ctx.backInfo),
+                                                       need_dx=wants_dx, relu_input=ctx.reluInput)
+        # one gradient slot per forward argument after ctx
+        return (d_input if wants_dx else None, d_weight) + (None,) * 6
 
 
 class GCNConv(torch.nn.Module):
@@ -58,6 +69,7 @@ class GCNConv(torch.nn.Module):
         self.reset_parameters()
 
     def reset_parameters(self):
+        # U(-1/sqrt(out), 1/sqrt(out)), EPPGCN/gcn_conv.py:47-49
         bound = 1.0 / math.sqrt(self.weights.size(1))
         with torch.no_grad():
             self.weights.uniform_(-bound, bound)

@@ -1,26 +1,31 @@
-"""Launch-parameter records the layer passes to the ops; the attribute names are the ones the
-reference's autograd function reads (EPPGCN/gcn_conv.py:13-14,21-27,36-38; records defined in
-EPPGCN/param.py).  The integers are hints sized for 32-lane warps: the HIP library picks its own
-wave64 mapping from the feature width and only requires them to be positive, so they are kept
-for signature compatibility and for reporting."""
+"""Launch-parameter records the layer passes to the ops.  The attribute names are the ones the
+reference's autograd function reads (EPPGCN/gcn_conv.py:13-14,21-27,36-38; the records are
+defined in EPPGCN/param.py).  The integers are hints sized for 32-lane warps: the HIP library
+picks its own wave64 mapping from the feature width and only requires them to be positive, so
+they are kept for signature compatibility and for reporting."""
 from __future__ import annotations
+
+# upper bounds of the feature width -> (lanes per group, groups per block); 64 threads each,
+# i.e. one wavefront (table of EPPGCN/param.py:6-24)
+_BLOCK_SHAPES = ((8, (2, 32)), (32, (4, 16)), (96, (8, 8)), (192, (16, 4)))
 
 
 def getBlockSize(dim):
-    """(lanes per group, groups per block) for a feature width; always 64 threads, i.e. one
-    wavefront (table of EPPGCN/param.py:6-24)."""
-    if dim < 8:
-        return 2, 32
-    if dim < 32:
-        return 4, 16
-    if dim < 96:
-        return 8, 8
-    if dim < 192:
-        return 16, 4
+    for below, shape in _BLOCK_SHAPES:
+        if dim < below:
+            return shape
     return 32, 2
 
 
-class inputProperty(object):
+class _Record(object):
+    """Attribute bag: every keyword becomes an attribute of the same name."""
+
+    def _take(self, **fields):
+        for name, value in fields.items():
+            setattr(self, name, value)
+
+
+class inputProperty(_Record):
     """Forward-side inputs: CSR, scale vector, neighbour groups and launch hints."""
 
     MAX_warpPerBlock = 8
@@ -31,26 +36,22 @@ class inputProperty(object):
                  verbose=False):
         if dataset_obj is None:
             raise ValueError("Dataset object MUST SET !!!")
-        self.dataset_obj = dataset_obj
-        self.row_pointers = row_pointers
-        self.column_index = column_index
-        self.degrees = degrees
-        self.num_nodes = dataset_obj.num_nodes
-        self.avgNodeDegree = dataset_obj.avg_degree
-        self.avgEdgeSpan = getattr(dataset_obj, "avg_edgeSpan", -1)
-        self.partSize = partSize
-        self.dimWorker = dimWorker
-        self.warpPerBlock = warpPerBlock
-        self.dimWorker_input = self.dimWorker_hidden = dimWorker
-        self.warpPerBlock_input = self.warpPerBlock_hidden = warpPerBlock
-        self.inputDim = dataset_obj.num_features
-        self.hiddenDim = hiddenDim
-        self.manual_mode = manual_mode
-        self.verbose_flag = verbose
-        self.state_set_input = False
-        self.share_memory = (sharedMem if sharedMem is not None else 100) * 0.4
-        self.partPtr = None
-        self.part2Node = None
+        self._take(dataset_obj=dataset_obj, row_pointers=row_pointers, column_index=column_index, degrees=degrees,
+                   partSize=partSize, dimWorker=dimWorker, warpPerBlock=warpPerBlock, hiddenDim=hiddenDim,
+                   manual_mode=manual_mode, verbose_flag=verbose, partPtr=None, part2Node=None,
+                   state_set_input=False)
+        self._take(num_nodes=dataset_obj.num_nodes, avgNodeDegree=dataset_obj.avg_degree,
+                   avgEdgeSpan=getattr(dataset_obj, "avg_edgeSpan", -1), inputDim=dataset_obj.num_features)
+        # per-layer-kind hints chosen by decider(); set_input() / set_hidden() select one pair
+        self._take(dimWorker_input=dimWorker, dimWorker_hidden=dimWorker, warpPerBlock_input=warpPerBlock,
+                   warpPerBlock_hidden=warpPerBlock)
+        self.share_memory = 0.4 * (100 if sharedMem is None else sharedMem)
+
+    def _warps_for(self, width):
+        """Warps per block from the reference's shared-memory estimate, between 1 and 8."""
+        per_warp = 4 * (self.partSize + width)
+        estimate_kb = min(self.MAX_warpPerBlock * (per_warp + 4 * self.gap_smem) / 1e3, self.share_memory)
+        return max(1, min(int(estimate_kb * 1e3 / per_warp), self.MAX_warpPerBlock))
 
     def decider(self):
         """The reference's rule (EPPGCN/param.py:72-127): group size = int(average degree), warps per
@@ -60,72 +61,49 @@ class inputProperty(object):
         build_part)."""
         if not (self.manual_mode and self.partSize):
             self.partSize = max(1, int(self.avgNodeDegree))
-        kb_in = self.MAX_warpPerBlock * (self.partSize * 4 + self.inputDim * 4 + self.gap_smem * 4) / 1e3
-        kb_hid = self.MAX_warpPerBlock * (self.partSize * 4 + self.hiddenDim * 4 + self.gap_smem * 4) / 1e3
-        kb_in, kb_hid = min(kb_in, self.share_memory), min(kb_hid, self.share_memory)
-        self.warpPerBlock_input = max(1, min(int(kb_in * 1e3 / (self.partSize * 4 + self.inputDim * 4)),
-                                             self.MAX_warpPerBlock))
-        self.warpPerBlock_hidden = max(1, min(int(kb_hid * 1e3 / (self.partSize * 4 + self.hiddenDim * 4)),
-                                              self.MAX_warpPerBlock))
-        self.dimWorker_input = min(self.inputDim, 32)
-        self.dimWorker_hidden = min(self.hiddenDim, 32)
+        self._take(warpPerBlock_input=self._warps_for(self.inputDim),
+                   warpPerBlock_hidden=self._warps_for(self.hiddenDim),
+                   dimWorker_input=min(self.inputDim, 32), dimWorker_hidden=min(self.hiddenDim, 32))
         if self.verbose_flag:
             print("\n=> AUTO Decider Complete !!!\n")
 
-    def set_input(self):
-        self.dimWorker = self.dimWorker_input
-        self.warpPerBlock = self.warpPerBlock_input
-        self.state_set_input = True
+    def _select(self, which):
+        self._take(dimWorker=getattr(self, "dimWorker_" + which), warpPerBlock=getattr(self, "warpPerBlock_" + which),
+                   state_set_input=(which == "input"))
         return self
+
+    def set_input(self):
+        return self._select("input")
 
     def set_hidden(self):
-        self.dimWorker = self.dimWorker_hidden
-        self.warpPerBlock = self.warpPerBlock_hidden
-        self.state_set_input = False
-        return self
+        return self._select("hidden")
 
     def print_param(self):
-        if self.verbose_flag:
-            mode = "manual" if self.manual_mode else "auto"
-            which = "INPUT" if self.state_set_input else "HIDDEN"
-            print("# {} {} partSize: {}".format(mode, which, self.partSize))
-            print("# {} {} dimWorker: {}".format(mode, which, self.dimWorker))
-            print("# {} {} warpPerBlock: {}".format(mode, which, self.warpPerBlock))
+        if not self.verbose_flag:
+            return
+        tag = "{} {}".format("manual" if self.manual_mode else "auto", "INPUT" if self.state_set_input else "HIDDEN")
+        for name in ("partSize", "dimWorker", "warpPerBlock"):
+            print("# {} {}: {}".format(tag, name, getattr(self, name)))
 
 
-class maskInputProperty(object):
+class maskInputProperty(_Record):
     """Inputs of one path-marking step (one per layer, first iteration only)."""
 
     def __init__(self, src_mask=None, ngh_mask=None, backEdgeMask=None, node_degs=None, num_layers=None,
                  layer=None, dim=None):
-        self.src_mask = src_mask
-        self.ngh_mask = ngh_mask
-        self.backEdgeMask = backEdgeMask
-        self.node_degs = node_degs
-        self.num_layers = num_layers
-        self.layer = layer
-        self.blockx, self.blocky = getBlockSize(dim)
-        self.dim = dim
+        blockx, blocky = getBlockSize(dim)
+        self._take(src_mask=src_mask, ngh_mask=ngh_mask, backEdgeMask=backEdgeMask, node_degs=node_degs,
+                   num_layers=num_layers, layer=layer, dim=dim, blockx=blockx, blocky=blocky)
 
 
-class backInputProperty(object):
+class backInputProperty(_Record):
     """The compacted backward path of one layer, filled in after path preparation."""
 
     def __init__(self, id=None, partPointer=None, edgeList=None, degrees=None, partSize=None, numParts=None,
                  dim=None, layer=None):
-        self.id = id
-        self.partPointer = partPointer
-        self.edgeList = edgeList
-        self.degrees = degrees
-        self.partSize = partSize
-        self.numParts = numParts
-        self.dim = dim
-        self.layer = layer
-        self.blockx, self.blocky = getBlockSize(dim)
+        blockx, blocky = getBlockSize(dim)
+        self._take(degrees=degrees, dim=dim, layer=layer, blockx=blockx, blocky=blocky)
+        self.fillProperty(id, partPointer, edgeList, partSize, numParts)
 
     def fillProperty(self, id=None, partPointer=None, edgeList=None, partSize=None, numParts=None):
-        self.id = id
-        self.partPointer = partPointer
-        self.edgeList = edgeList
-        self.partSize = partSize
-        self.numParts = numParts
+        self._take(id=id, partPointer=partPointer, edgeList=edgeList, partSize=partSize, numParts=numParts)
