@@ -338,3 +338,31 @@ def test_module_mark_compact_equals_the_two_reference_steps(GNNA):
     id_b, el_b, info_b = GNNA.mark_compact(p2n, pp, dev(col), dev(src), ngh_b, degs_b, 2, 1)
     assert torch.equal(id_a, id_b) and torch.equal(el_a, el_b) and float(info_a[0]) == float(info_b[0])
     assert torch.equal(ngh_a, ngh_b) and torch.equal(degs_a, degs_b)
+
+
+def test_epoch_replayed_from_a_hip_graph_follows_the_eager_trajectory(GNNA):
+    """One whole training epoch (layer ops, loss, backward, Adam) captured into a HIP graph: every
+    replay, with eager work and synchronisations in between, gives the loss of the eager trainer
+    at the same step."""
+    from eppgcn_amd import graphs, train
+    g = graphs.make_graph("cfg2_chunglu", device="cuda")
+    mask = graphs.bernoulli_mask(g.num_nodes, 0.1, 2, "cuda")
+    eager = train.Trainer(g, train_mask=mask, labels="uniform")
+    graphed = train.Trainer(g, train_mask=mask, labels="uniform")
+    for tr in (eager, graphed):
+        for i in range(4):
+            tr.train_step(i == 0)
+    graph, loss = graphed.capture_epoch()          # three more eager epochs on a side stream, then the capture
+    for _ in range(3):
+        eager.train_step(False)
+    for step in range(6):
+        want = float(eager.train_step(False))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = float(loss)
+        assert abs(got - want) <= 1e-5 * abs(want), f"replay {step}: {got} vs {want}"
+        _ = torch.randn(512, 512, device="cuda") @ torch.randn(512, 512, device="cuda")   # unrelated eager work
+        torch.cuda.synchronize()
+    w_e = eager.model.convs[0].weights.detach()
+    w_g = graphed.model.convs[0].weights.detach()
+    assert torch.allclose(w_e, w_g, rtol=1e-4, atol=1e-6)
