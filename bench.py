@@ -299,18 +299,25 @@ def cpu_baseline(args, g, wl, x16, x22, dy22, dy16, bytes_epoch):
     host = {k: v.cpu().numpy() for k, v in (("x16", x16), ("x22", x22), ("dy22", dy22), ("dy16", dy16))}
     paths = [(p.ids.cpu().numpy(), p.part_pointer.cpu().numpy(), p.edge_list.cpu().numpy(), p.num_parts)
              for p in wl.paths]
-    t0 = time.perf_counter()
-    co.spmm_groups(host["x16"], col, s, pp, p2n, n, threads=True)
-    co.spmm_groups(host["x22"], col, s, pp, p2n, n, threads=True)
-    ids, bpp, el, npb = paths[1]
-    co.ours_backward(host["dy22"], ids, bpp, el, s, npb, threads=True)
-    ids, bpp, el, npb = paths[0]
-    co.ours_backward(host["dy16"], ids, bpp, el, s, npb, threads=True)
-    dt = time.perf_counter() - t0
+    def epoch():
+        co.spmm_groups(host["x16"], col, s, pp, p2n, n, threads=True)
+        co.spmm_groups(host["x22"], col, s, pp, p2n, n, threads=True)
+        ids, bpp, el, npb = paths[1]
+        co.ours_backward(host["dy22"], ids, bpp, el, s, npb, threads=True)
+        ids, bpp, el, npb = paths[0]
+        co.ours_backward(host["dy16"], ids, bpp, el, s, npb, threads=True)
+
+    # bounded sample: whole epochs for about 10 s (at least 1 after a first, untimed one; at most 12)
+    epoch()
+    done, t0 = 0, time.perf_counter()
+    while done < 12 and (done == 0 or time.perf_counter() - t0 < 10.0):
+        epoch()
+        done += 1
+    dt = (time.perf_counter() - t0) / done
     return {"value": round(bytes_epoch / dt / 1e9, 2), "unit": "GB/s", "cores": co.num_threads(), "kind": "port",
             "ms_per_epoch": round(dt * 1e3, 1),
-            "sample": f"one epoch (4 aggregations) of {args.config}, OpenMP C restatement, "
-                      f"{co.num_threads()} threads of {os.cpu_count()} host cpus"}
+            "sample": f"mean of {done} whole epochs (4 aggregations each) of {args.config} after one untimed epoch, "
+                      f"OpenMP C restatement, {co.num_threads()} threads of {os.cpu_count()} host cpus"}
 
 
 if __name__ == "__main__":
