@@ -32,7 +32,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="cfg4_rmat22",
-                    choices=["cfg1_uniform", "cfg2_chunglu", "cfg3_rmat20", "cfg4_rmat22"])
+                    help="cfg1_uniform, cfg2_chunglu, cfg3_rmat20, cfg4_rmat22 (the metric's configuration), or "
+                         "rmat:<scale>:<pairs per vertex> for an R-MAT graph of another size")
     ap.add_argument("--train_ratio", type=float, default=0.1)
     ap.add_argument("--backsize_mode", default="constant", choices=["constant", "map", "threshold"])
     ap.add_argument("--backsize", type=int, default=32)

@@ -269,4 +269,9 @@ CONFIGS = {
 
 
 def make_graph(name: str, device="cpu", scale_mode: str = "inv_sqrt") -> Graph:
+    """A named benchmark configuration, or ``rmat:<scale>:<pairs per vertex>`` for an R-MAT graph
+    of another size (same generator and seed as the named ones), e.g. ``rmat:24:16``."""
+    if name.startswith("rmat:"):
+        _, scale, factor = name.split(":")
+        return rmat_graph(int(scale), int(factor), seed=0, device=device, scale_mode=scale_mode)
     return CONFIGS[name](device=device, scale_mode=scale_mode)
