@@ -392,6 +392,7 @@ __global__ __launch_bounds__(256) void ginfo_hist_kernel(const int* __restrict__
 constexpr int kSplitBlock = 256;
 constexpr int kSplitItems = 8;
 constexpr int kSplitTile = kSplitBlock * kSplitItems;
+constexpr int kSmallGroups = 4;     // groups per vertex up to which the owning thread writes them itself
 
 template <bool kFromRowPtr>
 __global__ __launch_bounds__(kSplitBlock) void split_groups_kernel(
@@ -403,6 +404,8 @@ __global__ __launch_bounds__(kSplitBlock) void split_groups_kernel(
     __shared__ int s_g[kSplitTile];
     __shared__ uint64_t s_wave[kSplitBlock / kWave];
     __shared__ uint64_t s_tile_excl;
+    __shared__ int s_big[kSplitTile];
+    __shared__ int s_big_count;
     const int tile = acquire_tile(st, &s_tile);
     if (tile >= num_tiles) return;
     const int lane = threadIdx.x & (kWave - 1);
@@ -451,21 +454,45 @@ __global__ __launch_bounds__(kSplitBlock) void split_groups_kernel(
         run += (static_cast<uint64_t>(q[j]) << 31) | static_cast<uint64_t>(g[j]);
     }
     const int tile_q = static_cast<int>(tile_total >> 31);
-    if (threadIdx.x == 0) s_q[kSplitTile] = tile_q;
+    if (threadIdx.x == 0) {
+        s_q[kSplitTile] = tile_q;
+        s_big_count = 0;
+    }
     __syncthreads();
 
-    for (int o = threadIdx.x; o < tile_q; o += kSplitBlock) {
-        // last slot with s_q[slot] <= o
-        int lo = 0, hi = kSplitTile;
-        while (lo < hi) {
-            const int mid = (lo + hi + 1) >> 1;
-            if (s_q[mid] <= o) lo = mid; else hi = mid - 1;
+    // A vertex with at most kSmallGroups groups is written by the thread that owns it; the others
+    // go on a list and are written by whole waves, 64 groups per step, so that a tile full of hubs
+    // (the first vertices of an R-MAT graph have 10^5 groups each) costs coalesced stores only.
+#pragma unroll
+    for (int j = 0; j < kSplitItems; ++j) {
+        const int slot = threadIdx.x * kSplitItems + j;
+        if (q[j] > kSmallGroups) {
+            s_big[atomicAdd(&s_big_count, 1)] = slot;
+        } else {
+            const int start = s_g[slot];
+            const long long first = static_cast<long long>(q_base) + s_q[slot];
+            for (int k = 0; k < q[j]; ++k) {
+                const long long dst = first + k;
+                if (dst < capacity) {
+                    part_ptr_out[dst] = start + k * part_size;
+                    if (part2node_out && dst + 1 < capacity) part2node_out[dst] = static_cast<int>(base) + slot;
+                }
+            }
         }
-        const int j = o - s_q[lo];
-        const long long dst = static_cast<long long>(q_base) + o;
-        if (dst < capacity) {
-            part_ptr_out[dst] = s_g[lo] + j * part_size;
-            if (part2node_out && dst + 1 < capacity) part2node_out[dst] = static_cast<int>(base) + lo;
+    }
+    __syncthreads();
+    const int big = s_big_count;
+    for (int b = wave; b < big; b += kSplitBlock / kWave) {
+        const int slot = s_big[b];
+        const int count = s_q[slot + 1] - s_q[slot];
+        const int start = s_g[slot];
+        const long long first = static_cast<long long>(q_base) + s_q[slot];
+        for (int k = lane; k < count; k += kWave) {
+            const long long dst = first + k;
+            if (dst < capacity) {
+                part_ptr_out[dst] = start + k * part_size;
+                if (part2node_out && dst + 1 < capacity) part2node_out[dst] = static_cast<int>(base) + slot;
+            }
         }
     }
     if (tile == num_tiles - 1 && threadIdx.x == 0) {
