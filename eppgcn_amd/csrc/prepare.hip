@@ -95,15 +95,17 @@ __global__ __launch_bounds__(kMaskBlock) void mask_forward_kernel(
             kept += __popcll(ballot & below_hi & ~((1ull << lo) - 1ull));
         }
     }
-    // groups of one row sit in adjacent lanes: suffix sums within a run of equal rows
+    // adjacent lanes whose groups belong to one row form a run: suffix sums within a run, then one
+    // atomic per run.  A lane absorbs the lane `off` above only if no run starts in between.
+    const int prev_row = __shfl_up(row, 1, kWave);
+    const uint64_t heads = __ballot(lane == 0 || prev_row != row);
 #pragma unroll
     for (int off = 1; off < kWave; off <<= 1) {
         const int other = __shfl_down(kept, off, kWave);
-        const int other_row = __shfl_down(row, off, kWave);
-        if (lane + off < kWave && other_row == row) kept += other;
+        const uint64_t between = (heads >> 1 >> lane) & ((1ull << off) - 1ull);   // lanes lane+1 .. lane+off
+        if (lane + off < kWave && between == 0) kept += other;
     }
-    const int prev_row = __shfl_up(row, 1, kWave);
-    if (lane < ng && (lane == 0 || prev_row != row) && kept > 0) atomicAdd(node_degs + row, kept);
+    if (lane < ng && ((heads >> lane) & 1ull) && kept > 0) atomicAdd(node_degs + row, kept);
 }
 
 // ================================================================ compaction

@@ -628,3 +628,36 @@ def test_rmat22_headline_size_exact_integer_sums_with_plans(api):
         assert torch.equal(path.edge_list[:path.valid_len], g.column_index[keep])
         assert torch.equal(path.ids[:path.valid_len].long(), row[keep])
         del keep, dy, pruned, unpruned, xi
+
+
+@pytest.mark.parametrize("name", ["small", "hub", "medium"])
+def test_marking_with_empty_groups_in_the_group_arrays(api, name):
+    """Caller-made group arrays may hold empty groups (two groups starting at the same slot);
+    build_part never makes them, so this is the only test of the owner search both marking kernels
+    fall back to.  Empty groups carry arbitrary rows, which must not be marked or counted."""
+    indptr, col = GRAPHS[name]()
+    n = indptr.size - 1
+    rng = np.random.default_rng(12)
+    pp, p2n = co.build_part(6, indptr)
+    where = np.sort(rng.integers(0, p2n.size + 1, size=max(3, p2n.size // 7)))
+    pp2 = np.insert(pp, where, pp[where]).astype(np.int32)            # duplicate starts = empty groups
+    p2n2 = np.insert(p2n, where, rng.integers(0, n, where.size)).astype(np.int32)
+    assert np.all(np.diff(pp2) >= 0) and (np.diff(pp2) == 0).sum() == where.size
+    src = rng.random(n) < 0.3
+    for is_last in (False, True):
+        want_ngh = np.zeros(n, bool)
+        want_bem = np.full(col.size, -1, np.int32)
+        want_degs = np.zeros(n, np.int32)
+        co.mask_forward(p2n2, pp2, col, src, None if is_last else want_ngh, want_bem, want_degs, is_last)
+        want_id, want_edge, want_v = co.compact_mask(want_bem, col)
+        ngh = torch.zeros(n, dtype=torch.bool, device="cuda")
+        bem = torch.full((col.size,), -1, dtype=torch.int32, device="cuda")
+        degs = torch.zeros(n, dtype=torch.int32, device="cuda")
+        api.mask_forward(dev(p2n2), dev(pp2), dev(col), dev(src), None if is_last else ngh, bem, degs, is_last)
+        assert np.array_equal(bem.cpu().numpy(), want_bem) and np.array_equal(degs.cpu().numpy(), want_degs)
+        assert np.array_equal(ngh.cpu().numpy(), want_ngh)
+        ngh2 = torch.zeros(n, dtype=torch.bool, device="cuda")
+        degs2 = torch.zeros(n, dtype=torch.int32, device="cuda")
+        oid, oedge, v = api.mark_compact(dev(p2n2), dev(pp2), dev(col), dev(src), None if is_last else ngh2, degs2, is_last)
+        assert v == want_v and np.array_equal(oid.cpu().numpy(), want_id) and np.array_equal(oedge.cpu().numpy(), want_edge)
+        assert np.array_equal(degs2.cpu().numpy(), want_degs) and np.array_equal(ngh2.cpu().numpy(), want_ngh)
