@@ -661,3 +661,32 @@ def test_marking_with_empty_groups_in_the_group_arrays(api, name):
         oid, oedge, v = api.mark_compact(dev(p2n2), dev(pp2), dev(col), dev(src), None if is_last else ngh2, degs2, is_last)
         assert v == want_v and np.array_equal(oid.cpu().numpy(), want_id) and np.array_equal(oedge.cpu().numpy(), want_edge)
         assert np.array_equal(degs2.cpu().numpy(), want_degs) and np.array_equal(ngh2.cpu().numpy(), want_ngh)
+
+
+@pytest.mark.parametrize("name", ["small", "hub", "medium"])
+@pytest.mark.parametrize("dim", [16, 22, 70])
+def test_aggregation_with_empty_groups(api, name, dim):
+    """Empty groups (two groups starting at the same slot) that name the row of the group after
+    them keep a row's groups consecutive, which is all the aggregation requires; they add nothing."""
+    indptr, col = GRAPHS[name]()
+    n = indptr.size - 1
+    s = scale_inv_sqrt(indptr)
+    rng = np.random.default_rng(14)
+    pp, p2n = co.build_part(5, indptr)
+    where = np.sort(rng.integers(0, p2n.size, size=max(3, p2n.size // 5)))
+    pp2 = np.insert(pp, where, pp[where]).astype(np.int32)
+    p2n2 = np.insert(p2n, where, p2n[where]).astype(np.int32)
+    x = rng.standard_normal((n, dim)).astype(np.float32)
+    want = co.spmm_f64(x, indptr, col, s)
+    bound = co.spmm_f64(np.abs(x), indptr, col, s) + 1e-30
+    for workspace in (True, None):
+        got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp2), dev(p2n2), part_size=5, workspace=workspace)
+        assert_close(got.cpu().numpy(), want, bound, f"empty groups, workspace={workspace}")
+    plan = api.build_plan(dev(pp2), dev(col), p2n2.size, col.size, n, dim, part2node=dev(p2n2))
+    api.set_plan_shift(9)
+    try:
+        plan = api.build_plan(dev(pp2), dev(col), p2n2.size, col.size, n, dim, part2node=dev(p2n2))
+    finally:
+        api.set_plan_shift(0)
+    got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp2), dev(p2n2), part_size=5, plan=plan)
+    assert_close(got.cpu().numpy(), want, bound, "empty groups with a plan")
