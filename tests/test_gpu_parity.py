@@ -690,3 +690,37 @@ def test_aggregation_with_empty_groups(api, name, dim):
         api.set_plan_shift(0)
     got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp2), dev(p2n2), part_size=5, plan=plan)
     assert_close(got.cpu().numpy(), want, bound, "empty groups with a plan")
+
+
+@pytest.mark.parametrize("dim", [16, 22, 7, 64])
+@pytest.mark.parametrize("shift_in,shift_out", [(1, 0), (0, 1), (1, 1), (2, 3)])
+def test_aggregation_with_misaligned_feature_buffers(api, dim, shift_in, shift_out):
+    """Feature and output matrices that start 4, 8 or 12 bytes into an allocation (views of larger
+    tensors) take the narrower vector paths; with and without a workspace, forward and pruned."""
+    indptr, col = GRAPHS["medium"]()
+    n = indptr.size - 1
+    s = scale_inv_sqrt(indptr)
+    rng = np.random.default_rng(16)
+    x = rng.standard_normal((n, dim)).astype(np.float32)
+    want = co.spmm_f64(x, indptr, col, s)
+    bound = co.spmm_f64(np.abs(x), indptr, col, s) + 1e-30
+    pp, p2n = api.build_part(8, dev(indptr), col.size)
+    xin = torch.empty(n * dim + 4, device="cuda")[shift_in: shift_in + n * dim].view(n, dim)
+    xin.copy_(dev(x))
+    out = torch.empty(n * dim + 4, device="cuda")[shift_out: shift_out + n * dim].view(n, dim)
+    assert xin.data_ptr() % 16 == 4 * shift_in and out.data_ptr() % 16 == 4 * shift_out
+    for workspace in (True, None):
+        out.fill_(3.0)
+        api.spmm_forward(xin, dev(col), dev(s), pp, p2n, part_size=8, out=out, workspace=workspace)
+        assert_close(out.cpu().numpy(), want, bound, f"forward, workspace={workspace}")
+    src = rng.random(n) < 0.4
+    degs = torch.zeros(n, dtype=torch.int32, device="cuda")
+    ids, edge_list, v = api.mark_compact(p2n, pp, dev(col), dev(src), None, degs, True)
+    bpp, p, _ = api.split_back_part(degs, col.size, 8)
+    xm = x * src[:, None]
+    xin.copy_(dev(xm))
+    want_b = co.spmm_f64(xm, indptr, col, s)
+    for workspace in (True, None):
+        out.fill_(3.0)
+        api.ours_backward(xin, ids, bpp, edge_list, dev(s), p, 8, out=out, workspace=workspace)
+        assert_close(out.cpu().numpy(), want_b, bound, f"pruned backward, workspace={workspace}")
