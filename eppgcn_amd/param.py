@@ -17,6 +17,13 @@ def getBlockSize(dim):
     return 32, 2
 
 
+# Smallest automatic forward group size.  The reference's rule, int(average degree), was tuned for
+# one 32-lane warp walking a group serially; a wave64 team gathers 8 rows at a time, and groups
+# below about 16 slots leave most of that depth unused (R-MAT scale 20, average degree 8.8:
+# group size 8 / 16 / 32 -> 0.245 / 0.214 / 0.212 ms per width-22 forward launch).
+MIN_AUTO_PART_SIZE = 16
+
+
 class _Record(object):
     """Attribute bag: every keyword becomes an attribute of the same name."""
 
@@ -57,10 +64,10 @@ class inputProperty(_Record):
         """The reference's rule (EPPGCN/param.py:72-127): group size = int(average degree), warps per
         block from a shared-memory estimate capped at 8, dimension workers = min(width, 32).
         Unlike the reference, a manual group size is respected in manual mode and the automatic
-        one never drops below 1 (an average degree below 1 would otherwise divide by zero in
-        build_part)."""
+        one never drops below MIN_AUTO_PART_SIZE (the reference's can reach 0, which divides by
+        zero in build_part)."""
         if not (self.manual_mode and self.partSize):
-            self.partSize = max(1, int(self.avgNodeDegree))
+            self.partSize = max(MIN_AUTO_PART_SIZE, int(self.avgNodeDegree))
         self._take(warpPerBlock_input=self._warps_for(self.inputDim),
                    warpPerBlock_hidden=self._warps_for(self.hiddenDim),
                    dimWorker_input=min(self.inputDim, 32), dimWorker_hidden=min(self.hiddenDim, 32))

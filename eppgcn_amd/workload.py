@@ -12,7 +12,7 @@ from typing import List
 
 import torch
 
-from . import capi, graphs
+from . import capi, graphs, param
 
 
 @dataclasses.dataclass
@@ -68,7 +68,8 @@ def prepare(graph: graphs.Graph, num_layers: int = 2, train_ratio: float = 0.1, 
     n, e = g.num_nodes, g.num_edges
     if plan is None:             # default: plans where the feature table outgrows the caches
         plan = capi.plan_recommended(n, max(widths))
-    ps = part_size or max(1, int(g.avg_degree))       # EPPGCN/param.py:80
+    # EPPGCN/param.py:80 takes int(average degree); the floor is the wave64 re-fit of that rule
+    ps = part_size or max(param.MIN_AUTO_PART_SIZE, int(g.avg_degree))
     part_ptr, part2node = capi.build_part(ps, g.row_pointers, e)
     if train_mask is None:
         train_mask = graphs.bernoulli_mask(n, train_ratio, mask_seed, dev)

@@ -85,7 +85,7 @@ def test_decider_rules():
     ds.avg_degree = 0.4
     info = param.inputProperty(None, None, None, 32, 32, 8, 100, hiddenDim=16, dataset_obj=ds, manual_mode=False)
     info.decider()
-    assert info.partSize == 1                      # never 0
+    assert info.partSize == param.MIN_AUTO_PART_SIZE == 16     # never 0: the wave64 floor
     info = param.inputProperty(None, None, None, 5, 32, 8, 100, hiddenDim=16, dataset_obj=_DS(), manual_mode=True)
     info.decider()
     assert info.partSize == 5                      # manual group size respected
