@@ -124,6 +124,13 @@ class Trainer:
             self.back_props[i].fillProperty(ids, part_pointer, edge_list, part_size, int(num_parts[0].item()))
             ds.edge_masks[i] = None      # the marking buffer is not needed after compaction
 
+    def _loss(self, out):
+        """Mean negative log-likelihood of the training rows (F.nll_loss of F.log_softmax,
+        EPPGCN/gcn_main.py:252-253).  Written as a gather and a mean: torch's nll_loss kernels
+        reduce all rows in one workgroup (0.53 + 0.33 ms per epoch for 4.2e5 rows here)."""
+        logp = F.log_softmax(out.index_select(0, self.train_idx), dim=1)
+        return -logp.gather(1, self.train_y.unsqueeze(1)).mean()
+
     def train_step(self, is_first_iter: bool, record_loss: bool = False, phase_timers: bool = True):
         """One epoch.  ``phase_timers`` keeps the reference's three host synchronisations per epoch
         that split the time into forward / loss / backward (EPPGCN/gcn_main.py:242,254,260); without
@@ -148,7 +155,7 @@ class Trainer:
         if self.train_idx is None:
             self.train_idx = ds.train_mask.nonzero().squeeze(1)
             self.train_y = ds.y[self.train_idx]
-        loss = F.nll_loss(F.log_softmax(out.index_select(0, self.train_idx), dim=1), self.train_y)
+        loss = self._loss(out)
         sync()
         self.loss_time += time.perf_counter() - t
         t = time.perf_counter()
@@ -211,7 +218,7 @@ class Trainer:
         def epoch():
             self.optimizer.zero_grad(set_to_none=True)
             out = self.model(ds.x, self.inputInfo, self.mask_props, self.back_props, False, False)
-            loss = F.nll_loss(F.log_softmax(out.index_select(0, self.train_idx), dim=1), self.train_y)
+            loss = self._loss(out)
             loss.backward()
             self.optimizer.step()
             return loss
