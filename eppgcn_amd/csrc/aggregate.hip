@@ -39,7 +39,7 @@ namespace eppgcn {
 
 constexpr int kAggBlock = 256;
 constexpr int kAggWaves = kAggBlock / kWave;
-constexpr int kStageCap = 512;   // staged slots per wave and pass
+constexpr int kStageCap = 1024;  // slots of the staged window of a wave
 // Staged slot s lives at LDS word s + s/32: teams read their groups at strides that are
 // often a power of two (a backward group size of 32 puts all 16 teams of a wave on one bank);
 // one pad word per 32 slots spreads such strides over the 32 banks.
@@ -201,6 +201,8 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
     using V = Vec<VW>;
     __shared__ int stage_col[kAggWaves][kStageWords];
     __shared__ float stage_scale[kAggWaves][kPrescaled ? 1 : kStageWords];
+    __shared__ int meta_int[kAggWaves][4][kWave];      // first slot, end slot, row, flags of the wave's groups
+    __shared__ float meta_scale[kAggWaves][kWave];     // scale of the group's row
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
@@ -208,7 +210,43 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
     const int tl = lane % TS;
     int* my_col = stage_col[wave];
     float* my_scale = stage_scale[wave];
+    int* m_beg = meta_int[wave][0];
+    int* m_end = meta_int[wave][1];
+    int* m_row = meta_int[wave][2];
+    int* m_flags = meta_int[wave][3];
+    float* m_scale = meta_scale[wave];
     const long long wave_first = (static_cast<long long>(blockIdx.x) * kAggWaves + wave) * TPW * rounds;
+    if (wave_first >= num_parts) return;                   // wave-uniform; the LDS rows are wave-private
+    // the wave's groups (TPW * rounds <= 64 of them): one group per lane loads its description once,
+    // so that the rounds below start from LDS instead of from a chain of dependent global loads
+    const int ng = static_cast<int>(min(static_cast<long long>(TPW) * rounds, num_parts - wave_first));
+    {
+        int gb = 0, ge = 0, rw = 0, fl = 0;
+        float sr = 0.f;
+        if (lane < ng) {
+            const int p = static_cast<int>(wave_first) + lane;
+            gb = groups.part_ptr[p];
+            ge = groups.part_ptr[p + 1];
+            if (ge > gb) {
+                rw = groups.row_of(p, gb);
+                const bool prev = groups.has_prev(p, rw, gb);
+                const bool next = groups.has_next(p, rw, ge, num_parts);
+                fl = 16 | (prev ? 1 : 0) | (next ? 2 : 0) | (groups.joins_left(p, prev) ? 4 : 0) |
+                     (groups.joins_right(p, next) ? 8 : 0);
+                sr = scale[rw];
+            }
+        }
+        m_beg[lane] = gb;
+        m_end[lane] = ge;
+        m_row[lane] = rw;
+        m_flags[lane] = fl;
+        m_scale[lane] = sr;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int slots_end = m_end[ng - 1];                   // end of the slot range of the wave's groups
+    int win_beg = 0, win_end = 0;                          // staged window [win_beg, win_end), wave-uniform
 
     V carry[CPL];                // partial sum of the run that continues from the previous round (team 0)
     bool carry_valid = false;    // wave-uniform
@@ -220,26 +258,24 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
         for (int j = 0; j < VW; ++j) carry[k].v[j] = 0.f;
 
     for (int round = 0; round < rounds; ++round) {
-        const long long p0 = wave_first + static_cast<long long>(round) * TPW;
-        if (p0 >= num_parts) break;                          // wave-uniform
-        const int np = min(TPW, static_cast<int>(num_parts - p0));
-        const int p = static_cast<int>(p0) + team;
+        const int g0 = round * TPW;
+        if (g0 >= ng) break;                                 // wave-uniform
+        const int np = min(TPW, ng - g0);
         const bool active = team < np;
-        const bool more_rounds = round + 1 < rounds && p0 + TPW < num_parts;
+        const bool more_rounds = round + 1 < rounds && g0 + TPW < ng;
 
-        int gbeg = 0, gend = 0, row = 0;
+        int gbeg = 0, gend = 0, row = 0, flags = 0;
         float s_row = 0.f;
         if (active) {
-            gbeg = groups.part_ptr[p];
-            gend = groups.part_ptr[p + 1];
-            if (gend > gbeg) {
-                row = groups.row_of(p, gbeg);
-                s_row = scale[row];
-            }
+            gbeg = m_beg[g0 + team];
+            gend = m_end[g0 + team];
+            row = m_row[g0 + team];
+            flags = m_flags[g0 + team];
+            s_row = m_scale[g0 + team];
         }
-        bool live = active && gend > gbeg;
-        const int wbeg = __shfl(gbeg, 0, kWave);
-        const int wend = __shfl(gend, (np - 1) * TS, kWave);
+        bool live = active && (flags & 16) != 0;
+        const int wbeg = m_beg[g0];
+        const int wend = m_end[g0 + np - 1];
 
         V acc[CPL];
 #pragma unroll
@@ -247,49 +283,57 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
 #pragma unroll
             for (int j = 0; j < VW; ++j) acc[k].v[j] = 0.f;
 
-        // the groups of the round are one contiguous slot range: stage it with coalesced loads
-        for (int cb = wbeg; cb < wend; cb += kStageCap) {
-            const int cn = min(kStageCap, wend - cb);
-            {
-                int c[kPasses];
+        // the groups of the wave cover one contiguous slot range; a window of it is staged in LDS with
+        // coalesced loads and lasts for as many rounds as it covers
+        for (int cb = wbeg; cb < wend;) {
+            if (cb < win_beg || cb >= win_end) {                 // wave-uniform
+                __builtin_amdgcn_wave_barrier();                 // all teams are done with the old window
+                const int cn_new = min(kStageCap, slots_end - cb);
 #pragma unroll
-                for (int r = 0; r < kPasses; ++r) {
-                    const int i = lane + r * kWave;
-                    c[r] = i < cn ? col[cb + i] : 0;
-                }
-                if constexpr (!kPrescaled) {
-                    float sc[kPasses];
+                for (int half = 0; half < 2; ++half) {
+                    int c[kPasses / 2];
 #pragma unroll
-                    for (int r = 0; r < kPasses; ++r) {
-                        const int i = lane + r * kWave;
-                        sc[r] = i < cn ? scale[c[r]] : 0.f;
+                    for (int r = 0; r < kPasses / 2; ++r) {
+                        const int i = lane + (half * (kPasses / 2) + r) * kWave;
+                        c[r] = i < cn_new ? col[cb + i] : 0;
+                    }
+                    if constexpr (!kPrescaled) {
+                        float sc[kPasses / 2];
+#pragma unroll
+                        for (int r = 0; r < kPasses / 2; ++r) {
+                            const int i = lane + (half * (kPasses / 2) + r) * kWave;
+                            sc[r] = i < cn_new ? scale[c[r]] : 0.f;
+                        }
+#pragma unroll
+                        for (int r = 0; r < kPasses / 2; ++r) {
+                            const int i = lane + (half * (kPasses / 2) + r) * kWave;
+                            if (i < cn_new) my_scale[stage_index(i)] = sc[r];
+                        }
                     }
 #pragma unroll
-                    for (int r = 0; r < kPasses; ++r) {
-                        const int i = lane + r * kWave;
-                        if (i < cn) my_scale[stage_index(i)] = sc[r];
+                    for (int r = 0; r < kPasses / 2; ++r) {
+                        const int i = lane + (half * (kPasses / 2) + r) * kWave;
+                        if (i < cn_new) my_col[stage_index(i)] = c[r];
                     }
                 }
-#pragma unroll
-                for (int r = 0; r < kPasses; ++r) {
-                    const int i = lane + r * kWave;
-                    if (i < cn) my_col[stage_index(i)] = c[r];
-                }
+                win_beg = cb;
+                win_end = cb + cn_new;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const int pass_end = min(wend, win_end);
 
             // every team walks the part of its group that lies in this pass, U rows in flight
             const int lo = max(gbeg, cb);
-            const int hi = live ? min(gend, cb + cn) : lo;
+            const int hi = live ? min(gend, pass_end) : lo;
             for (int i = lo; i < hi; i += U) {
                 V v[U][CPL];
                 float w[U];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const bool ok = i + u < hi;
-                    const int word = stage_index(ok ? i + u - cb : 0);
+                    const int word = stage_index(ok ? i + u - win_beg : 0);
                     const int c = my_col[word];
                     if constexpr (!kPrescaled) w[u] = ok ? s_row * my_scale[word] : 0.f;
                     const float* src = in + static_cast<size_t>(c) * ld_in;
@@ -314,7 +358,7 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
                             else acc[k].v[j] = fmaf(w[u], v[u][k].v[j], acc[k].v[j]);
                         }
             }
-            __builtin_amdgcn_wave_barrier();   // all teams are done with the stage before it is refilled
+            cb = pass_end;
         }
         if constexpr (kPrescaled) {
 #pragma unroll
@@ -324,10 +368,10 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
         }
 
         // ---- combine with the carried run, reduce across teams, flush or carry on
-        bool prev = live && groups.has_prev(p, row, gbeg);
-        const bool next = live && groups.has_next(p, row, gend, num_parts);
-        const bool joins_left = live && groups.joins_left(p, prev);
-        const bool joins_right = live && groups.joins_right(p, next);
+        bool prev = live && (flags & 1) != 0;
+        const bool next = live && (flags & 2) != 0;
+        const bool joins_left = live && (flags & 4) != 0;
+        const bool joins_right = live && (flags & 8) != 0;
         bool orphan = false;           // a carried sum met an empty group (malformed input): never store plainly
         if (carry_valid && team == 0) {
             // the first group of this round continues the carried run
@@ -465,6 +509,7 @@ static hipError_t launch_one(float* out, const float* in, const int* col, const 
     }
     if (rounds < 1) rounds = 1;
     if (rounds > kMaxRounds) rounds = kMaxRounds;
+    if (rounds > kWave / TPW) rounds = kWave / TPW;      // a wave describes its groups one per lane
     const long long groups_per_block = static_cast<long long>(TPW) * kAggWaves * rounds;
     const long long grid = (num_parts + groups_per_block - 1) / groups_per_block;
     hipLaunchKernelGGL((aggregate_kernel<VW, OVW, TS, CPL, U, kPrescaled, Groups>),
