@@ -24,7 +24,7 @@ EXPORTS = [
     "eppgcn_clear_time", "eppgcn_get_time_ms", "eppgcn_set_team_size", "eppgcn_set_rounds", "eppgcn_set_plan_shift", "eppgcn_set_plan_keep_rows",
     "eppgcn_feature_workspace_pitch", "eppgcn_update_forward", "eppgcn_update_backward_input",
     "eppgcn_update_workspace_bytes", "eppgcn_update_backward_weight", "eppgcn_update_supported",
-    "eppgcn_mark_compact_workspace_bytes", "eppgcn_mark_compact",
+    "eppgcn_mark_compact_workspace_bytes", "eppgcn_mark_compact", "eppgcn_set_plan_length_classes",
 ]
 
 _lib = None
@@ -83,6 +83,8 @@ def load():
     lib.eppgcn_set_rounds.restype = None
     lib.eppgcn_set_plan_shift.argtypes = [i]
     lib.eppgcn_set_plan_shift.restype = None
+    lib.eppgcn_set_plan_length_classes.argtypes = [i]
+    lib.eppgcn_set_plan_length_classes.restype = None
     lib.eppgcn_set_plan_keep_rows.argtypes = [i]
     lib.eppgcn_set_plan_keep_rows.restype = None
     lib.eppgcn_mark_compact_workspace_bytes.argtypes = [i64]
@@ -478,6 +480,10 @@ def set_team_size(lanes: int):
 
 def set_rounds(rounds: int):
     load().eppgcn_set_rounds(int(rounds))
+
+
+def set_plan_length_classes(on: bool):
+    load().eppgcn_set_plan_length_classes(int(bool(on)))
 
 
 def set_plan_shift(shift: int):

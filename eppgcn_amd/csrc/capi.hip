@@ -19,6 +19,7 @@ size_t plan_workspace_bytes(long long);
 int schedule_shift(int);
 void set_schedule_shift(int);
 void set_plan_keep_rows(int);
+void set_plan_length_classes(int);
 int launch_build_plan(const int*, const int*, const int*, const int*, int, long long, int, int, void*, size_t, void*,
                       size_t, hipStream_t);
 void set_agg_force_team(int);
@@ -78,7 +79,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 4; }
+int eppgcn_abi_version(void) { return 5; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -390,6 +391,7 @@ void eppgcn_set_team_size(int lanes) { set_agg_force_team(lanes); }
 void eppgcn_set_rounds(int rounds) { set_agg_force_rounds(rounds); }
 void eppgcn_set_plan_shift(int shift) { set_schedule_shift(shift); }
 void eppgcn_set_plan_keep_rows(int groups) { set_plan_keep_rows(groups); }
+void eppgcn_set_plan_length_classes(int on) { set_plan_length_classes(on); }
 
 // ---- dense update
 int eppgcn_feature_workspace_pitch(int dim) { return dim > 0 ? workspace_pitch(dim) : 0; }

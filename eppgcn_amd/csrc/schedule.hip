@@ -37,8 +37,8 @@ static size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 // 2..16 groups cost more than the L2 hits of their later groups save).
 __global__ __launch_bounds__(256) void plan_keys_kernel(const int* __restrict__ part_ptr, const int* __restrict__ col,
                                                        const int* __restrict__ part2node, const int* __restrict__ ids,
-                                                       int num_parts, int shift, int keep, unsigned* __restrict__ keys,
-                                                       int* __restrict__ iota)
+                                                       int num_parts, int shift, int keep, int classes,
+                                                       unsigned* __restrict__ keys, int* __restrict__ iota)
 {
     const int p = blockIdx.x * blockDim.x + threadIdx.x;
     if (p >= num_parts) return;
@@ -60,7 +60,16 @@ __global__ __launch_bounds__(256) void plan_keys_kernel(const int* __restrict__ 
     const bool end_found = !(last + 1 < num_parts && same_row(last + 1));
     const bool short_row = start_found && end_found && last - start + 1 <= keep;
     const int key_col = short_row ? col[part_ptr[start]] : col[beg];
-    keys[p] = static_cast<unsigned>(key_col) >> shift;
+    unsigned key = static_cast<unsigned>(key_col) >> shift;
+    if (classes) {
+        // second key: length class of a row that is a single group (a class = one gather step of 8
+        // slots), so that the groups a wave works on in one round take the same number of steps;
+        // rows of several groups consist of full groups but for the last one: class 3
+        const int len = end - beg;
+        const int cls = (short_row && start == last) ? min(3, (len - 1) >> 3) : 3;
+        key = (key << 2) | static_cast<unsigned>(cls);
+    }
+    keys[p] = key;
 }
 
 __global__ __launch_bounds__(256) void plan_sizes_kernel(const int* __restrict__ part_ptr, const int* __restrict__ order,
@@ -184,6 +193,8 @@ int workspace_pitch(int dim);   // aggregate.hip
 
 static int g_force_shift = 0;
 static int g_keep_rows = 8;
+static int g_length_classes = 1;
+void set_plan_length_classes(int on) { g_length_classes = on ? 1 : 0; }
 void set_schedule_shift(int shift) { g_force_shift = shift; }
 void set_plan_keep_rows(int keep) { g_keep_rows = keep < 0 ? 0 : keep; }
 
@@ -232,7 +243,8 @@ int launch_build_plan(const int* part_ptr, const int* col, const int* part2node,
     uint64_t* desc = reinterpret_cast<uint64_t*>(st + 1);
     void* temp = base + 5 * slab + scan_state_bytes(num_parts);
     int bits = 1;
-    while (bits < 32 && (static_cast<long long>(num_nodes) >> shift) >= (1ll << bits)) ++bits;
+    while (bits < 30 && (static_cast<long long>(num_nodes) >> shift) >= (1ll << bits)) ++bits;
+    if (g_length_classes) bits += 2;
     size_t temp_bytes = 0;
     EPPGCN_HIP(sort_temp_bytes(num_parts, bits, &temp_bytes));
     if (5 * slab + scan_state_bytes(num_parts) + temp_bytes > workspace_bytes) {
@@ -241,7 +253,7 @@ int launch_build_plan(const int* part_ptr, const int* col, const int* part2node,
     }
     const unsigned blocks = static_cast<unsigned>((num_parts + 255) / 256);
     hipLaunchKernelGGL(plan_keys_kernel, dim3(blocks), dim3(256), 0, stream, part_ptr, col, part2node, ids, num_parts,
-                       shift, g_keep_rows, keys_in, iota);
+                       shift, g_keep_rows, g_length_classes, keys_in, iota);
     EPPGCN_HIP(hipGetLastError());
     EPPGCN_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, iota, order,
                                          static_cast<size_t>(num_parts), 0u, static_cast<unsigned>(bits), stream));

@@ -275,6 +275,9 @@ void eppgcn_set_rounds(int rounds);
 void eppgcn_set_plan_shift(int shift);
 /* Rows with at most this many groups stay together in a plan (default 8; 0 = block every group). */
 void eppgcn_set_plan_keep_rows(int groups);
+/* Within a column block, order single-group rows by length class (1-8, 9-16, 17-24, 25+ slots) so
+ * that the groups of one round take the same number of gather steps (default on). */
+void eppgcn_set_plan_length_classes(int on);
 
 #ifdef __cplusplus
 }

@@ -272,12 +272,14 @@ def test_plan_is_a_stable_column_block_reordering(api, name, ps):
         groups_per_row = np.bincount(p2n, minlength=n)
         row_first_group = np.concatenate([[0], np.cumsum(groups_per_row)[:-1]])
         key_col = np.where(groups_per_row[p2n] <= 8, col[pp[row_first_group[p2n]]], col[pp[:-1]])[order]
+        # second key: length class (steps of 8 slots) of rows that are a single group, 3 for the rest
+        cls = np.where(groups_per_row[p2n] == 1, np.minimum(3, (np.diff(pp) - 1) >> 3), 3)[order]
         ok = False
         for shift in ([forced] if forced else range(8, 18)):
-            blocks = key_col >> shift
-            if np.all(np.diff(blocks) >= 0) and np.all((np.diff(blocks) > 0) | (np.diff(order) > 0)):
+            keys = ((key_col >> shift) << 2) | cls
+            if np.all(np.diff(keys) >= 0) and np.all((np.diff(keys) > 0) | (np.diff(order) > 0)):
                 ok = True
-        assert ok, "not ordered by a power-of-two column block with stable ties"
+        assert ok, "not ordered by (power-of-two column block, length class) with stable ties"
         prev = np.concatenate([[False], p2n[1:] == p2n[:-1]])[order]
         nxt = np.concatenate([p2n[1:] == p2n[:-1], [False]])[order]
         jl = prev & np.concatenate([[False], order[1:] == order[:-1] + 1])
