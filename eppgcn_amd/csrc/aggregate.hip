@@ -181,10 +181,12 @@ __global__ __launch_bounds__(256) void scale_rows_flat4_kernel(float4* dst, cons
 // VW: floats per load of the input (row pitch ld_in, `chunks` vectors per row are read);
 // OVW: floats per store of the output (row pitch ld_out, columns < width_out are written).
 //
-// A wave runs `rounds` rounds; round r covers the TPW consecutive groups starting at
-// (wave * rounds + r) * TPW.  When the last run of a round is continued by the first group of
-// the next round of the same wave its partial sum is carried in registers instead of being
-// flushed, so a long row costs one flush per wave, not one per group.
+// A wave owns TPW * rounds (at most 64) consecutive groups.  It first loads their descriptions,
+// one group per lane, into LDS, then runs `rounds` rounds; round r gives the TPW groups
+// r * TPW ... to the TPW teams.  The slots of the wave's groups are one contiguous range, of which a
+// window of kStageCap slots is staged in LDS and refilled when a round runs past its end.  When the
+// last run of a round is continued by the first group of the next round its partial sum is carried
+// in registers instead of being flushed, so a long row costs one flush per wave, not one per group.
 //
 // A "run" is a maximal stretch of adjacent teams whose groups continue one another (same row,
 // adjacent in the original group order).  Only such groups are summed across teams, so that
