@@ -60,7 +60,13 @@ template <> struct Vec<2> {
         float2 t = *reinterpret_cast<const float2*>(p);
         Vec r; r.v[0] = t.x; r.v[1] = t.y; return r;
     }
-    __device__ void store(float* p) const { *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]); }
+    // output rows are written once and not read again by the kernel: non-temporal stores
+    __device__ void store(float* p) const
+    {
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        const f2 t = {v[0], v[1]};
+        __builtin_nontemporal_store(t, reinterpret_cast<f2*>(p));
+    }
 };
 template <> struct Vec<4> {
     float v[4];
@@ -69,7 +75,12 @@ template <> struct Vec<4> {
         float4 t = *reinterpret_cast<const float4*>(p);
         Vec r; r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w; return r;
     }
-    __device__ void store(float* p) const { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
+    __device__ void store(float* p) const
+    {
+        typedef float f4 __attribute__((ext_vector_type(4)));
+        const f4 t = {v[0], v[1], v[2], v[3]};
+        __builtin_nontemporal_store(t, reinterpret_cast<f4*>(p));
+    }
 };
 
 // ---------------------------------------------------------------- group sources
@@ -297,7 +308,7 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
 #pragma unroll
                     for (int r = 0; r < kPasses / 2; ++r) {
                         const int i = lane + (half * (kPasses / 2) + r) * kWave;
-                        c[r] = i < cn_new ? col[cb + i] : 0;
+                        c[r] = i < cn_new ? __builtin_nontemporal_load(col + cb + i) : 0;   // streamed once: keep it out of the rows' way
                     }
                     if constexpr (!kPrescaled) {
                         float sc[kPasses / 2];
