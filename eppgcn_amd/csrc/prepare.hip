@@ -515,7 +515,10 @@ __global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* __restrict__ 
     const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
     const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     uint4* v = reinterpret_cast<uint4*>(p + head);
-    for (size_t i = tid; i < vecs; i += stride) v[i] = make_uint4(0u, 0u, 0u, 0u);
+    // non-temporal: the zeros are not read back before the kernel that follows has filled the caches
+    typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+    const uintx4 zero = {0u, 0u, 0u, 0u};
+    for (size_t i = tid; i < vecs; i += stride) __builtin_nontemporal_store(zero, reinterpret_cast<uintx4*>(v) + i);
     const size_t tail = head + 4 * vecs;
     if (tid < head) p[tid] = 0u;
     if (tid < words - tail) p[tail + tid] = 0u;
