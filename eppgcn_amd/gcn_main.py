@@ -1,0 +1,138 @@
+"""Command line of the reference's training driver (EPPGCN/gcn_main.py:20-51,272-292) over this
+package: the same flags, the same report lines (``for_time``, ``loss_time``, ``back_time``,
+``build_time``, ``Time``), so a sweep script that formats a ``gcn_main.py`` command per dataset x
+mask ratio x depth (EPPGCN/bench_EPPGCN.py:41-61) only has to point at ``python -m
+eppgcn_amd.gcn_main``.
+
+Differences, all deliberate:
+  * ``--backsize_mode net`` needs the reference's unpublished predictor weights
+    (EPPGCN/net_pred.py:63) and is refused with a message; the default here is ``map``.
+  * ``--dataset`` also accepts a synthetic graph name (``cfg1_uniform``, ``rmat:<scale>:<factor>``
+    ...) when no graph file is given; the train mask is then drawn instead of read.
+  * the device is the current one (the reference hard-codes device 1, gcn_main.py:69).
+  * ``--degree_norm inv_sqrt`` (an addition) fills the scale vector with deg^-1/2 instead of the
+    reference loader's sqrt(deg) (EPPGCN/dataset.py:117-119).
+  * ``--model gin`` is accepted by the reference's parser but never read by it; here too.
+  * ``--single_spmm`` / ``--verify_spmm`` are parsed and never read by the reference; here
+    ``--single_spmm True`` times the forward aggregation alone and ``--verify_spmm True``
+    compares one forward aggregation with torch's dense result on the device."""
+from __future__ import annotations
+
+import argparse
+import os.path as osp
+import sys
+import time
+
+import torch
+
+
+def build_parser() -> argparse.ArgumentParser:
+    tf = dict(type=str, choices=["True", "False"])
+    ap = argparse.ArgumentParser(description="GCN training over the GNNAdvisor ops (HIP, gfx950)")
+    ap.add_argument("--dataDir", type=str, default="../osdi-ae-graphs", help="directory of the graph and mask files")
+    ap.add_argument("--dataset", type=str, default="amazon0601", help="graph file stem or synthetic graph name")
+    ap.add_argument("--dim", type=int, default=96, help="input feature width")
+    ap.add_argument("--hidden", type=int, default=16, help="hidden width")
+    ap.add_argument("--classes", type=int, default=22, help="output width")
+    ap.add_argument("--layers", type=int, default=2, help="number of layers")
+    ap.add_argument("--train_ratio", type=float, default=0.1, help="train mask ratio")
+    ap.add_argument("--model", type=str, default="gcn", choices=["gcn", "gin"])
+    ap.add_argument("--num_epoches", type=int, default=100, help="timed epochs after 10 warm-up epochs")
+    ap.add_argument("--partSize", type=int, default=32, help="forward neighbour-group size (manual mode)")
+    ap.add_argument("--dimWorker", type=int, default=32, help="launch hint, kept for compatibility")
+    ap.add_argument("--warpPerBlock", type=int, default=8, help="launch hint, kept for compatibility")
+    ap.add_argument("--sharedMem", type=int, default=100, help="launch hint, kept for compatibility")
+    ap.add_argument("--manual_mode", default="False", help="True: use --partSize, False: decider", **tf)
+    ap.add_argument("--verbose_mode", default="False", **tf)
+    ap.add_argument("--loadFromTxt", default="True", help="True: <dataset>_snap edge list, False: <dataset>.npz", **tf)
+    ap.add_argument("--single_spmm", default="False", help="time the forward aggregation alone", **tf)
+    ap.add_argument("--verify_spmm", default="False", help="check one forward aggregation against torch", **tf)
+    ap.add_argument("--backsize", type=int, default=0, help="backward group size of all layers (constant mode)")
+    ap.add_argument("--backsize_mode", type=str, default="map", choices=["map", "net", "constant"])
+    ap.add_argument("--degree_norm", type=str, default="sqrt", choices=["sqrt", "inv_sqrt"],
+                    help="scale vector: sqrt(deg) as the reference's loader fills it, or deg^-1/2 (symmetric GCN norm)")
+    ap.add_argument("--kernel_timers", default="True", **tf,
+                    help="True: per-op device timers for the print_time report, as the reference always has; "
+                         "False: none (the epochs are then issued without a host wait per op)")
+    return ap
+
+
+def load_dataset(args, device):
+    """The reference's file naming (gcn_main.py:74-79); a name with no file behind it is tried as
+    a synthetic graph."""
+    from . import dataset as ds_mod, graphs, train
+    txt = args.loadFromTxt == "True"
+    path = osp.join(args.dataDir, args.dataset + ("_snap" if txt else ".npz"))
+    if osp.exists(path):
+        return ds_mod.custom_dataset(path, args.dataDir, args.train_ratio, args.dim, args.classes, args.layers,
+                                     load_from_txt=txt, verbose=args.verbose_mode == "True", device=device,
+                                     scale_mode=args.degree_norm)
+    try:
+        graph = graphs.make_graph(args.dataset, device, scale_mode=args.degree_norm)
+    except Exception:
+        raise FileNotFoundError(f"{path} does not exist and '{args.dataset}' names no synthetic graph")
+    return train.GraphDataset(graph, args.dim, args.classes, args.layers, train_ratio=args.train_ratio)
+
+
+def _single_spmm(tr, epochs, verify):
+    """Forward aggregation of the hidden width alone, `epochs` times; optionally checked against
+    a sparse product formed by torch on the device."""
+    ds, info = tr.dataset, tr.inputInfo
+    width = tr.model.convs[0].weights.shape[1]
+    x = torch.randn(ds.num_nodes, width, device=ds.x.device)
+    eye = torch.eye(width, device=x.device)
+    call = lambda: tr.GNNA.forward(x, eye, info.row_pointers, info.column_index, info.degrees, info.partPtr,
+                                   info.part2Node, info.partSize, info.dimWorker, info.warpPerBlock)[0]
+    out = call()
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    for _ in range(epochs):
+        call()
+    torch.cuda.synchronize()
+    print("single_spmm (ms): {:.4f}".format((time.perf_counter() - t) * 1e3 / max(1, epochs)))
+    if verify:
+        rows = torch.repeat_interleave(torch.arange(ds.num_nodes, device=x.device),
+                                       (info.row_pointers[1:] - info.row_pointers[:-1]).long())
+        cols = info.column_index.long()
+        ref = torch.zeros_like(out, dtype=torch.float64)
+        ref.index_add_(0, rows, (info.degrees[rows] * info.degrees[cols]).double().unsqueeze(1) * x[cols].double())
+        bound = 1e-5 * ref.abs().max().item() + 1e-30
+        err = (out.double() - ref).abs().max().item()
+        print("verify_spmm: max abs error {:.3e} (bound {:.3e}) -> {}".format(err, bound, "PASS" if err <= bound else "FAIL"))
+        return err <= bound
+    return True
+
+
+def main(argv=None) -> int:
+    args = build_parser().parse_args(argv)
+    print("||" + args.dataset + "   " + str(args.train_ratio) + "   " + str(args.layers))
+    if args.backsize_mode == "net":
+        print("backsize_mode 'net' needs predictor weights the reference does not publish; use 'map' or 'constant'",
+              file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("a GPU is required", file=sys.stderr)
+        return 2
+    from . import train
+    device = torch.device("cuda", torch.cuda.current_device())
+    ds = load_dataset(args, device)
+    verbose = args.verbose_mode == "True"
+    tr = train.Trainer(None, hidden=args.hidden, backsize_mode=args.backsize_mode, backsize=args.backsize,
+                       dataset=ds, part_size=args.partSize, dim_worker=args.dimWorker,
+                       warp_per_block=args.warpPerBlock, shared_mem=args.sharedMem,
+                       manual_mode=args.manual_mode == "True", verbose=verbose, weight_seed=None)
+    if verbose:
+        print(tr.model)
+    if args.single_spmm == "True" or args.verify_spmm == "True":
+        return 0 if _single_spmm(tr, args.num_epoches, args.verify_spmm == "True") else 1
+    res = tr.run(args.num_epoches, warmup=10, kernel_timing=args.kernel_timers == "True")
+    tr.GNNA.print_time()
+    for key in ("for_time", "loss_time", "back_time", "build_time"):
+        print("{}: {:.6f}".format(key, res[key]))
+    print("Time: {:.6f}".format(res["Time"]))
+    print()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

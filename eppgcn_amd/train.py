@@ -77,9 +77,11 @@ class Trainer:
 
     def __init__(self, graph: graphs.Graph, dim=96, hidden=16, num_classes=22, num_layers=2, train_ratio=0.1,
                  train_mask=None, backsize_mode="constant", backsize=32, labels="ones", weight_seed=3, lr=0.01,
-                 fuse_relu=True, dataset=None):
+                 fuse_relu=True, dataset=None, part_size=32, dim_worker=32, warp_per_block=8, shared_mem=100,
+                 manual_mode=False, verbose=False):
         """``dataset``: a loaded ``eppgcn_amd.dataset.custom_dataset`` (or any object with the same
-        attributes) to train on instead of synthetic features over ``graph``."""
+        attributes) to train on instead of synthetic features over ``graph``.  ``part_size`` ...
+        ``manual_mode`` are the driver's forward launch flags (EPPGCN/gcn_main.py:34-40)."""
         self.GNNA = gnnadvisor()
         self.backsize_mode, self.backsize = backsize_mode, backsize
         if dataset is not None:
@@ -89,9 +91,12 @@ class Trainer:
             ds = GraphDataset(graph, dim, num_classes, num_layers, train_mask, train_ratio, labels)
         self.dataset = ds
         self.num_layers = num_layers
-        info = inputProperty(ds.row_pointers, ds.column_index, ds.degrees, 32, 32, 8, 100, hiddenDim=hidden,
-                             dataset_obj=ds, manual_mode=False)
+        info = inputProperty(ds.row_pointers, ds.column_index, ds.degrees, part_size, dim_worker, warp_per_block,
+                             shared_mem, hiddenDim=hidden, dataset_obj=ds, manual_mode=manual_mode, verbose=verbose)
         info.decider()
+        if verbose:
+            info.set_input().print_param()
+            info.set_hidden().print_param()
         part_ptr, part2node = self.GNNA.build_part(info.partSize, ds.row_pointers)
         info.partPtr, info.part2Node = part_ptr.int(), part2node.int()
         self.inputInfo = info

@@ -288,6 +288,35 @@ def test_training_from_a_dataset_file(GNNA, tmp_path):
     assert np.linalg.norm(tr.model.convs[1].weights.grad.cpu().numpy() - want_g1) / np.linalg.norm(want_g1) < 1e-4
 
 
+def test_driver_command_line_end_to_end(GNNA, tmp_path, capsys):
+    """`python -m eppgcn_amd.gcn_main` with the reference's flags on reference-format files: the
+    report carries the reference's lines (EPPGCN/gcn_main.py:286-291), --verify_spmm passes, a
+    synthetic graph name works without files and a missing file is an error, not a crash."""
+    from eppgcn_amd import dataset as dsmod, gcn_main
+    indptr, col = random_symmetric_csr(400, 1500, 17)
+    n = indptr.size - 1
+    rows = np.repeat(np.arange(n), np.diff(indptr))
+    np.savetxt(str(tmp_path / "toy_snap"), np.stack([rows, col], 1), fmt="%d")
+    dsmod.write_train_mask(str(tmp_path), 0.3, np.random.default_rng(2).random(n) < 0.3)
+    common = ["--dataset", "toy", "--dataDir", str(tmp_path), "--dim", "24", "--hidden", "16", "--classes", "5",
+              "--train_ratio", "0.3", "--num_epoches", "3", "--degree_norm", "inv_sqrt"]
+    for extra in (["--layers", "3", "--backsize_mode", "map"],
+                  ["--layers", "2", "--backsize_mode", "constant", "--backsize", "8", "--kernel_timers", "False",
+                   "--manual_mode", "True", "--partSize", "4", "--verbose_mode", "True"]):
+        assert gcn_main.main(common + extra) == 0
+        out = capsys.readouterr().out
+        for key in ("for_time:", "loss_time:", "back_time:", "build_time:", "Time:"):
+            assert sum(line.startswith(key) for line in out.splitlines()) == 1, (key, out)
+        assert out.startswith("||toy   0.3   ")
+    assert gcn_main.main(common + ["--verify_spmm", "True"]) == 0
+    assert "PASS" in capsys.readouterr().out
+    assert gcn_main.main(["--dataset", "cfg1_uniform", "--num_epoches", "2", "--degree_norm", "inv_sqrt",
+                          "--backsize_mode", "constant", "--backsize", "16"]) == 0
+    capsys.readouterr()
+    with pytest.raises(FileNotFoundError):
+        gcn_main.main(["--dataset", "no_such_graph", "--dataDir", str(tmp_path)])
+
+
 @pytest.mark.parametrize("num_layers", [3, 4])
 def test_deeper_models_follow_the_mask_chain(GNNA, num_layers):
     """3 and 4 layers (the reference sweeps 3-6): the marking of layer i feeds layer i+1's source

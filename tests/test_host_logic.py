@@ -101,3 +101,23 @@ def test_algorithmic_bytes_nominal_values():
     assert workload.bytes_pruned_backward(10, 50, 7, 22) == 50 * 96 + 10 * 88 + 56
     assert workload.bytes_compact(100, 10) == 400 + 120
     assert workload.bytes_compulsory(10, 100, 16) == 400 + 80 + 1280
+
+
+def test_driver_command_line_takes_the_reference_flags(capsys):
+    """Every flag EPPGCN/bench_EPPGCN.py:54-58 puts on the command line parses, with the
+    reference's defaults (EPPGCN/gcn_main.py:21-50) except the 'net' group-size predictor, which
+    is refused before anything touches a device."""
+    from eppgcn_amd import gcn_main
+    line = ("--dataset cora --dim 1433 --hidden 16 --classes 7 --layers 3 --partSize 0 --model gcn --warpPerBlock 8 "
+            "--manual_mode False --verbose_mode False --loadFromTxt True --dataDir /data/cora --train_ratio 0.3 "
+            "--backsize_mode constant --backsize 32").split()
+    a = gcn_main.build_parser().parse_args(line)
+    assert (a.dataset, a.dim, a.classes, a.layers, a.train_ratio, a.backsize_mode, a.backsize) == \
+        ("cora", 1433, 7, 3, 0.3, "constant", 32)
+    d = gcn_main.build_parser().parse_args([])
+    assert (d.dim, d.hidden, d.classes, d.layers, d.train_ratio, d.num_epoches, d.partSize, d.dimWorker,
+            d.warpPerBlock, d.sharedMem, d.manual_mode, d.loadFromTxt, d.backsize) == \
+        (96, 16, 22, 2, 0.1, 100, 32, 32, 8, 100, "False", "True", 0)
+    assert gcn_main.main(["--backsize_mode", "net"]) == 2
+    out = capsys.readouterr()
+    assert out.out.startswith("||amazon0601   0.1   2") and "net" in out.err
