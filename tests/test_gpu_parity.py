@@ -726,3 +726,58 @@ def test_aggregation_with_misaligned_feature_buffers(api, dim, shift_in, shift_o
         out.fill_(3.0)
         api.ours_backward(xin, ids, bpp, edge_list, dev(s), p, 8, out=out, workspace=workspace)
         assert_close(out.cpu().numpy(), want_b, bound, f"pruned backward, workspace={workspace}")
+
+
+def test_element_offsets_beyond_int32(api):
+    """[N, 256] matrices of more than 2^31 elements (8.6 GB each): every row offset has to be
+    formed in 64 bits.  Ring graph with self-loops, unit scale, small integer features, so the
+    result is exactly x[i-1] + x[i] + x[i+1] whatever the order of summation; the pruned backward
+    over a mask that keeps the last rows must equal the unpruned one on the masked gradient, and
+    the dense update must reach the last rows too."""
+    n, dim = (1 << 23) + 5, 256
+    assert n * dim > (1 << 31)
+    idx = torch.arange(n, device="cuda")
+    col = torch.stack([(idx - 1) % n, idx, (idx + 1) % n], 1).sort(dim=1).values.to(torch.int32).reshape(-1)
+    indptr = (torch.arange(n + 1, device="cuda") * 3).to(torch.int32)
+    ones = torch.ones(n, device="cuda")
+    pp, p2n = api.build_part(2, indptr)
+    from eppgcn_amd import graphs
+    x = torch.empty(n, dim, device="cuda")
+    step = 1 << 20
+    for r0 in range(0, n, step):                       # in pieces: the generator works in int64
+        r1 = min(n, r0 + step)
+        x[r0:r1] = (graphs.uniform32(11, torch.arange(r0 * dim, r1 * dim, device="cuda")) % 17 - 8).reshape(-1, dim)
+    want = x + torch.roll(x, 1, 0)
+    want += torch.roll(x, -1, 0)
+    got = api.spmm_forward(x, col, ones, pp, p2n, part_size=2)
+    assert torch.equal(got[-4096:], want[-4096:]) and torch.equal(got[:4096], want[:4096])
+    assert torch.equal(got, want)
+    del got
+    # pruned backward: mask = the last 3000 vertices and every 1000th one
+    src = (idx >= n - 3000) | (idx % 1000 == 0)
+    e = col.numel()
+    bem = torch.full((e,), -1, dtype=torch.int32, device="cuda")
+    degs = torch.zeros(n, dtype=torch.int32, device="cuda")
+    api.mask_forward(p2n, pp, col, src, None, bem, degs, True)
+    oid, oedge, v = api.compact_back_edge(bem, col)
+    bpp, p, v2 = api.split_back_part(degs, e, 2)
+    assert v == v2 == int(src[col.long()].sum())
+    x *= src[:, None]
+    want = x + torch.roll(x, 1, 0)
+    want += torch.roll(x, -1, 0)
+    got = api.ours_backward(x, oid, bpp, oedge, ones, p, part_size=2)
+    assert torch.equal(got, want)
+    del got, want
+    # dense update of the last rows: [n, 256] x [256, 16] with integer operands is exact in fp32
+    w = (graphs.uniform32(12, torch.arange(dim * 16, device="cuda")) % 5 - 2).reshape(dim, 16).float()
+    y = api.update_forward(x, w, ones)
+    tail = slice(n - 3000, n)
+    assert torch.equal(y[tail, :16], x[tail] @ w)
+    # input gradient and weight gradient with the non-zero rows at the end of the matrices
+    g = torch.zeros(n, 16, device="cuda")
+    g[tail] = (graphs.uniform32(13, torch.arange(3000 * 16, device="cuda")) % 7 - 3).reshape(3000, 16).float()
+    dx = api.update_backward_input(g, w)
+    assert torch.equal(dx[tail], g[tail] @ w.t()) and not dx[: n - 3000].any()
+    del dx
+    dw = api.update_backward_weight(x, g)
+    assert torch.equal(dw, x[tail].t() @ g[tail])
