@@ -23,6 +23,7 @@
 
 #include <c10/hip/HIPStream.h>
 
+#include <cstdint>
 #include <list>
 #include <vector>
 
@@ -51,6 +52,12 @@ void check(int rc, const char* what)
 #define CHECK_MASK(x) \
     CHECK_INPUT(x);   \
     TORCH_CHECK((x).scalar_type() == torch::kBool || (x).scalar_type() == torch::kUInt8, #x " must be bool")
+
+// Slots and vertices are int32 on the device, and the kernels step through slot ranges in strides of
+// up to 1024 past a group's end before clamping: leave that much headroom below 2^31.
+#define CHECK_COUNTS(edges, vertices)                                                                      \
+    TORCH_CHECK((edges).numel() <= INT32_MAX - 1024, #edges " holds more slots than int32 indexing allows"); \
+    TORCH_CHECK((vertices) <= INT32_MAX - 1024, "more vertices than int32 indexing allows")
 
 void* stream_of(const Tensor& t)
 {
@@ -228,6 +235,7 @@ std::vector<Tensor> forward(Tensor input, Tensor weight, Tensor row_pointers, Te
     TORCH_CHECK(input.dim() == 2 && weight.dim() == 2 && input.size(1) == weight.size(0), "shape mismatch");
     TORCH_CHECK(degrees.numel() == input.size(0), "degrees must have one entry per vertex");
     TORCH_CHECK(part_pointers.numel() >= part2Node.numel() + 1, "part_pointers needs num_parts + 1 entries");
+    CHECK_COUNTS(column_index, input.size(0));
     const int64_t n = input.size(0);
     const int dim = static_cast<int>(weight.size(1));
     auto output = torch::empty({n, dim}, input.options());
@@ -268,6 +276,7 @@ std::vector<Tensor> backward(Tensor d_output, Tensor X, Tensor W, Tensor row_poi
     TORCH_CHECK(X.dim() == 2 && W.dim() == 2 && X.size(0) == d_output.size(0) && X.size(1) == W.size(0) &&
                     W.size(1) == d_output.size(1), "X, W and d_output do not fit together");
     TORCH_CHECK(part_pointers.numel() >= part2Node.numel() + 1, "part_pointers needs num_parts + 1 entries");
+    CHECK_COUNTS(column_index, d_output.size(0));
     auto d_input_prime = torch::empty_like(d_output);
     auto scaled = feature_scratch(d_output);     // d_output belongs to autograd: scale into scratch
     check(eppgcn_spmm_backward(d_input_prime.data_ptr<float>(), f32(d_output), i32(row_pointers),
@@ -292,6 +301,7 @@ void mask_forward(Tensor id, Tensor partPointer, Tensor edgeList, Tensor src_mas
     TORCH_CHECK(partPointer.numel() >= id.numel() + 1, "partPointer needs num_parts + 1 entries");
     TORCH_CHECK(backEdgeMask.numel() >= edgeList.numel(), "backEdgeMask is shorter than the edge list");
     TORCH_CHECK(src_mask.numel() == node_degs.numel(), "src_mask and node_degs must have one entry per vertex");
+    CHECK_COUNTS(edgeList, node_degs.numel());
     TORCH_CHECK(is_last || ngh_mask.numel() == node_degs.numel(), "ngh_mask must have one entry per vertex");
     check(eppgcn_mask_forward(i32(id), i32(partPointer), i32(edgeList),
                               static_cast<const uint8_t*>(src_mask.data_ptr()),
@@ -313,6 +323,7 @@ std::vector<Tensor> ours_backward(Tensor d_output, Tensor X, Tensor W, Tensor id
                     W.size(1) == d_output.size(1), "X, W and d_output do not fit together");
     TORCH_CHECK(numParts >= 0 && partPointer.numel() >= static_cast<int64_t>(numParts) + 1,
                 "partPointer needs numParts + 1 entries");
+    CHECK_COUNTS(edgeList, d_output.size(0));
     auto d_input_prime = torch::empty_like(d_output);
     auto scaled = feature_scratch(d_output);     // d_output belongs to autograd: scale into scratch
     check(eppgcn_ours_backward(d_input_prime.data_ptr<float>(), f32(d_output), i32(id), i32(partPointer),
@@ -417,6 +428,7 @@ std::vector<Tensor> mark_compact(Tensor id, Tensor partPointer, Tensor edgeList,
     const bool is_last = layer == num_layers;
     TORCH_CHECK(partPointer.numel() >= id.numel() + 1, "partPointer needs num_parts + 1 entries");
     TORCH_CHECK(src_mask.numel() == node_degs.numel(), "src_mask and node_degs must have one entry per vertex");
+    CHECK_COUNTS(edgeList, node_degs.numel());
     TORCH_CHECK(is_last || ngh_mask.numel() == node_degs.numel(), "ngh_mask must have one entry per vertex");
     const int64_t length = edgeList.numel();
     auto out_id = torch::empty({length}, edgeList.options());

@@ -36,6 +36,12 @@
  *     with zeros in the padding (eppgcn_update_forward writes exactly that) and
  *     the scaling pass is skipped.  Results of the modes agree to rounding (a few
  *     ulp per term).
+ *   - Limits: vertices and slots (CSR entries, kept edges) are int32 as in the
+ *     reference and must stay below 2^31 - 1024 (the kernels step through slot
+ *     ranges 1024 at a time before clamping); element offsets into the [N, dim]
+ *     matrices are formed in 64 bits, so N * dim may exceed 2^31.  The slot count
+ *     of an aggregation call lives on the device (part_pointers[num_parts]), so
+ *     that bound is the caller's to keep; the extension module checks it.
  */
 #ifndef EPPGCN_HIP_H_
 #define EPPGCN_HIP_H_
