@@ -50,7 +50,7 @@ def load():
     lib.eppgcn_feature_workspace_floats.restype = sz
     lib.eppgcn_plan_recommended.argtypes = [i64, i]
     lib.eppgcn_plan_recommended.restype = i
-    lib.eppgcn_plan_bytes.argtypes = [i64, i64]
+    lib.eppgcn_plan_bytes.argtypes = [i64, i64, i64]
     lib.eppgcn_plan_bytes.restype = sz
     lib.eppgcn_plan_workspace_bytes.argtypes = [i64]
     lib.eppgcn_plan_workspace_bytes.restype = sz
@@ -225,19 +225,33 @@ def feature_workspace(num_nodes: int, dim: int, device):
 class Plan:
     """A column-blocked execution plan (device buffer + the sizes it was built for)."""
 
-    def __init__(self, buffer, base_ptr, num_parts, num_slots):
+    def __init__(self, buffer, base_ptr, num_parts, num_slots, num_nodes):
         self.buffer, self.base_ptr, self.num_parts, self.num_slots = buffer, base_ptr, num_parts, num_slots
+        self.num_nodes = num_nodes
+
+    def _offsets(self):
+        def al(x):
+            return (x + 255) // 256 * 256
+        p = self.num_parts
+        off = self.base_ptr - self.buffer.data_ptr()
+        o1 = off + al(4 * (p + 1)); o2 = o1 + al(4 * p); o3 = o2 + al(p)
+        o4 = o3 + al(4 * ((self.num_nodes + 31) // 32))
+        return off, o1, o2, o3, o4
 
     def view(self):
         """(ptr, row, flags, col) as torch tensors, for tests."""
-        def al(x):
-            return (x + 255) // 256 * 256
         p, s = self.num_parts, self.num_slots
-        off = self.base_ptr - self.buffer.data_ptr()
+        off, o1, o2, o3, o4 = self._offsets()
         raw = self.buffer.view(torch.uint8)
-        o1 = off + al(4 * (p + 1)); o2 = o1 + al(4 * p); o3 = o2 + al(p)
         return (raw[off: off + 4 * (p + 1)].view(torch.int32), raw[o1: o1 + 4 * p].view(torch.int32),
-                raw[o2: o2 + p], raw[o3: o3 + 4 * s].view(torch.int32))
+                raw[o2: o2 + p], raw[o4: o4 + 4 * s].view(torch.int32))
+
+    def single_rows(self):
+        """bool[num_nodes]: rows recorded as one non-empty group (skipped by the output clear), for tests."""
+        _, _, _, o3, _ = self._offsets()
+        words = self.buffer.view(torch.uint8)[o3: o3 + 4 * ((self.num_nodes + 31) // 32)].view(torch.int32)
+        r = torch.arange(self.num_nodes, device=words.device)
+        return ((words[r >> 5] >> (r & 31)) & 1).bool()
 
 
 def _aligned_buffer(nbytes, device):
@@ -257,7 +271,7 @@ def build_plan(part_ptr, column_index, num_parts: int, num_slots: int, num_nodes
         raise EppgcnError("part_ptr needs num_parts + 1 entries")
     if column_index.numel() < num_slots:
         raise EppgcnError("column_index is shorter than num_slots")
-    nbytes = lib.eppgcn_plan_bytes(int(num_parts), int(num_slots))
+    nbytes = lib.eppgcn_plan_bytes(int(num_parts), int(num_slots), int(num_nodes))
     buf, base = _aligned_buffer(nbytes, part_ptr.device)
     wbytes = lib.eppgcn_plan_workspace_bytes(int(num_parts))
     ws, wbase = _aligned_buffer(wbytes, part_ptr.device)
@@ -265,7 +279,7 @@ def build_plan(part_ptr, column_index, num_parts: int, num_slots: int, num_nodes
                                  int(num_slots), int(num_nodes), int(dim), C.c_void_p(base), nbytes,
                                  C.c_void_p(wbase), wbytes, _stream()))
     torch.cuda.current_stream().synchronize()      # the workspace is released on return
-    return Plan(buf, base, int(num_parts), int(num_slots))
+    return Plan(buf, base, int(num_parts), int(num_slots), int(num_nodes))
 
 
 def plan_recommended(num_nodes: int, dim: int) -> bool:
@@ -273,11 +287,11 @@ def plan_recommended(num_nodes: int, dim: int) -> bool:
     return bool(load().eppgcn_plan_recommended(int(num_nodes), int(dim)))
 
 
-def _plan_ptr(plan, num_parts):
+def _plan_ptr(plan, num_parts, num_nodes):
     if plan is None:
         return None
-    if plan.num_parts != num_parts:
-        raise EppgcnError("the plan was built for a different number of groups")
+    if plan.num_parts != num_parts or plan.num_nodes != num_nodes:
+        raise EppgcnError("the plan was built for a different number of groups or vertices")
     return C.c_void_p(plan.base_ptr)
 
 
@@ -310,7 +324,7 @@ def spmm_forward(feats, column_index, degrees, part_ptr, part2node, part_size=32
     ws = workspace if feats is None else _feature_workspace(workspace, feats)
     _check(fn(_ptr(out), _ptr(feats), _ptr(row_pointers), _ptr(column_index), _ptr(degrees), _ptr(part_ptr),
               _ptr(part2node), n, dim, num_parts, part_size, dim_worker, warp_per_block, _ptr(ws),
-              0 if ws is None else ws.numel(), _plan_ptr(plan, num_parts), _stream()))
+              0 if ws is None else ws.numel(), _plan_ptr(plan, num_parts, n), _stream()))
     return out
 
 
@@ -329,7 +343,7 @@ def ours_backward(d_output, ids, part_pointer, edge_list, degrees, num_parts, pa
     _check(lib.eppgcn_ours_backward(_ptr(out), _ptr(d_output), _ptr(ids), _ptr(part_pointer), _ptr(edge_list),
                                     _ptr(degrees), n, dim, int(num_parts), part_size, layer, blockx, blocky,
                                     _ptr(ws), 0 if ws is None else ws.numel(),
-                                    _plan_ptr(plan, int(num_parts)), _stream()))
+                                    _plan_ptr(plan, int(num_parts), n), _stream()))
     return out
 
 

@@ -631,11 +631,16 @@ static int vector_width(int pitch, int width, const void* p)
 template <class Groups>
 static int aggregate_dispatch(float* out, const float* in, const int* col, const float* scale, Groups g,
                               int num_nodes, int dim, int num_parts, int group_size, float* workspace,
-                              hipStream_t stream, double* sink, double* sink2)
+                              hipStream_t stream, double* sink, double* sink2, const uint32_t* single_rows = nullptr)
 {
     const bool prescaled = workspace != nullptr;
     int ld_in = dim;
-    if (int rc = launch_zero_words(out, static_cast<size_t>(num_nodes) * dim, stream)) return rc;
+    // rows the kernel writes with one plain store (a plan knows them) need no clearing
+    if (single_rows && num_parts > 0) {
+        if (int rc = launch_zero_rows_unless(out, single_rows, num_nodes, dim, stream)) return rc;
+    } else {
+        if (int rc = launch_zero_words(out, static_cast<size_t>(num_nodes) * dim, stream)) return rc;
+    }
     if (num_parts == 0) return kOk;
     if (prescaled) {
         // in == nullptr: the caller (the dense update) already wrote the scaled, padded rows
@@ -687,9 +692,9 @@ int aggregate_forward_groups(float* out, const float* in, const int* col, const 
                              double* sink2)
 {
     if (plan && workspace && num_parts > 0) {
-        const PlanView v = plan_view(const_cast<void*>(plan), num_parts);
+        const PlanView v = plan_view(const_cast<void*>(plan), num_parts, num_nodes);
         return aggregate_dispatch(out, in, v.col, scale, PlanGroups{v.ptr, v.row, v.flags}, num_nodes, dim, num_parts,
-                                  group_size, workspace, stream, sink, sink2);
+                                  group_size, workspace, stream, sink, sink2, v.single);
     }
     return aggregate_dispatch(out, in, col, scale, ForwardGroups{part_ptr, part2node}, num_nodes, dim, num_parts,
                               group_size, workspace, stream, sink, sink2);
@@ -701,9 +706,9 @@ int aggregate_compacted_groups(float* out, const float* in, const int* ids, cons
                                double* sink2)
 {
     if (plan && workspace && num_parts > 0) {
-        const PlanView v = plan_view(const_cast<void*>(plan), num_parts);
+        const PlanView v = plan_view(const_cast<void*>(plan), num_parts, num_nodes);
         return aggregate_dispatch(out, in, v.col, scale, PlanGroups{v.ptr, v.row, v.flags}, num_nodes, dim, num_parts,
-                                  group_size, workspace, stream, sink, sink2);
+                                  group_size, workspace, stream, sink, sink2, v.single);
     }
     return aggregate_dispatch(out, in, edge_list, scale, CompactedGroups{part_ptr, ids}, num_nodes, dim, num_parts,
                               group_size, workspace, stream, sink, sink2);

@@ -79,7 +79,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 5; }
+int eppgcn_abi_version(void) { return 6; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -170,7 +170,10 @@ int eppgcn_plan_recommended(int64_t num_nodes, int dim)
     if (num_nodes <= 0 || dim <= 0) return 0;
     return static_cast<double>(feature_workspace_floats(num_nodes, dim)) * 4.0 >= 192.0 * (1 << 20) ? 1 : 0;
 }
-size_t eppgcn_plan_bytes(int64_t num_parts, int64_t num_slots) { return plan_bytes(num_parts, num_slots); }
+size_t eppgcn_plan_bytes(int64_t num_parts, int64_t num_slots, int64_t num_nodes)
+{
+    return plan_bytes(num_parts, num_slots, num_nodes);
+}
 size_t eppgcn_plan_workspace_bytes(int64_t num_parts) { return plan_workspace_bytes(num_parts); }
 
 int eppgcn_build_plan(const int32_t* part_pointers, const int32_t* column_index, const int32_t* part2node,

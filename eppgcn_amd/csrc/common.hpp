@@ -44,32 +44,46 @@ int hip_fail(hipError_t e, const char* what);
 // hipMemsetAsync everywhere so that every call of the library can be captured into a HIP graph
 // (memset nodes are the one node kind callers are told to avoid on this platform).
 int launch_zero_words(void* p, size_t words, hipStream_t stream);
+// Zeroes the rows of out[num_rows, dim] whose bit in `skip` is clear (rows with a set bit are left as they are).
+int launch_zero_rows_unless(float* out, const uint32_t* skip, long long num_rows, int dim, hipStream_t stream);
 
 // ---------------------------------------------------------------- execution plan layout
-// One caller-owned buffer: ptr[P+1] | row[P] | flags[P] | col[S], each part 256-byte aligned
-// (contents described in schedule.hip).  Offsets depend on the group count alone.
+// One caller-owned buffer: ptr[P+1] | row[P] | flags[P] | single[ceil(N/32)] | col[S], each part
+// 256-byte aligned (contents described in schedule.hip).  Offsets depend on the group count and the
+// vertex count alone.
 struct PlanView {
     int* ptr;
     int* row;
     uint8_t* flags;
+    uint32_t* single;   // bit r: row r consists of exactly one non-empty group (it is written by one plain store)
     int* col;
 };
 inline size_t plan_align(size_t x) { return (x + 255) / 256 * 256; }
-inline size_t plan_bytes(long long num_parts, long long num_slots)
+inline size_t plan_single_words(long long num_nodes)
+{
+    return (static_cast<size_t>(num_nodes > 0 ? num_nodes : 0) + 31) / 32;
+}
+inline size_t plan_bytes(long long num_parts, long long num_slots, long long num_nodes)
 {
     const size_t p = static_cast<size_t>(num_parts > 0 ? num_parts : 0);
     const size_t s = static_cast<size_t>(num_slots > 0 ? num_slots : 0);
-    return plan_align(4 * (p + 1)) + plan_align(4 * p) + plan_align(p) + plan_align(4 * s);
+    return plan_align(4 * (p + 1)) + plan_align(4 * p) + plan_align(p) + plan_align(4 * plan_single_words(num_nodes)) +
+           plan_align(4 * s);
 }
-inline PlanView plan_view(void* plan, long long num_parts)
+inline PlanView plan_view(void* plan, long long num_parts, long long num_nodes)
 {
     const size_t p = static_cast<size_t>(num_parts);
     char* b = static_cast<char*>(plan);
     PlanView v;
     v.ptr = reinterpret_cast<int*>(b);
-    v.row = reinterpret_cast<int*>(b + plan_align(4 * (p + 1)));
-    v.flags = reinterpret_cast<uint8_t*>(b + plan_align(4 * (p + 1)) + plan_align(4 * p));
-    v.col = reinterpret_cast<int*>(b + plan_align(4 * (p + 1)) + plan_align(4 * p) + plan_align(p));
+    b += plan_align(4 * (p + 1));
+    v.row = reinterpret_cast<int*>(b);
+    b += plan_align(4 * p);
+    v.flags = reinterpret_cast<uint8_t*>(b);
+    b += plan_align(p);
+    v.single = reinterpret_cast<uint32_t*>(b);
+    b += plan_align(4 * plan_single_words(num_nodes));
+    v.col = reinterpret_cast<int*>(b);
     return v;
 }
 

@@ -123,7 +123,7 @@ const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& ro
     PlanEntry e{part_ptr.data_ptr(), col.data_ptr(), rows.data_ptr(), num_parts,
                 static_cast<int64_t>(part_ptr._version()), static_cast<int64_t>(col._version()),
                 static_cast<int64_t>(rows._version()), dc, part_ptr, col, rows, Tensor(), nullptr};
-    const size_t bytes = eppgcn_plan_bytes(num_parts, num_slots);
+    const size_t bytes = eppgcn_plan_bytes(num_parts, num_slots, num_nodes);
     void* base = nullptr;
     e.plan = aligned_bytes(bytes, part_ptr, &base);
     e.plan_ptr = base;

@@ -540,6 +540,95 @@ int launch_zero_words(void* p, size_t words, hipStream_t stream)
     return kOk;
 }
 
+// out[num_rows, dim]: one thread per vector of VW floats; a row whose bit in `skip` is set is left alone.
+// Index: unsigned when the vector count fits in 32 bits (the row of a vector is then a 32-bit division).
+template <int VW, class Index>
+__global__ __launch_bounds__(256) void zero_rows_unless_kernel(float* __restrict__ out, const uint32_t* __restrict__ skip,
+                                                               Index total_vecs, Index vecs_per_row)
+{
+    typedef float fvec __attribute__((ext_vector_type(VW)));
+    const Index stride = static_cast<Index>(gridDim.x) * blockDim.x;
+    for (Index i = static_cast<Index>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs; i += stride) {
+        const Index r = i / vecs_per_row;
+        if (!((skip[r >> 5] >> (r & 31)) & 1u)) {
+            if constexpr (VW == 1) {
+                __builtin_nontemporal_store(0.f, out + i);
+            } else {
+                fvec z = {};
+                __builtin_nontemporal_store(z, reinterpret_cast<fvec*>(out) + i);
+            }
+        }
+        if (total_vecs - i <= stride) break;      // the next index would run past the end (and could wrap)
+    }
+}
+
+// The same for a 16-byte aligned matrix of rows of at least 4 floats, whatever the row length: one
+// thread per 16 bytes of the flat array.  A vector lies in one row or straddles two; it is written
+// whole when no row it touches is skipped and float by float otherwise.
+template <class Index>
+__global__ __launch_bounds__(256) void zero_flat_unless_kernel(float* __restrict__ out, const uint32_t* __restrict__ skip,
+                                                               Index total_floats, Index dim)
+{
+    typedef float fvec4 __attribute__((ext_vector_type(4)));
+    const Index vecs = total_floats / 4;
+    const Index stride = static_cast<Index>(gridDim.x) * blockDim.x;
+    const Index tid = static_cast<Index>(blockIdx.x) * blockDim.x + threadIdx.x;
+    for (Index j = tid; j < vecs; j += stride) {
+        const Index f0 = 4 * j;
+        const Index r0 = f0 / dim;
+        const Index in_r0 = (r0 + 1) * dim - f0;           // floats of the vector that belong to row r0
+        const Index r1 = in_r0 < 4 ? r0 + 1 : r0;
+        const bool keep0 = ((skip[r0 >> 5] >> (r0 & 31)) & 1u) != 0;
+        const bool keep1 = ((skip[r1 >> 5] >> (r1 & 31)) & 1u) != 0;
+        if (!keep0 && !keep1) {
+            fvec4 z = {};
+            __builtin_nontemporal_store(z, reinterpret_cast<fvec4*>(out) + j);
+        } else if (keep0 != keep1) {
+#pragma unroll
+            for (Index k = 0; k < 4; ++k)
+                if (!(k < in_r0 ? keep0 : keep1)) out[f0 + k] = 0.f;
+        }
+        if (vecs - j <= stride) break;                     // the next index would run past the end (and could wrap)
+    }
+    const Index tail = 4 * vecs;                            // up to 3 floats of the last row
+    if (tid < total_floats - tail) {
+        const Index r = (tail + tid) / dim;
+        if (!((skip[r >> 5] >> (r & 31)) & 1u)) out[tail + tid] = 0.f;
+    }
+}
+
+template <class Index>
+static void launch_zero_rows_typed(float* out, const uint32_t* skip, long long num_rows, int dim, hipStream_t stream)
+{
+    const uintptr_t a = reinterpret_cast<uintptr_t>(out);
+    const long long floats = num_rows * dim;
+    if (dim >= 4 && a % 16 == 0) {
+        long long blocks = (floats / 4 + 255) / 256;
+        if (blocks > 256 * 64) blocks = 256 * 64;
+        if (blocks < 1) blocks = 1;
+        hipLaunchKernelGGL((zero_flat_unless_kernel<Index>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, out,
+                           skip, static_cast<Index>(floats), static_cast<Index>(dim));
+        return;
+    }
+    const int vw = (dim % 2 == 0 && a % 8 == 0) ? 2 : 1;
+    const long long total = floats / vw;
+    long long blocks = (total + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    const dim3 grid(static_cast<unsigned>(blocks)), block(256);
+    const Index t = static_cast<Index>(total), v = static_cast<Index>(dim / vw);
+    if (vw == 2) hipLaunchKernelGGL((zero_rows_unless_kernel<2, Index>), grid, block, 0, stream, out, skip, t, v);
+    else hipLaunchKernelGGL((zero_rows_unless_kernel<1, Index>), grid, block, 0, stream, out, skip, t, v);
+}
+
+int launch_zero_rows_unless(float* out, const uint32_t* skip, long long num_rows, int dim, hipStream_t stream)
+{
+    if (num_rows <= 0 || dim <= 0) return kOk;
+    if (num_rows * dim < (1ll << 32)) launch_zero_rows_typed<unsigned>(out, skip, num_rows, dim, stream);
+    else launch_zero_rows_typed<unsigned long long>(out, skip, num_rows, dim, stream);
+    EPPGCN_HIP(hipGetLastError());
+    return kOk;
+}
+
 size_t scan_workspace_bytes(long long length, int tile)
 {
     const long long tiles = (length + tile - 1) / tile;

@@ -12,6 +12,8 @@
 //                bit2 this group continues the previous plan entry (same row, next original
 //                index), bit3 the next plan entry continues this one
 //     col[S]     column ids, group by group in plan order
+//     single[ceil(N/32)]  bit r set: row r has exactly one group and the group is not empty; the
+//                kernel writes such a row with one plain store, so the output clear can skip it
 //
 // The re-ordering changes no result, only which groups run together.  It depends on the graph
 // and the groups alone: a caller builds it once and passes it to every aggregation call.
@@ -159,6 +161,7 @@ __global__ __launch_bounds__(256) void plan_fill_kernel(const int* __restrict__ 
         }
         const bool joins_left = prev && q > 0 && order[q - 1] == p - 1;
         const bool joins_right = next && q + 1 < num_parts && order[q + 1] == p + 1;
+        if (end > beg && !prev && !next) atomicOr(plan.single + (row >> 5), 1u << (row & 31));
         plan.row[q] = row;
         plan.flags[q] = static_cast<uint8_t>((prev ? 1 : 0) | (next ? 2 : 0) | (joins_left ? 4 : 0) | (joins_right ? 8 : 0));
     }
@@ -228,8 +231,8 @@ int launch_build_plan(const int* part_ptr, const int* col, const int* part2node,
                       size_t workspace_bytes, hipStream_t stream)
 {
     if (num_parts <= 0) return kOk;
-    if (plan_size < plan_bytes(num_parts, num_slots)) {
-        set_error("build_plan: plan buffer smaller than eppgcn_plan_bytes(num_parts, num_slots)");
+    if (plan_size < plan_bytes(num_parts, num_slots, num_nodes)) {
+        set_error("build_plan: plan buffer smaller than eppgcn_plan_bytes(num_parts, num_slots, num_nodes)");
         return kErrInvalidArgument;
     }
     const size_t slab = align256(sizeof(int) * (static_cast<size_t>(num_parts) + 1));
@@ -262,7 +265,8 @@ int launch_build_plan(const int* part_ptr, const int* col, const int* part2node,
     const int tiles = (num_parts + kScanTile - 1) / kScanTile;
     hipLaunchKernelGGL(plan_scan_init_kernel, dim3((tiles + 255) / 256), dim3(256), 0, stream, st, desc, tiles);
     EPPGCN_HIP(hipGetLastError());
-    PlanView v = plan_view(plan, num_parts);
+    PlanView v = plan_view(plan, num_parts, num_nodes);
+    if (int rc = launch_zero_words(v.single, plan_single_words(num_nodes), stream)) return rc;
     hipLaunchKernelGGL(exclusive_scan_kernel, dim3(tiles), dim3(kScanBlock), 0, stream, sizes, v.ptr, num_parts, tiles,
                        st, desc);
     EPPGCN_HIP(hipGetLastError());

@@ -83,12 +83,16 @@ int eppgcn_feature_workspace_pitch(int dim);
  *   forward groups : part_pointers + column_index + part2node (ids = NULL)
  *   backward path  : part_pointer + edge_list + ids (part2node = NULL)
  * num_slots = number of slots the groups cover (num_edges, or the kept length).  The plan must
- * be rebuilt when the groups change.  No counterpart in the reference. */
+ * be rebuilt when the groups change, and an aggregation call that is given a plan must be given the
+ * num_parts and num_nodes the plan was built with (its layout depends on both).  The plan also
+ * records, one bit per vertex, the rows that consist of a single non-empty group: the kernel
+ * writes those with one plain store, so the output clear of a planned call skips them.
+ * No counterpart in the reference. */
 /* 1 when a plan is expected to pay off: the [num_nodes, dim] feature table (192 MB or more) does
  * not stay resident in the last-level caches by itself.  Measured: at 268 MB the plan takes the
  * width-16 forward from 2.03 to 1.35 ms, at 67 MB it costs 5 % (its partial sums need atomics). */
 int eppgcn_plan_recommended(int64_t num_nodes, int dim);
-size_t eppgcn_plan_bytes(int64_t num_parts, int64_t num_slots);
+size_t eppgcn_plan_bytes(int64_t num_parts, int64_t num_slots, int64_t num_nodes);
 size_t eppgcn_plan_workspace_bytes(int64_t num_parts);
 int eppgcn_build_plan(const int32_t* part_pointers, const int32_t* column_index,
                       const int32_t* part2node, const int32_t* ids, int num_parts, int64_t num_slots,

@@ -286,6 +286,8 @@ def test_plan_is_a_stable_column_block_reordering(api, name, ps):
         jr = nxt & np.concatenate([order[1:] == order[:-1] + 1, [False]])
         assert np.array_equal(flags & 1, prev) and np.array_equal((flags >> 1) & 1, nxt)
         assert np.array_equal((flags >> 2) & 1, jl) and np.array_equal((flags >> 3) & 1, jr)
+        # rows made of one group are recorded for the output clear to skip
+        assert np.array_equal(plan.single_rows().cpu().numpy(), groups_per_row == 1)
 
 
 @pytest.mark.parametrize("rounds", [0, 1, 3])
@@ -312,14 +314,19 @@ def test_planned_aggregation_exact_integer_sums(api, rounds, dim, shift):
             pp, p2n = co.build_part(ps, indptr)
             dpp, dcol, dp2n = dev(pp), dev(col), dev(p2n)
             plan = api.build_plan(dpp, dcol, p2n.size, col.size, n, dim, part2node=dp2n)
-            got = api.spmm_forward(dev(x), dcol, dev(s), dpp, dp2n, part_size=ps, plan=plan)
+            # the output buffer arrives full of NaN: rows the clear skips must be written whole
+            got = api.spmm_forward(dev(x), dcol, dev(s), dpp, dp2n, part_size=ps, plan=plan,
+                                   out=torch.full((n, dim), float("nan"), device="cuda"))
             assert np.array_equal(got.cpu().numpy().astype(np.float64), want), f"forward ps={ps}"
             oid, oedge, bpp, p = _gpu_path(api, indptr, col, src, 5, ps)
             if p == 0:
                 continue
             bplan = api.build_plan(bpp, oedge, p, int(keep.sum()), n, dim, ids=oid)
             dy = dev((x * src[:, None]).astype(np.float32))
-            gb = api.ours_backward(dy, oid, bpp, oedge, dev(s), p, part_size=ps, plan=bplan)
+            kept_per_row = np.bincount(cf.row_index(indptr)[keep], minlength=n)
+            assert np.array_equal(bplan.single_rows().cpu().numpy(), (kept_per_row >= 1) & (kept_per_row <= ps))
+            gb = api.ours_backward(dy, oid, bpp, oedge, dev(s), p, part_size=ps, plan=bplan,
+                                   out=torch.full((n, dim), float("nan"), device="cuda"))
             assert np.array_equal(gb.cpu().numpy().astype(np.float64), want_b), f"pruned ps={ps}"
     finally:
         api.set_rounds(0)
@@ -327,7 +334,7 @@ def test_planned_aggregation_exact_integer_sums(api, rounds, dim, shift):
 
 
 @pytest.mark.parametrize("name", ["isolated", "hub", "medium"])
-@pytest.mark.parametrize("dim", [16, 22, 100])
+@pytest.mark.parametrize("dim", [16, 22, 100, 7, 5, 3])
 def test_planned_aggregation_within_tolerance(api, name, dim):
     indptr, col = GRAPHS[name]()
     n = indptr.size - 1
@@ -338,7 +345,8 @@ def test_planned_aggregation_within_tolerance(api, name, dim):
     for ps in (4, 32):
         pp, p2n = co.build_part(ps, indptr)
         plan = api.build_plan(dev(pp), dev(col), p2n.size, col.size, n, dim, part2node=dev(p2n))
-        got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp), dev(p2n), part_size=ps, plan=plan)
+        got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp), dev(p2n), part_size=ps, plan=plan,
+                               out=torch.full((n, dim), float("nan"), device="cuda"))
         assert_close(got.cpu().numpy(), want, bound, f"{name} D={dim} ps={ps} planned")
 
 
@@ -690,8 +698,12 @@ def test_aggregation_with_empty_groups(api, name, dim):
         plan = api.build_plan(dev(pp2), dev(col), p2n2.size, col.size, n, dim, part2node=dev(p2n2))
     finally:
         api.set_plan_shift(0)
-    got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp2), dev(p2n2), part_size=5, plan=plan)
+    got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp2), dev(p2n2), part_size=5, plan=plan,
+                           out=torch.full((n, dim), float("nan"), device="cuda"))
     assert_close(got.cpu().numpy(), want, bound, "empty groups with a plan")
+    groups = np.bincount(p2n2, minlength=n)
+    filled = np.bincount(p2n2[np.diff(pp2) > 0], minlength=n)
+    assert np.array_equal(plan.single_rows().cpu().numpy(), (groups == 1) & (filled == 1))
 
 
 @pytest.mark.parametrize("dim", [16, 22, 7, 64])
@@ -715,6 +727,11 @@ def test_aggregation_with_misaligned_feature_buffers(api, dim, shift_in, shift_o
         out.fill_(3.0)
         api.spmm_forward(xin, dev(col), dev(s), pp, p2n, part_size=8, out=out, workspace=workspace)
         assert_close(out.cpu().numpy(), want, bound, f"forward, workspace={workspace}")
+    # with a plan the output clear skips single-group rows: the narrower clears must do the same
+    plan = api.build_plan(pp, dev(col), p2n.numel(), col.size, n, dim, part2node=p2n)
+    out.fill_(float("nan"))
+    api.spmm_forward(xin, dev(col), dev(s), pp, p2n, part_size=8, out=out, plan=plan)
+    assert_close(out.cpu().numpy(), want, bound, "forward with a plan")
     src = rng.random(n) < 0.4
     degs = torch.zeros(n, dtype=torch.int32, device="cuda")
     ids, edge_list, v = api.mark_compact(p2n, pp, dev(col), dev(src), None, degs, True)
