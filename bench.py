@@ -178,12 +178,13 @@ def main():
 
     def bwd22():
         capi.ours_backward(dy22, p_last.ids, p_last.part_pointer, p_last.edge_list, g.degrees, p_last.num_parts,
-                           p_last.part_size, 2, 4, 16, out22, workspace=ws22, plan=p_last.plan)
+                           p_last.part_size, 2, 4, 16, out22, workspace=ws22, plan=p_last.plan,
+                           gathered_rows=p_last.gathered_rows)
 
     def bwd16():
         capi.ours_backward(dy16, p_first.ids, p_first.part_pointer, p_first.edge_list, g.degrees,
                            p_first.num_parts, p_first.part_size, 1, 4, 16, out16, workspace=ws16,
-                           plan=p_first.plan)
+                           plan=p_first.plan, gathered_rows=p_first.gathered_rows)
 
     kernels = [
         ("fwd_agg_d16", fwd16, workload.bytes_forward(n, e, 16)),

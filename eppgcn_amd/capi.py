@@ -25,6 +25,7 @@ EXPORTS = [
     "eppgcn_feature_workspace_pitch", "eppgcn_update_forward", "eppgcn_update_backward_input",
     "eppgcn_update_workspace_bytes", "eppgcn_update_backward_weight", "eppgcn_update_supported",
     "eppgcn_mark_compact_workspace_bytes", "eppgcn_mark_compact", "eppgcn_set_plan_length_classes",
+    "eppgcn_mark_gathered_rows",
 ]
 
 _lib = None
@@ -58,7 +59,9 @@ def load():
     lib.eppgcn_build_plan.restype = i
     lib.eppgcn_spmm_forward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, sz, p, p]
     lib.eppgcn_spmm_backward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, sz, p, p]
-    lib.eppgcn_ours_backward.argtypes = [p, p, p, p, p, p, i, i, i, i, i, i, i, p, sz, p, p]
+    lib.eppgcn_ours_backward.argtypes = [p, p, p, p, p, p, i, i, i, i, i, i, i, p, sz, p, p, p]
+    lib.eppgcn_mark_gathered_rows.argtypes = [p, i64, i, p, p, C.POINTER(i64), p]
+    lib.eppgcn_mark_gathered_rows.restype = i
     lib.eppgcn_mask_forward.argtypes = [p, p, p, p, p, p, p, i, i64, i, i, i, p]
     lib.eppgcn_compact_workspace_bytes.argtypes = [i64]
     lib.eppgcn_compact_workspace_bytes.restype = sz
@@ -328,8 +331,22 @@ def spmm_forward(feats, column_index, degrees, part_ptr, part2node, part_size=32
     return out
 
 
+def mark_gathered_rows(edge_list, valid_len: int, num_nodes: int):
+    """-> (bitmap int32[(N+31)//32] with bit c set for every c in edge_list[:valid_len], number of set bits)."""
+    lib = load()
+    _dev(edge_list, torch.int32, "edge_list")
+    if edge_list.numel() < valid_len:
+        raise EppgcnError("edge_list is shorter than valid_len")
+    bitmap = torch.empty((int(num_nodes) + 31) // 32 + 1, dtype=torch.int32, device=edge_list.device)
+    count = C.c_int64(0)
+    _check(lib.eppgcn_mark_gathered_rows(_ptr(edge_list), int(valid_len), int(num_nodes), _ptr(bitmap),
+                                         _ptr(bitmap[-1:]), C.byref(count), _stream()))
+    return bitmap[:-1], int(count.value)
+
+
 def ours_backward(d_output, ids, part_pointer, edge_list, degrees, num_parts, part_size=32, layer=1,
-                  blockx=4, blocky=16, out=None, workspace=True, plan=None):
+                  blockx=4, blocky=16, out=None, workspace=True, plan=None, gathered_rows=None):
+    """``gathered_rows``: the bitmap of ``mark_gathered_rows`` for this path, or None."""
     lib = load()
     _dev(d_output, torch.float32, "d_output"); _dev(ids, torch.int32, "ids")
     _dev(part_pointer, torch.int32, "part_pointer"); _dev(edge_list, torch.int32, "edge_list")
@@ -343,7 +360,7 @@ def ours_backward(d_output, ids, part_pointer, edge_list, degrees, num_parts, pa
     _check(lib.eppgcn_ours_backward(_ptr(out), _ptr(d_output), _ptr(ids), _ptr(part_pointer), _ptr(edge_list),
                                     _ptr(degrees), n, dim, int(num_parts), part_size, layer, blockx, blocky,
                                     _ptr(ws), 0 if ws is None else ws.numel(),
-                                    _plan_ptr(plan, int(num_parts), n), _stream()))
+                                    _plan_ptr(plan, int(num_parts), n), _ptr(gathered_rows), _stream()))
     return out
 
 

@@ -140,51 +140,76 @@ struct PlanGroups {
 // row pitch ld_dst is a multiple of 4 floats, so every thread writes one aligned float4; rows
 // padded to whole 32-byte sectors let the gather fetch fewer sectors per row and use 16-byte
 // loads for widths such as 22 whose rows are only 8-byte aligned in the caller's layout.
-__global__ __launch_bounds__(256) void scale_rows_kernel(float* __restrict__ dst, const float* __restrict__ src,
-                                                         const float* __restrict__ scale, long long total_vecs,
-                                                         int vecs_per_row, int dim, bool pairs)
+//
+// `rows` (optional): one bit per row; a row whose bit is clear is skipped (the caller knows that
+// no group gathers it, e.g. the rows outside the kept path of a pruned backward), so the pass costs
+// what the gathered rows cost.  Index: unsigned when the element count fits in 32 bits.
+__device__ inline bool row_wanted(const uint32_t* __restrict__ rows, unsigned long long r)
 {
-    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
-    for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs; i += stride) {
-        const long long r = i / vecs_per_row;
-        const int c0 = static_cast<int>(i - r * vecs_per_row) * 4;
-        const float s = scale[r];
-        const float* row = src + r * dim;
-        float4 v;
-        if (pairs) {                 // even width, 8-byte aligned source: a pair is all in or all out
-            const float2 lo = c0 < dim ? *reinterpret_cast<const float2*>(row + c0) : make_float2(0.f, 0.f);
-            const float2 hi = c0 + 2 < dim ? *reinterpret_cast<const float2*>(row + c0 + 2) : make_float2(0.f, 0.f);
-            v = make_float4(s * lo.x, s * lo.y, s * hi.x, s * hi.y);
-        } else {
-            v.x = c0 + 0 < dim ? s * row[c0 + 0] : 0.f;
-            v.y = c0 + 1 < dim ? s * row[c0 + 1] : 0.f;
-            v.z = c0 + 2 < dim ? s * row[c0 + 2] : 0.f;
-            v.w = c0 + 3 < dim ? s * row[c0 + 3] : 0.f;
+    return rows == nullptr || ((rows[r >> 5] >> (r & 31)) & 1u) != 0;
+}
+
+template <class Index>
+__global__ __launch_bounds__(256) void scale_rows_kernel(float* __restrict__ dst, const float* __restrict__ src,
+                                                         const float* __restrict__ scale,
+                                                         const uint32_t* __restrict__ rows, Index total_vecs,
+                                                         Index vecs_per_row, Index dim, bool pairs)
+{
+    const Index stride = static_cast<Index>(gridDim.x) * blockDim.x;
+    for (Index i = static_cast<Index>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs; i += stride) {
+        const Index r = i / vecs_per_row;
+        if (row_wanted(rows, r)) {
+            const Index c0 = (i - r * vecs_per_row) * 4;
+            const float s = scale[r];
+            const float* row = src + static_cast<size_t>(r) * dim;
+            float4 v;
+            if (pairs) {                 // even width, 8-byte aligned source: a pair is all in or all out
+                const float2 lo = c0 < dim ? *reinterpret_cast<const float2*>(row + c0) : make_float2(0.f, 0.f);
+                const float2 hi = c0 + 2 < dim ? *reinterpret_cast<const float2*>(row + c0 + 2) : make_float2(0.f, 0.f);
+                v = make_float4(s * lo.x, s * lo.y, s * hi.x, s * hi.y);
+            } else {
+                v.x = c0 + 0 < dim ? s * row[c0 + 0] : 0.f;
+                v.y = c0 + 1 < dim ? s * row[c0 + 1] : 0.f;
+                v.z = c0 + 2 < dim ? s * row[c0 + 2] : 0.f;
+                v.w = c0 + 3 < dim ? s * row[c0 + 3] : 0.f;
+            }
+            *reinterpret_cast<float4*>(dst + static_cast<size_t>(i) * 4) = v;
         }
-        *reinterpret_cast<float4*>(dst + i * 4) = v;
+        if (total_vecs - i <= stride) break;      // the next index would run past the end (and could wrap)
     }
 }
 
 // In-place / unpadded form for a workspace that aliases the input: dst[i] = scale[row(i)] * src[i].
+template <class Index>
 __global__ __launch_bounds__(256) void scale_rows_flat_kernel(float* __restrict__ dst, const float* __restrict__ src,
-                                                              const float* __restrict__ scale, long long total, int dim)
+                                                              const float* __restrict__ scale,
+                                                              const uint32_t* __restrict__ rows, Index total, Index dim)
 {
-    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
-    for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride)
-        dst[i] = scale[i / dim] * src[i];
+    const Index stride = static_cast<Index>(gridDim.x) * blockDim.x;
+    for (Index i = static_cast<Index>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const Index r = i / dim;
+        if (row_wanted(rows, r)) dst[i] = scale[r] * src[i];
+        if (total - i <= stride) break;
+    }
 }
 
 // Same for rows of a multiple of 4 floats and 16-byte aligned buffers: one float4 per thread.
+template <class Index>
 __global__ __launch_bounds__(256) void scale_rows_flat4_kernel(float4* dst, const float4* src,
-                                                               const float* __restrict__ scale, long long total_vecs,
-                                                               int vecs_per_row)
+                                                               const float* __restrict__ scale,
+                                                               const uint32_t* __restrict__ rows, Index total_vecs,
+                                                               Index vecs_per_row)
 {
-    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
-    for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs; i += stride) {
-        const float s = scale[i / vecs_per_row];
-        float4 v = src[i];
-        v.x *= s; v.y *= s; v.z *= s; v.w *= s;
-        dst[i] = v;
+    const Index stride = static_cast<Index>(gridDim.x) * blockDim.x;
+    for (Index i = static_cast<Index>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs; i += stride) {
+        const Index r = i / vecs_per_row;
+        if (row_wanted(rows, r)) {
+            const float s = scale[r];
+            float4 v = src[i];
+            v.x *= s; v.y *= s; v.z *= s; v.w *= s;
+            dst[i] = v;
+        }
+        if (total_vecs - i <= stride) break;
     }
 }
 
@@ -588,32 +613,40 @@ size_t feature_workspace_floats(long long num_nodes, int dim)
     return static_cast<size_t>(num_nodes) * static_cast<size_t>(workspace_pitch(dim));
 }
 
-static int launch_scale_rows(float* dst, const float* src, const float* scale, int num_nodes, int dim, int ld_dst,
-                             hipStream_t stream)
+template <class Index>
+static void launch_scale_rows_typed(float* dst, const float* src, const float* scale, const uint32_t* rows,
+                                    long long num_nodes, int dim, int ld_dst, hipStream_t stream)
+{
+    auto grid_for = [](long long threads) {
+        long long blocks = (threads + 255) / 256;
+        if (blocks > 256 * 32) blocks = 256 * 32;
+        return dim3(static_cast<unsigned>(blocks < 1 ? 1 : blocks));
+    };
+    if (dst == src || ld_dst == dim) {
+        const long long total = num_nodes * dim;
+        if (dim % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0) {
+            hipLaunchKernelGGL((scale_rows_flat4_kernel<Index>), grid_for(total / 4), dim3(256), 0, stream,
+                               reinterpret_cast<float4*>(dst), reinterpret_cast<const float4*>(src), scale, rows,
+                               static_cast<Index>(total / 4), static_cast<Index>(dim / 4));
+            return;
+        }
+        hipLaunchKernelGGL((scale_rows_flat_kernel<Index>), grid_for(total), dim3(256), 0, stream, dst, src, scale, rows,
+                           static_cast<Index>(total), static_cast<Index>(dim));
+    } else {
+        const long long vecs = num_nodes * (ld_dst / 4);
+        hipLaunchKernelGGL((scale_rows_kernel<Index>), grid_for(vecs), dim3(256), 0, stream, dst, src, scale, rows,
+                           static_cast<Index>(vecs), static_cast<Index>(ld_dst / 4), static_cast<Index>(dim),
+                           dim % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 8 == 0);
+    }
+}
+
+static int launch_scale_rows(float* dst, const float* src, const float* scale, const uint32_t* rows, int num_nodes,
+                             int dim, int ld_dst, hipStream_t stream)
 {
     if (static_cast<long long>(num_nodes) * dim == 0) return kOk;
-    if (dst == src || ld_dst == dim) {
-        const long long total = static_cast<long long>(num_nodes) * dim;
-        if (dim % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0) {
-            long long blocks = (total / 4 + 255) / 256;
-            if (blocks > 256 * 32) blocks = 256 * 32;
-            hipLaunchKernelGGL(scale_rows_flat4_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
-                               reinterpret_cast<float4*>(dst), reinterpret_cast<const float4*>(src), scale, total / 4,
-                               dim / 4);
-            EPPGCN_HIP(hipGetLastError());
-            return kOk;
-        }
-        long long blocks = (total + 255) / 256;
-        if (blocks > 256 * 32) blocks = 256 * 32;
-        hipLaunchKernelGGL(scale_rows_flat_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, dst, src,
-                           scale, total, dim);
-    } else {
-        const long long vecs = static_cast<long long>(num_nodes) * (ld_dst / 4);
-        long long blocks = (vecs + 255) / 256;
-        if (blocks > 256 * 32) blocks = 256 * 32;
-        hipLaunchKernelGGL(scale_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, dst, src, scale,
-                           vecs, ld_dst / 4, dim, dim % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 8 == 0);
-    }
+    const long long elems = static_cast<long long>(num_nodes) * (ld_dst > dim ? ld_dst : dim);
+    if (elems < (1ll << 32)) launch_scale_rows_typed<unsigned>(dst, src, scale, rows, num_nodes, dim, ld_dst, stream);
+    else launch_scale_rows_typed<unsigned long long>(dst, src, scale, rows, num_nodes, dim, ld_dst, stream);
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }
@@ -631,7 +664,8 @@ static int vector_width(int pitch, int width, const void* p)
 template <class Groups>
 static int aggregate_dispatch(float* out, const float* in, const int* col, const float* scale, Groups g,
                               int num_nodes, int dim, int num_parts, int group_size, float* workspace,
-                              hipStream_t stream, double* sink, double* sink2, const uint32_t* single_rows = nullptr)
+                              hipStream_t stream, double* sink, double* sink2, const uint32_t* single_rows = nullptr,
+                              const uint32_t* gathered_rows = nullptr)
 {
     const bool prescaled = workspace != nullptr;
     int ld_in = dim;
@@ -646,7 +680,7 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
         // in == nullptr: the caller (the dense update) already wrote the scaled, padded rows
         ld_in = workspace == in ? dim : workspace_pitch(dim);
         if (in)
-            if (int rc = launch_scale_rows(workspace, in, scale, num_nodes, dim, ld_in, stream)) return rc;
+            if (int rc = launch_scale_rows(workspace, in, scale, gathered_rows, num_nodes, dim, ld_in, stream)) return rc;
         in = workspace;
     }
     KernelTimer timer(stream, sink, sink2);   // brackets the aggregation kernel alone
@@ -700,18 +734,20 @@ int aggregate_forward_groups(float* out, const float* in, const int* col, const 
                               group_size, workspace, stream, sink, sink2);
 }
 
+// gathered_rows: nullptr, or one bit per vertex, set for every vertex that occurs in edge_list; the
+// pre-scaling pass then skips the rows no group reads.
 int aggregate_compacted_groups(float* out, const float* in, const int* ids, const int* part_ptr,
                                const int* edge_list, const float* scale, const void* plan, int num_nodes, int dim,
-                               int num_parts, int group_size, float* workspace, hipStream_t stream, double* sink,
-                               double* sink2)
+                               int num_parts, int group_size, float* workspace, const uint32_t* gathered_rows,
+                               hipStream_t stream, double* sink, double* sink2)
 {
     if (plan && workspace && num_parts > 0) {
         const PlanView v = plan_view(const_cast<void*>(plan), num_parts, num_nodes);
         return aggregate_dispatch(out, in, v.col, scale, PlanGroups{v.ptr, v.row, v.flags}, num_nodes, dim, num_parts,
-                                  group_size, workspace, stream, sink, sink2, v.single);
+                                  group_size, workspace, stream, sink, sink2, v.single, gathered_rows);
     }
     return aggregate_dispatch(out, in, edge_list, scale, CompactedGroups{part_ptr, ids}, num_nodes, dim, num_parts,
-                              group_size, workspace, stream, sink, sink2);
+                              group_size, workspace, stream, sink, sink2, nullptr, gathered_rows);
 }
 
 }  // namespace eppgcn

@@ -14,7 +14,7 @@ namespace eppgcn {
 int aggregate_forward_groups(float*, const float*, const int*, const float*, const int*, const int*, const void*, int,
                              int, int, int, float*, hipStream_t, double*, double*);
 int aggregate_compacted_groups(float*, const float*, const int*, const int*, const int*, const float*, const void*,
-                               int, int, int, int, float*, hipStream_t, double*, double*);
+                               int, int, int, int, float*, const uint32_t*, hipStream_t, double*, double*);
 size_t plan_workspace_bytes(long long);
 int schedule_shift(int);
 void set_schedule_shift(int);
@@ -41,6 +41,7 @@ int launch_mark_compact(const int*, const int*, const int*, const uint8_t*, uint
 int launch_split(bool, const int*, int, int, int*, int*, long long, bool, void*, hipStream_t);
 int launch_count_nonzero(const int*, long long, int*, hipStream_t);
 int launch_ginfo_hist(const int*, long long, int*, hipStream_t);
+int launch_mark_listed_rows(const int*, long long, long long, uint32_t*, int*, hipStream_t);
 
 // ---- errors
 static thread_local std::string g_last_error;
@@ -79,7 +80,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 6; }
+int eppgcn_abi_version(void) { return 7; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -126,7 +127,7 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
 int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
                          const int32_t* edge_list, const float* degrees, int num_nodes, int dim, int num_parts,
                          int part_size, int layer, int blockx, int blocky, float* workspace,
-                         size_t workspace_floats, const void* plan, void* stream)
+                         size_t workspace_floats, const void* plan, const uint32_t* gathered_rows, void* stream)
 {
     // part_size only sizes the work per wave (the reference's kernel ignores it, EPPGCN_kernel.cu:636)
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
@@ -142,7 +143,8 @@ int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* i
     EPPGCN_REQUIRE(!workspace || workspace == d_output || workspace_floats >= feature_workspace_floats(num_nodes, dim),
                    "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
     return aggregate_compacted_groups(d_input, d_output, ids, part_pointer, edge_list, degrees, plan, num_nodes,
-                                      dim, num_parts, part_size > 0 ? part_size : 1, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms,
+                                      dim, num_parts, part_size > 0 ? part_size : 1, workspace, gathered_rows,
+                                      static_cast<hipStream_t>(stream), &g_back_agg_ms,
                                       layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr);
 }
 
@@ -242,6 +244,23 @@ int eppgcn_mark_compact(const int32_t* part2node, const int32_t* part_pointers, 
         ScanState host;
         if (int rc = read_state(workspace, s, &host)) return rc;
         *h_valid_len = host.counts[0];
+    }
+    return kOk;
+}
+
+int eppgcn_mark_gathered_rows(const int32_t* edge_list, int64_t valid_len, int num_nodes, uint32_t* bitmap,
+                              int32_t* d_count, int64_t* h_count, void* stream)
+{
+    EPPGCN_REQUIRE(valid_len >= 0 && valid_len < (1ll << 31) && num_nodes >= 0, "lengths must be non-negative int32");
+    EPPGCN_REQUIRE(d_count && (num_nodes == 0 || bitmap) && (valid_len == 0 || edge_list), "null pointer");
+    EPPGCN_REQUIRE(aligned(bitmap, 4) && aligned(d_count, 4), "bitmap and counter must be 4-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (int rc = launch_mark_listed_rows(edge_list, valid_len, num_nodes, bitmap, d_count, s)) return rc;
+    if (h_count) {
+        int v = 0;
+        EPPGCN_HIP(hipMemcpyAsync(&v, d_count, sizeof(int), hipMemcpyDeviceToHost, s));
+        EPPGCN_HIP(hipStreamSynchronize(s));
+        *h_count = v;
     }
     return kOk;
 }

@@ -82,6 +82,7 @@ struct PlanEntry {
     const void* col;
     const void* rows;
     int64_t num_parts;
+    int64_t num_nodes;          // the plan's layout depends on it
     int64_t version_part, version_col, version_rows;
     int dim_class;
     Tensor keep_part, keep_col, keep_rows, plan;
@@ -111,7 +112,7 @@ const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& ro
     const int dc = dim_class_of(dim);
     for (auto it = g_plans.begin(); it != g_plans.end(); ++it) {
         if (it->part_ptr == part_ptr.data_ptr() && it->col == col.data_ptr() && it->rows == rows.data_ptr() &&
-            it->num_parts == num_parts && it->dim_class == dc &&
+            it->num_parts == num_parts && it->num_nodes == num_nodes && it->dim_class == dc &&
             it->version_part == static_cast<int64_t>(part_ptr._version()) &&
             it->version_col == static_cast<int64_t>(col._version()) &&
             it->version_rows == static_cast<int64_t>(rows._version())) {
@@ -120,7 +121,7 @@ const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& ro
         }
     }
     if (num_slots < 0) num_slots = part_ptr[num_parts].item<int64_t>();   // slots the groups cover (one 4-byte read)
-    PlanEntry e{part_ptr.data_ptr(), col.data_ptr(), rows.data_ptr(), num_parts,
+    PlanEntry e{part_ptr.data_ptr(), col.data_ptr(), rows.data_ptr(), num_parts, num_nodes,
                 static_cast<int64_t>(part_ptr._version()), static_cast<int64_t>(col._version()),
                 static_cast<int64_t>(rows._version()), dc, part_ptr, col, rows, Tensor(), nullptr};
     const size_t bytes = eppgcn_plan_bytes(num_parts, num_slots, num_nodes);
@@ -140,27 +141,52 @@ const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& ro
     return g_plans.front().plan_ptr;
 }
 
-// A heavily pruned path gathers from few distinct rows, which stay cached without a plan: plans are
-// built for paths that keep at least half of the edges.  The decision is remembered per path.
+// Per backward path, remembered from its first use:
+//   - whether it runs with a plan: a heavily pruned path gathers from few distinct rows, which stay
+//     cached without one, so plans are built for paths that keep at least half of the edges;
+//   - the bitmap of the rows it gathers, when they are fewer than half of the vertices: the
+//     pre-scaling pass of the gradient then touches those rows only.
+// An entry is valid for exactly the tensors it was made from (same storage, same version counters);
+// it holds references to them so that their memory cannot be handed to other tensors meanwhile.
 struct PathChoice {
     const void* part_ptr;
-    int64_t num_parts;
+    const void* edge_ptr;
+    int64_t num_parts, num_nodes;
+    int64_t version_part, version_edge;
     bool use_plan;
+    Tensor keep_part, keep_edge, gathered;     // gathered: undefined when the path reads most rows
 };
-std::vector<PathChoice> g_path_choices;
+std::list<PathChoice> g_path_choices;
 
-const void* backward_plan(const Tensor& part_pointer, const Tensor& edge_list, const Tensor& ids, int64_t num_parts,
-                          int num_nodes, int dim)
+const PathChoice& path_choice(const Tensor& part_pointer, const Tensor& edge_list, int64_t num_parts, int num_nodes,
+                              int64_t* valid_len_out)
 {
-    if (num_parts <= 0) return nullptr;
-    for (const auto& c : g_path_choices)
-        if (c.part_ptr == part_pointer.data_ptr() && c.num_parts == num_parts)
-            return c.use_plan ? plan_for(part_pointer, edge_list, ids, false, num_parts, -1, num_nodes, dim) : nullptr;
+    *valid_len_out = -1;
+    for (auto it = g_path_choices.begin(); it != g_path_choices.end(); ++it) {
+        if (it->part_ptr == part_pointer.data_ptr() && it->edge_ptr == edge_list.data_ptr() &&
+            it->num_parts == num_parts && it->num_nodes == num_nodes &&
+            it->version_part == static_cast<int64_t>(part_pointer._version()) &&
+            it->version_edge == static_cast<int64_t>(edge_list._version())) {
+            g_path_choices.splice(g_path_choices.begin(), g_path_choices, it);
+            return g_path_choices.front();
+        }
+    }
     const int64_t valid_len = part_pointer[num_parts].item<int64_t>();
-    const bool use = g_plan_policy > 0 || 2 * valid_len >= edge_list.numel();
-    if (g_path_choices.size() >= 64) g_path_choices.erase(g_path_choices.begin());
-    g_path_choices.push_back({part_pointer.data_ptr(), num_parts, use});
-    return use ? plan_for(part_pointer, edge_list, ids, false, num_parts, valid_len, num_nodes, dim) : nullptr;
+    *valid_len_out = valid_len;
+    TORCH_CHECK(valid_len >= 0 && valid_len <= edge_list.numel(), "partPointer[numParts] lies outside edgeList");
+    PathChoice c{part_pointer.data_ptr(), edge_list.data_ptr(), num_parts, num_nodes,
+                 static_cast<int64_t>(part_pointer._version()), static_cast<int64_t>(edge_list._version()),
+                 g_plan_policy > 0 || 2 * valid_len >= edge_list.numel(), part_pointer, edge_list, Tensor()};
+    auto bitmap = torch::empty({(static_cast<int64_t>(num_nodes) + 31) / 32 + 1}, edge_list.options());
+    int64_t distinct = 0;
+    check(eppgcn_mark_gathered_rows(i32(edge_list), valid_len, num_nodes,
+                                    reinterpret_cast<uint32_t*>(bitmap.data_ptr<int32_t>()),
+                                    bitmap.data_ptr<int32_t>() + bitmap.numel() - 1, &distinct, stream_of(edge_list)),
+          "mark_gathered_rows");
+    if (2 * distinct < num_nodes) c.gathered = bitmap;
+    g_path_choices.push_front(std::move(c));
+    if (g_path_choices.size() > 8) g_path_choices.pop_back();
+    return g_path_choices.front();
 }
 
 Tensor feature_scratch(const Tensor& feats)
@@ -326,14 +352,23 @@ std::vector<Tensor> ours_backward(Tensor d_output, Tensor X, Tensor W, Tensor id
     CHECK_COUNTS(edgeList, d_output.size(0));
     auto d_input_prime = torch::empty_like(d_output);
     auto scaled = feature_scratch(d_output);     // d_output belongs to autograd: scale into scratch
+    const int num_nodes = static_cast<int>(d_output.size(0));
+    const void* plan = nullptr;
+    const uint32_t* gathered = nullptr;
+    if (numParts > 0) {
+        int64_t valid_len = -1;
+        const PathChoice& choice = path_choice(partPointer, edgeList, numParts, num_nodes, &valid_len);
+        if (choice.gathered.defined())
+            gathered = reinterpret_cast<const uint32_t*>(choice.gathered.data_ptr<int32_t>());
+        if (choice.use_plan)
+            plan = plan_for(partPointer, edgeList, id, false, numParts, valid_len, num_nodes,
+                            static_cast<int>(d_output.size(1)));
+    }
     check(eppgcn_ours_backward(d_input_prime.data_ptr<float>(), f32(d_output), i32(id), i32(partPointer),
                                i32(edgeList), f32(degrees), static_cast<int>(d_output.size(0)),
                                static_cast<int>(d_output.size(1)), numParts, partSize > 0 ? partSize : 1, layer, blockx,
                                blocky, scaled.numel() ? scaled.data_ptr<float>() : nullptr,
-                               static_cast<size_t>(scaled.numel()),
-                               backward_plan(partPointer, edgeList, id, numParts, static_cast<int>(d_output.size(0)),
-                                             static_cast<int>(d_output.size(1))),
-                               stream_of(d_output)),
+                               static_cast<size_t>(scaled.numel()), plan, gathered, stream_of(d_output)),
           "ours_backward");
     return dense_backward(d_input_prime, X, W, need_dx, relu_input);
 }

@@ -355,6 +355,25 @@ __global__ __launch_bounds__(256) void count_nonzero_kernel(const int* __restric
     if ((threadIdx.x & (kWave - 1)) == 0 && local) atomicAdd(d_count, local);
 }
 
+// bitmap bit c is set for every c = list[i], i < length; *d_count receives the number of distinct values.
+// A bit that already reads as set is not touched again, so the atomics are about one per distinct value
+// and wave, not one per entry.
+__global__ __launch_bounds__(256) void mark_listed_rows_kernel(const int* __restrict__ list, long long length,
+                                                               uint32_t* __restrict__ bitmap, int* __restrict__ d_count)
+{
+    int fresh = 0;
+    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+    for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < length; i += stride) {
+        const unsigned c = static_cast<unsigned>(list[i]);
+        const uint32_t bit = 1u << (c & 31);
+        if ((__builtin_nontemporal_load(bitmap + (c >> 5)) & bit) == 0)
+            fresh += (atomicOr(bitmap + (c >> 5), bit) & bit) == 0;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) fresh += __shfl_xor(fresh, off, kWave);
+    if ((threadIdx.x & (kWave - 1)) == 0 && fresh) atomicAdd(d_count, fresh);
+}
+
 // Degree histogram of get_ginfo (EPPGCN/GCNConv/EPPGCN.cpp:356-377): hist[0] = #(deg != 0),
 // hist[3..9] = the seven buckets, the last one also taking deg <= 0 and deg >= 160.
 __global__ __launch_bounds__(256) void ginfo_hist_kernel(const int* __restrict__ node_deg, int length, int* __restrict__ hist)
@@ -760,6 +779,20 @@ int launch_count_nonzero(const int* in, long long length, int* d_count, hipStrea
     if (blocks > 1024) blocks = 1024;
     hipLaunchKernelGGL(count_nonzero_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, in,
                        static_cast<int>(length), d_count);
+    EPPGCN_HIP(hipGetLastError());
+    return kOk;
+}
+
+int launch_mark_listed_rows(const int* list, long long length, long long num_rows, uint32_t* bitmap, int* d_count,
+                            hipStream_t stream)
+{
+    if (int rc = launch_zero_words(bitmap, static_cast<size_t>((num_rows + 31) / 32), stream)) return rc;
+    if (int rc = launch_zero_words(d_count, 1, stream)) return rc;
+    if (length == 0) return kOk;
+    long long blocks = (length + 1023) / 1024;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(mark_listed_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, list, length,
+                       bitmap, d_count);
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }

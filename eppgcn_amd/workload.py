@@ -28,6 +28,7 @@ class BackwardPath:
     valid_len: int
     valid_node: int
     plan: object = None      # column-blocked execution plan of this path (speed only)
+    gathered_rows: torch.Tensor = None   # bitmap of the rows the path gathers, when fewer than half (speed only)
 
 
 @dataclasses.dataclass
@@ -105,8 +106,10 @@ def prepare(graph: graphs.Graph, num_layers: int = 2, train_ratio: float = 0.1, 
         # a heavily pruned path gathers from few distinct rows, which stay cached without a plan
         path_plan = (capi.build_plan(part_pointer, edge_list, num_parts, valid_len, n, width, ids=ids)
                      if plan and num_parts > 0 and 2 * valid_len >= e else None)
+        # the pre-scaling pass of the gradient only has to cover the rows the path reads
+        bitmap, distinct = capi.mark_gathered_rows(edge_list, valid_len, n)
         paths.append(BackwardPath(k + 1, ids, edge_list, part_pointer, node_degs[k], bps, num_parts,
-                                  valid_len, valid_node, path_plan))
+                                  valid_len, valid_node, path_plan, bitmap if 2 * distinct < n else None))
     # one plan of the forward groups serves every width (the column block is sized for the widest)
     plans = {}
     if plan and part2node.numel() > 0:

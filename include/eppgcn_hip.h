@@ -131,11 +131,23 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
  * part_pointer holds num_parts+1 entries.  Stands in for ours_backward_cuda minus
  * its two torch::mm (EPPGCN_kernel.cu:547-624; kernel :626-670; bound as
  * GNNA.ours_backward, EPPGCN.cpp:157-184,393).  `layer` (1-based) only selects the
- * per-layer timer; blockx/blocky are the caller's hints and must be positive. */
+ * per-layer timer; blockx/blocky are the caller's hints and must be positive.
+ * gathered_rows: NULL, or the bitmap eppgcn_mark_gathered_rows made of this edge_list; the
+ * pre-scaling pass into the workspace then skips the rows of d_output that no group reads (with a
+ * 10 % train mask the last layer's path reads a tenth of the rows), which changes no result; with
+ * the workspace aliasing d_output, only those rows of d_output are overwritten with scaled values. */
 int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids,
                          const int32_t* part_pointer, const int32_t* edge_list, const float* degrees,
                          int num_nodes, int dim, int num_parts, int part_size, int layer,
-                         int blockx, int blocky, float* workspace, size_t workspace_floats, const void* plan, void* stream);
+                         int blockx, int blocky, float* workspace, size_t workspace_floats, const void* plan,
+                         const uint32_t* gathered_rows, void* stream);
+
+/* bitmap[(num_nodes + 31) / 32]: bit c is set for every vertex c that occurs in
+ * edge_list[0 .. valid_len) (the rows a pruned backward over this path gathers); *d_count (device)
+ * and, if not NULL, *h_count (host; synchronises the stream) receive the number of such vertices.
+ * Built once per path, next to the path itself.  No counterpart in the reference. */
+int eppgcn_mark_gathered_rows(const int32_t* edge_list, int64_t valid_len, int num_nodes, uint32_t* bitmap,
+                              int32_t* d_count, int64_t* h_count, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Execution-path preparation.

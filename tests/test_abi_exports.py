@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared_functions():
         assert hasattr(lib, name), f"{name} is declared in include/eppgcn_hip.h but not exported"
     assert sorted(capi.EXPORTS) == declared_functions()
-    assert capi.load().eppgcn_abi_version() == 6
+    assert capi.load().eppgcn_abi_version() == 7
 
 
 def test_host_only_heuristics_match_the_checker():

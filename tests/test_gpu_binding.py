@@ -85,6 +85,35 @@ def test_forward_and_both_backwards_with_dense_products(GNNA):
     assert np.linalg.norm(dx2.cpu().numpy() - want_dx) / np.linalg.norm(want_dx) < 1e-5
     assert np.linalg.norm(dw2.cpu().numpy() - want_dw) / np.linalg.norm(want_dw) < 1e-5
 
+    # the module remembers per path which rows it gathers (a fifth of them here) and pre-scales only
+    # those: a second gradient through the same path, and garbage in the rows the path never reads
+    dy_b = (rng.standard_normal((n, 16)) * src[:, None]).astype(np.float32)
+    g64_b = cf.aggregate_csr64(indptr, col, s, dy_b)
+    noisy = dy_b.copy()
+    never_read = np.ones(n, bool)
+    never_read[col[src[col]]] = False
+    noisy[never_read] = 1e30
+    dx3, dw3 = GNNA.ours_backward(dev(noisy), dev(x), dev(w), ids, part_pointer, edge_list, dev(s), ps, want_p, 1, 4, 16)
+    assert np.linalg.norm(dx3.cpu().numpy() - g64_b @ w.T.astype(np.float64)) / np.linalg.norm(g64_b @ w.T) < 1e-5
+    assert np.linalg.norm(dw3.cpu().numpy() - x.T.astype(np.float64) @ g64_b) / np.linalg.norm(x.T @ g64_b) < 1e-5
+    # a path rewritten in place (same storage) is a different path: nothing remembered may be reused
+    src_c = rng.random(n) < 0.25
+    bem.fill_(-1); degs.zero_()
+    GNNA.mask_forward(dev(p2n), dev(pp), dev(col), dev(src_c), torch.zeros(0, dtype=torch.bool, device="cuda"),
+                      bem, degs, 2, 2, 4, 16)
+    ids_c, edge_c, info_c = GNNA.compact_back_edge(bem, dev(col))
+    pp_c, pinfo_c = GNNA.split_back_part(degs, e, ps)
+    ids.copy_(ids_c); edge_list.copy_(edge_c); part_pointer.copy_(pp_c)
+    dy_c = (rng.standard_normal((n, 16)) * src_c[:, None]).astype(np.float32)
+    g64_c = cf.aggregate_csr64(indptr, col, s, dy_c)
+    dx4, dw4 = GNNA.ours_backward(dev(dy_c), dev(x), dev(w), ids, part_pointer, edge_list, dev(s), ps,
+                                  int(pinfo_c[0].item()), 1, 4, 16)
+    assert np.linalg.norm(dx4.cpu().numpy() - g64_c @ w.T.astype(np.float64)) / np.linalg.norm(g64_c @ w.T) < 1e-5
+    bem.fill_(-1); degs.zero_()
+    GNNA.mask_forward(dev(p2n), dev(pp), dev(col), dev(src), torch.zeros(0, dtype=torch.bool, device="cuda"),
+                      bem, degs, 2, 2, 4, 16)
+    ids, edge_list, info = GNNA.compact_back_edge(bem, dev(col))
+
     # legacy all-in-one call: same lists, threshold group size
     ids3, el3, pp3, info3 = GNNA.build_back_part(bem, dev(col), degs, 0, 16)
     ps3 = cf.threshold_back_part_size(cf.compact_count(degs.cpu().numpy()), v)

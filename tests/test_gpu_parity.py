@@ -424,6 +424,49 @@ def test_pruned_backward_vs_checker_and_unpruned(api, name, dim, ratio):
         assert_close(got2, want, bound, "noise outside the mask")
 
 
+@pytest.mark.parametrize("name", ["tiny", "isolated", "hub", "medium"])
+@pytest.mark.parametrize("ratio", [0.0, 0.02, 0.3, 1.0])
+def test_gathered_rows_bitmap_and_restricted_prescaling(api, name, ratio):
+    """The bitmap of the rows a path gathers is exactly the set of its column ids; with it the
+    pre-scaling pass leaves every other row of the workspace alone (here: NaN, as are the gradient
+    rows outside the set), and the result is the same as without it."""
+    indptr, col = GRAPHS[name]()
+    n = indptr.size - 1
+    rng = np.random.default_rng(int(ratio * 100) + n)
+    src = rng.random(n) < ratio
+    s = scale_inv_sqrt(indptr)
+    oid, oedge, bpp, p = _gpu_path(api, indptr, col, src, 5, 8)
+    v = int(src[col].sum())
+    bitmap, distinct = api.mark_gathered_rows(oedge, v, n)
+    want_rows = np.zeros(n, bool)
+    want_rows[col[src[col]]] = True
+    words = bitmap.cpu().numpy().view(np.uint32)
+    got_rows = ((words[np.arange(n) >> 5] >> (np.arange(n) & 31).astype(np.uint32)) & 1).astype(bool)
+    assert np.array_equal(got_rows, want_rows) and distinct == int(want_rows.sum())
+    assert words.size == (n + 31) // 32 and (n % 32 == 0 or words[-1] >> (n % 32) == 0)
+    if p == 0:
+        return
+    for dim in (16, 22, 7, 40):
+        dy = (rng.standard_normal((n, dim)) * src[:, None]).astype(np.float32)
+        want = co.spmm_f64(dy, indptr, col, s)
+        bound = cf.abs_sum_bound(indptr, col, s, dy)
+        poisoned = dy.copy()
+        poisoned[~want_rows] = np.nan
+        for alias in (False, True):
+            d_in = dev(poisoned)
+            ws = d_in if alias else torch.full((n * api.feature_workspace_pitch(dim),), float("nan"), device="cuda")
+            got = api.ours_backward(d_in, oid, bpp, oedge, dev(s), p, part_size=8, workspace=ws,
+                                    gathered_rows=bitmap)
+            assert_close(got.cpu().numpy(), want, bound, f"{name} r={ratio} D={dim} alias={alias}")
+            if not alias:     # rows outside the set were not written
+                pitch = api.feature_workspace_pitch(dim)
+                assert torch.isnan(ws.view(n, pitch)[dev(~want_rows)]).all()
+        plan = api.build_plan(bpp, oedge, p, v, n, dim, ids=oid)
+        got = api.ours_backward(dev(poisoned), oid, bpp, oedge, dev(s), p, part_size=8, plan=plan,
+                                gathered_rows=bitmap, out=torch.full((n, dim), float("nan"), device="cuda"))
+        assert_close(got.cpu().numpy(), want, bound, f"{name} r={ratio} D={dim} planned")
+
+
 def test_two_layer_mask_chain_on_gpu(api):
     """The wiring of the reference's driver for 2 layers (EPPGCN/gcn_main.py:130-139)."""
     indptr, col = GRAPHS["medium"]()
