@@ -25,7 +25,7 @@ EXPORTS = [
     "eppgcn_feature_workspace_pitch", "eppgcn_update_forward", "eppgcn_update_backward_input",
     "eppgcn_update_workspace_bytes", "eppgcn_update_backward_weight", "eppgcn_update_supported",
     "eppgcn_mark_compact_workspace_bytes", "eppgcn_mark_compact", "eppgcn_set_plan_length_classes",
-    "eppgcn_mark_gathered_rows",
+    "eppgcn_mark_gathered_rows", "eppgcn_set_wide_index",
 ]
 
 _lib = None
@@ -84,6 +84,8 @@ def load():
     lib.eppgcn_set_team_size.restype = None
     lib.eppgcn_set_rounds.argtypes = [i]
     lib.eppgcn_set_rounds.restype = None
+    lib.eppgcn_set_wide_index.argtypes = [i]
+    lib.eppgcn_set_wide_index.restype = None
     lib.eppgcn_set_plan_shift.argtypes = [i]
     lib.eppgcn_set_plan_shift.restype = None
     lib.eppgcn_set_plan_length_classes.argtypes = [i]
@@ -511,6 +513,11 @@ def set_team_size(lanes: int):
 
 def set_rounds(rounds: int):
     load().eppgcn_set_rounds(int(rounds))
+
+
+def set_wide_index(on: bool):
+    """Forces the 64-bit instantiations of the clear and pre-scaling kernels (for tests)."""
+    load().eppgcn_set_wide_index(int(bool(on)))
 
 
 def set_plan_length_classes(on: bool):

@@ -645,7 +645,7 @@ static int launch_scale_rows(float* dst, const float* src, const float* scale, c
 {
     if (static_cast<long long>(num_nodes) * dim == 0) return kOk;
     const long long elems = static_cast<long long>(num_nodes) * (ld_dst > dim ? ld_dst : dim);
-    if (elems < (1ll << 32)) launch_scale_rows_typed<unsigned>(dst, src, scale, rows, num_nodes, dim, ld_dst, stream);
+    if (elems < (1ll << 32) && !force_wide_index()) launch_scale_rows_typed<unsigned>(dst, src, scale, rows, num_nodes, dim, ld_dst, stream);
     else launch_scale_rows_typed<unsigned long long>(dst, src, scale, rows, num_nodes, dim, ld_dst, stream);
     EPPGCN_HIP(hipGetLastError());
     return kOk;

@@ -411,6 +411,7 @@ double eppgcn_get_time_ms(int which)
 
 void eppgcn_set_team_size(int lanes) { set_agg_force_team(lanes); }
 void eppgcn_set_rounds(int rounds) { set_agg_force_rounds(rounds); }
+void eppgcn_set_wide_index(int on) { set_force_wide_index(on != 0); }
 void eppgcn_set_plan_shift(int shift) { set_schedule_shift(shift); }
 void eppgcn_set_plan_keep_rows(int groups) { set_plan_keep_rows(groups); }
 void eppgcn_set_plan_length_classes(int on) { set_plan_length_classes(on); }

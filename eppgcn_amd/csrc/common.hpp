@@ -44,6 +44,10 @@ int hip_fail(hipError_t e, const char* what);
 // hipMemsetAsync everywhere so that every call of the library can be captured into a HIP graph
 // (memset nodes are the one node kind callers are told to avoid on this platform).
 int launch_zero_words(void* p, size_t words, hipStream_t stream);
+// The streaming helper kernels index with 32 bits when the element count allows; true forces their
+// 64-bit instantiations at any size (so that tests reach them without 16 GB matrices).
+bool force_wide_index();
+void set_force_wide_index(bool on);
 // Zeroes the rows of out[num_rows, dim] whose bit in `skip` is clear (rows with a set bit are left as they are).
 int launch_zero_rows_unless(float* out, const uint32_t* skip, long long num_rows, int dim, hipStream_t stream);
 

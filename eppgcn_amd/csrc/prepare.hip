@@ -639,10 +639,14 @@ static void launch_zero_rows_typed(float* out, const uint32_t* skip, long long n
     else hipLaunchKernelGGL((zero_rows_unless_kernel<1, Index>), grid, block, 0, stream, out, skip, t, v);
 }
 
+static bool g_force_wide_index = false;
+bool force_wide_index() { return g_force_wide_index; }
+void set_force_wide_index(bool on) { g_force_wide_index = on; }
+
 int launch_zero_rows_unless(float* out, const uint32_t* skip, long long num_rows, int dim, hipStream_t stream)
 {
     if (num_rows <= 0 || dim <= 0) return kOk;
-    if (num_rows * dim < (1ll << 32)) launch_zero_rows_typed<unsigned>(out, skip, num_rows, dim, stream);
+    if (num_rows * dim < (1ll << 32) && !force_wide_index()) launch_zero_rows_typed<unsigned>(out, skip, num_rows, dim, stream);
     else launch_zero_rows_typed<unsigned long long>(out, skip, num_rows, dim, stream);
     EPPGCN_HIP(hipGetLastError());
     return kOk;

@@ -292,6 +292,9 @@ void eppgcn_set_team_size(int lanes);
 /* Forces the number of consecutive group rounds one wave processes (0 = choose from
  * the group size so that a wave gathers about 512 rows).  For tuning runs. */
 void eppgcn_set_rounds(int rounds);
+/* The output-clear and pre-scaling kernels index with 32 bits while the matrices have fewer than 2^32
+ * elements; 1 forces their 64-bit instantiations at any size.  For tests. */
+void eppgcn_set_wide_index(int on);
 /* Forces the column block size of eppgcn_build_plan to 2^shift vertices (0 = choose from the
  * feature width).  For tuning runs. */
 void eppgcn_set_plan_shift(int shift);

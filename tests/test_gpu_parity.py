@@ -788,6 +788,50 @@ def test_aggregation_with_misaligned_feature_buffers(api, dim, shift_in, shift_o
         assert_close(out.cpu().numpy(), want_b, bound, f"pruned backward, workspace={workspace}")
 
 
+@pytest.mark.parametrize("dim", [16, 22, 7, 3])
+def test_wide_index_instantiations_of_the_streaming_kernels(api, dim):
+    """The clear and pre-scaling kernels have a 32-bit and a 64-bit index instantiation; the
+    second is only chosen by itself for matrices of 2^32 elements and more, so it is forced here:
+    padded, flat and aliased pre-scaling, restricted to gathered rows or not, full and selective
+    clear must give the results of the default instantiation bit for bit."""
+    indptr, col = GRAPHS["medium"]()
+    n = indptr.size - 1
+    rng = np.random.default_rng(dim)
+    s = scale_inv_sqrt(indptr)
+    x = rng.standard_normal((n, dim)).astype(np.float32)
+    src = rng.random(n) < 0.2
+    pp, p2n = co.build_part(6, indptr)
+    oid, oedge, bpp, p = _gpu_path(api, indptr, col, src, 6, 8)
+    bitmap, _ = api.mark_gathered_rows(oedge, int(src[col].sum()), n)
+    plan = api.build_plan(dev(pp), dev(col), p2n.size, col.size, n, dim, part2node=dev(p2n))
+    dy = (x * src[:, None]).astype(np.float32)
+
+    def run_all():
+        nan = lambda: torch.full((n, dim), float("nan"), device="cuda")
+        res = [api.spmm_forward(dev(x), dev(col), dev(s), dev(pp), dev(p2n), part_size=6, out=nan()),
+               api.spmm_forward(dev(x), dev(col), dev(s), dev(pp), dev(p2n), part_size=6, plan=plan, out=nan())]
+        alias = dev(x)
+        res.append(api.spmm_forward(alias, dev(col), dev(s), dev(pp), dev(p2n), part_size=6, workspace=alias, out=nan()))
+        res.append(api.ours_backward(dev(dy), oid, bpp, oedge, dev(s), p, part_size=8, gathered_rows=bitmap, out=nan()))
+        alias = dev(dy)
+        res.append(api.ours_backward(alias, oid, bpp, oedge, dev(s), p, part_size=8, workspace=alias,
+                                     gathered_rows=bitmap, out=nan()))
+        return [r.cpu().numpy() for r in res]
+
+    narrow = run_all()
+    api.set_wide_index(True)
+    try:
+        wide = run_all()
+    finally:
+        api.set_wide_index(False)
+    want = co.spmm_f64(x, indptr, col, s)
+    assert_close(narrow[1], want, cf.abs_sum_bound(indptr, col, s, x), "planned forward")
+    for k, (a, b) in enumerate(zip(narrow, wide)):
+        # float atomics make the order of a row's partial sums vary between runs: compare to rounding
+        assert np.allclose(a, b, rtol=1e-5, atol=1e-6), f"case {k}"
+        assert not np.isnan(b).any()
+
+
 def test_element_offsets_beyond_int32(api):
     """[N, 256] matrices of more than 2^31 elements (8.6 GB each): every row offset has to be
     formed in 64 bits.  Ring graph with self-loops, unit scale, small integer features, so the
