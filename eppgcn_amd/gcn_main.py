@@ -6,7 +6,9 @@ eppgcn_amd.gcn_main``.
 
 Differences, all deliberate:
   * ``--backsize_mode net`` needs the reference's unpublished predictor weights
-    (EPPGCN/net_pred.py:63) and is refused with a message; the default here is ``map``.
+    (EPPGCN/net_pred.py:63) and is refused with a message; the default here is ``constant``, and
+    ``--backsize 0`` (the default) then means 32, the group size the wave64 kernels were tuned to
+    (the fitted regression of ``map`` was made for small graphs and drops below 1 on large ones).
   * ``--dataset`` also accepts a synthetic graph name (``cfg1_uniform``, ``rmat:<scale>:<factor>``
     ...) when no graph file is given; the train mask is then drawn instead of read.
   * the device is the current one (the reference hard-codes device 1, gcn_main.py:69).
@@ -47,8 +49,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--loadFromTxt", default="True", help="True: <dataset>_snap edge list, False: <dataset>.npz", **tf)
     ap.add_argument("--single_spmm", default="False", help="time the forward aggregation alone", **tf)
     ap.add_argument("--verify_spmm", default="False", help="check one forward aggregation against torch", **tf)
-    ap.add_argument("--backsize", type=int, default=0, help="backward group size of all layers (constant mode)")
-    ap.add_argument("--backsize_mode", type=str, default="map", choices=["map", "net", "constant"])
+    ap.add_argument("--backsize", type=int, default=0, help="backward group size of all layers (constant mode; 0 = 32)")
+    ap.add_argument("--backsize_mode", type=str, default="constant", choices=["map", "net", "constant"])
     ap.add_argument("--degree_norm", type=str, default="sqrt", choices=["sqrt", "inv_sqrt"],
                     help="scale vector: sqrt(deg) as the reference's loader fills it, or deg^-1/2 (symmetric GCN norm)")
     ap.add_argument("--kernel_timers", default="True", **tf,
@@ -117,7 +119,7 @@ def main(argv=None) -> int:
     device = torch.device("cuda", torch.cuda.current_device())
     ds = load_dataset(args, device)
     verbose = args.verbose_mode == "True"
-    tr = train.Trainer(None, hidden=args.hidden, backsize_mode=args.backsize_mode, backsize=args.backsize,
+    tr = train.Trainer(None, hidden=args.hidden, backsize_mode=args.backsize_mode, backsize=args.backsize or 32,
                        dataset=ds, part_size=args.partSize, dim_worker=args.dimWorker,
                        warp_per_block=args.warpPerBlock, shared_mem=args.sharedMem,
                        manual_mode=args.manual_mode == "True", verbose=verbose, weight_seed=None)

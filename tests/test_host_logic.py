@@ -118,6 +118,7 @@ def test_driver_command_line_takes_the_reference_flags(capsys):
     assert (d.dim, d.hidden, d.classes, d.layers, d.train_ratio, d.num_epoches, d.partSize, d.dimWorker,
             d.warpPerBlock, d.sharedMem, d.manual_mode, d.loadFromTxt, d.backsize) == \
         (96, 16, 22, 2, 0.1, 100, 32, 32, 8, 100, "False", "True", 0)
+    assert d.backsize_mode == "constant"
     assert gcn_main.main(["--backsize_mode", "net"]) == 2
     out = capsys.readouterr()
     assert out.out.startswith("||amazon0601   0.1   2") and "net" in out.err
