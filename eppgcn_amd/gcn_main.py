@@ -14,6 +14,8 @@ Differences, all deliberate:
   * the device is the current one (the reference hard-codes device 1, gcn_main.py:69).
   * ``--degree_norm inv_sqrt`` (an addition) fills the scale vector with deg^-1/2 instead of the
     reference loader's sqrt(deg) (EPPGCN/dataset.py:117-119).
+  * ``--kernel_timers`` and ``--hip_graph`` (additions) switch the per-op device timers off and
+    replay the epoch from a HIP graph.
   * ``--model gin`` is accepted by the reference's parser but never read by it; here too.
   * ``--single_spmm`` / ``--verify_spmm`` are parsed and never read by the reference; here
     ``--single_spmm True`` times the forward aggregation alone and ``--verify_spmm True``
@@ -56,6 +58,9 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--kernel_timers", default="True", **tf,
                     help="True: per-op device timers for the print_time report, as the reference always has; "
                          "False: none (the epochs are then issued without a host wait per op)")
+    ap.add_argument("--hip_graph", default="False", **tf,
+                    help="True: record one epoch into a HIP graph after the warm-up and replay it (pays off on "
+                         "small graphs, where launches dominate); only the total time is then reported")
     return ap
 
 
@@ -127,6 +132,13 @@ def main(argv=None) -> int:
         print(tr.model)
     if args.single_spmm == "True" or args.verify_spmm == "True":
         return 0 if _single_spmm(tr, args.num_epoches, args.verify_spmm == "True") else 1
+    if args.hip_graph == "True":
+        tr.run(0, warmup=10)
+        res = tr.run_graphed(args.num_epoches)
+        print("build_time: {:.6f}".format(tr.build_time))
+        print("Time: {:.6f}".format(res["Time"]))
+        print()
+        return 0
     res = tr.run(args.num_epoches, warmup=10, kernel_timing=args.kernel_timers == "True")
     tr.GNNA.print_time()
     for key in ("for_time", "loss_time", "back_time", "build_time"):

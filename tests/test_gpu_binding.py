@@ -337,6 +337,9 @@ def test_driver_command_line_end_to_end(GNNA, tmp_path, capsys):
         for key in ("for_time:", "loss_time:", "back_time:", "build_time:", "Time:"):
             assert sum(line.startswith(key) for line in out.splitlines()) == 1, (key, out)
         assert out.startswith("||toy   0.3   ")
+    assert gcn_main.main(common + ["--hip_graph", "True"]) == 0
+    out = capsys.readouterr().out
+    assert "Time:" in out and "for_time" not in out
     assert gcn_main.main(common + ["--verify_spmm", "True"]) == 0
     assert "PASS" in capsys.readouterr().out
     assert gcn_main.main(["--dataset", "cfg1_uniform", "--num_epoches", "2", "--degree_norm", "inv_sqrt",
