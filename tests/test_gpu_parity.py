@@ -620,10 +620,14 @@ def test_aggregation_calls_replay_from_a_hip_graph(api):
     x = torch.zeros((n, 22), device="cuda")
     y_fwd, y_bwd = torch.empty_like(x), torch.empty_like(x)
     ws = api.feature_workspace(n, 22, "cuda")
+    # with a plan (selective output clear) and the gathered-rows bitmap (restricted pre-scaling)
+    plan = api.build_plan(pp, d_col, p2n.numel(), col.size, n, 22, part2node=p2n)
+    bitmap, _ = api.mark_gathered_rows(edge_list, v, n)
 
     def both():
-        api.spmm_forward(x, d_col, d_s, pp, p2n, 8, out=y_fwd, workspace=ws)
-        api.ours_backward(x, ids, part_pointer, edge_list, d_s, num_parts, 8, out=y_bwd, workspace=ws)
+        api.spmm_forward(x, d_col, d_s, pp, p2n, 8, out=y_fwd, workspace=ws, plan=plan)
+        api.ours_backward(x, ids, part_pointer, edge_list, d_s, num_parts, 8, out=y_bwd, workspace=ws,
+                          gathered_rows=bitmap)
 
     both()                                    # warm-up outside the capture
     torch.cuda.synchronize()
