@@ -889,3 +889,65 @@ def test_element_offsets_beyond_int32(api):
     del dx
     dw = api.update_backward_weight(x, g)
     assert torch.equal(dw, x[tail].t() @ g[tail])
+
+
+# ----------------------------------------------------------------------------- ragged random inputs
+def test_ragged_random_graphs_whole_path(api):
+    """Property-based: randomly drawn ragged graphs (empty rows, rows of several groups, no
+    edges at all), any mask density, group sizes from 1: every integer result of the device
+    path equals the closed forms bit for bit, both ways of preparing the path agree, and the
+    aggregations (plain, planned, pruned with the gathered-rows bitmap) stay within tolerance."""
+    from hypothesis import HealthCheck, given, settings
+    from hypothesis import strategies as st
+    from tests.test_oracle_fuzz import ragged_graph
+
+    @settings(max_examples=150, deadline=None, derandomize=True, database=None,
+              suppress_health_check=list(HealthCheck))
+    @given(ragged_graph(), st.integers(1, 9), st.integers(1, 9), st.sampled_from([0.0, 0.1, 0.5, 1.0]),
+           st.sampled_from([1, 3, 4, 16, 22]))
+    def check(graph, ps_fwd, ps_back, ratio, dim):
+        indptr, col, rng = graph
+        n, e = indptr.size - 1, col.size
+        d_col = dev(col) if e else torch.zeros(0, dtype=torch.int32, device="cuda")
+        pp, p2n = api.build_part(ps_fwd, dev(indptr), e)
+        w_pp, w_p2n = cf.build_part(ps_fwd, indptr)
+        assert np.array_equal(pp.cpu().numpy(), w_pp) and np.array_equal(p2n.cpu().numpy(), w_p2n)
+        src = rng.random(n) < ratio
+        w_id, w_edge, w_bpp, w_v, w_p, w_degs = cf.pruned_path(indptr, col, src, ps_back)
+        # marking then compaction
+        bem = torch.full((e,), -1, dtype=torch.int32, device="cuda")
+        degs = torch.zeros(n, dtype=torch.int32, device="cuda")
+        if p2n.numel():
+            api.mask_forward(p2n, pp, d_col, dev(src), None, bem, degs, True)
+        oid, oedge, v = api.compact_back_edge(bem, d_col)
+        assert v == w_v and np.array_equal(degs.cpu().numpy(), w_degs)
+        assert np.array_equal(oid.cpu().numpy(), w_id) and np.array_equal(oedge.cpu().numpy(), w_edge)
+        # the fused pass
+        if p2n.numel():
+            degs2 = torch.zeros(n, dtype=torch.int32, device="cuda")
+            fid, fedge, fv = api.mark_compact(p2n, pp, d_col, dev(src), None, degs2, True)
+            assert fv == w_v and torch.equal(degs2, degs)
+            assert np.array_equal(fid.cpu().numpy()[:w_v], w_id[:w_v])
+            assert np.array_equal(fedge.cpu().numpy()[:w_v], w_edge[:w_v])
+        bpp, p, v2 = api.split_back_part(degs, e, ps_back)
+        assert (p, v2) == (w_p, w_v) and np.array_equal(bpp.cpu().numpy(), w_bpp)
+        # aggregation
+        s = rng.uniform(0.2, 1.5, n).astype(np.float32)
+        x = rng.standard_normal((n, dim)).astype(np.float32)
+        want = co.spmm_f64(x, indptr, col, s)
+        bound = cf.abs_sum_bound(indptr, col, s, x) if e else np.zeros((n, dim))
+        nan = lambda: torch.full((n, dim), float("nan"), device="cuda")
+        got = api.spmm_forward(dev(x), d_col, dev(s), pp, p2n, part_size=ps_fwd, out=nan())
+        assert_close(got.cpu().numpy(), want, bound, "forward")
+        if p2n.numel():
+            plan = api.build_plan(pp, d_col, p2n.numel(), e, n, dim, part2node=p2n)
+            got = api.spmm_forward(dev(x), d_col, dev(s), pp, p2n, part_size=ps_fwd, plan=plan, out=nan())
+            assert_close(got.cpu().numpy(), want, bound, "planned forward")
+        dy = (x * src[:, None]).astype(np.float32)
+        want_b = co.spmm_f64(dy, indptr, col, s)
+        bitmap, _ = api.mark_gathered_rows(oedge, v, n)
+        got_b = api.ours_backward(dev(dy), oid, bpp, oedge, dev(s), p, part_size=ps_back, gathered_rows=bitmap,
+                                  out=nan())
+        assert_close(got_b.cpu().numpy(), want_b, bound, "pruned backward")
+
+    check()

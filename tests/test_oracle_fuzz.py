@@ -26,7 +26,8 @@ def ragged_graph(draw):
     return indptr, col, rng
 
 
-COMMON = dict(max_examples=150, deadline=None, suppress_health_check=[HealthCheck.too_slow])
+COMMON = dict(max_examples=200, deadline=None, derandomize=True, database=None,
+              suppress_health_check=[HealthCheck.too_slow])
 
 
 @settings(**COMMON)
