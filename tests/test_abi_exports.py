@@ -80,3 +80,37 @@ def test_argument_errors_are_reported_before_any_device_work():
     assert lib.eppgcn_feature_workspace_pitch(3) == 4 and lib.eppgcn_feature_workspace_pitch(40) == 40
     assert lib.eppgcn_update_workspace_bytes(0, 4, 4) == 0
     assert lib.eppgcn_mark_compact_workspace_bytes(4096 * 3 + 1) >= 32 + 8 * 4 + 4 * 5
+
+
+def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 and as C++ without torch or HIP
+    headers, and a C program must link against the library and call it.  Only host-side entry
+    points are called here (no GPU)."""
+    import subprocess
+    from eppgcn_amd import capi
+    inc = os.path.join(ROOT, "include")
+    src = tmp_path / "client.c"
+    src.write_text(
+        '#include "eppgcn_hip.h"\n'
+        "#include <stdio.h>\n"
+        "int main(void) {\n"
+        "    int clamped = 0;\n"
+        "    int ps = eppgcn_map_back_part_size(1000, 5000, &clamped);\n"
+        '    printf("%d %d %zu %d %d %d\\n", eppgcn_abi_version(), eppgcn_feature_workspace_pitch(22),\n'
+        "           eppgcn_feature_workspace_floats(10, 22), ps, clamped,\n"
+        "           eppgcn_spmm_forward(0, 0, 0, 0, 0, 0, 0, 4, 0, 0, 1, 1, 1, 0, 0, 0, 0));\n"
+        '    printf("%s\\n", eppgcn_last_error());\n'
+        "    return 0;\n"
+        "}\n")
+    for compiler, std in (("gcc", "-std=c99"), ("g++", "-std=c++11")):
+        subprocess.run([compiler, std, "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only", "-x",
+                        "c" if compiler == "gcc" else "c++", "-I", inc, str(src)], check=True)
+    exe = tmp_path / "client"
+    libdir = os.path.dirname(capi.LIB_PATH)
+    subprocess.run(["gcc", "-std=c99", "-I", inc, str(src), "-o", str(exe), "-L", libdir, "-leppgcn_hip",
+                    "-Wl,-rpath," + libdir, "-Wl,-rpath-link,/opt/rocm/lib"], check=True)
+    env = dict(os.environ, LD_LIBRARY_PATH="/opt/rocm/lib:" + os.environ.get("LD_LIBRARY_PATH", ""))
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True, env=env).stdout.split("\n")
+    from oracle import c_oracle as co
+    assert out[0].split() == ["7", "32", "320", str(max(1, co.map_back_part_size(1000, 5000))), "0", "-1"]
+    assert "dim > 0" in out[1]
