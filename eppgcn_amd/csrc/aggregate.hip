@@ -613,6 +613,47 @@ size_t feature_workspace_floats(long long num_nodes, int dim)
     return static_cast<size_t>(num_nodes) * static_cast<size_t>(workspace_pitch(dim));
 }
 
+// Restricted form of the pass for a sparse row set: a wave looks at 64 rows at a time, collects those
+// whose bit is set and scales them one 16-byte vector per lane, so the cost follows the rows that are
+// gathered instead of the size of the matrix.  dst rows are ld_dst floats apart (a multiple of 4,
+// 16-byte aligned); dst may be src (then ld_dst == dim).
+__global__ __launch_bounds__(256) void scale_listed_rows_kernel(float* __restrict__ dst, const float* __restrict__ src,
+                                                                const float* __restrict__ scale,
+                                                                const uint32_t* __restrict__ rows, unsigned num_rows,
+                                                                unsigned vecs_per_row, unsigned dim, bool pairs)
+{
+    __shared__ int lists[4][kWave];
+    int* list = lists[threadIdx.x / kWave];
+    const unsigned lane = threadIdx.x & (kWave - 1);
+    const unsigned waves = gridDim.x * 4u;
+    const unsigned blocks64 = (num_rows + 63u) / 64u;
+    for (unsigned b = blockIdx.x * 4u + threadIdx.x / kWave; b < blocks64; b += waves) {
+        const unsigned r0 = b * 64u + lane;
+        const bool wanted = r0 < num_rows && ((rows[r0 >> 5] >> (r0 & 31)) & 1u) != 0;
+        const unsigned count = compact_wanted_rows(list, r0, wanted);
+        const unsigned total = count * vecs_per_row;
+        for (unsigned t = lane; t < total; t += kWave) {
+            const unsigned k = t / vecs_per_row;
+            const unsigned c0 = (t - k * vecs_per_row) * 4;
+            const size_t r = static_cast<size_t>(list[k]);
+            const float s = scale[r];
+            const float* row = src + r * dim;
+            float4 v;
+            if (pairs) {
+                const float2 lo = c0 < dim ? *reinterpret_cast<const float2*>(row + c0) : make_float2(0.f, 0.f);
+                const float2 hi = c0 + 2 < dim ? *reinterpret_cast<const float2*>(row + c0 + 2) : make_float2(0.f, 0.f);
+                v = make_float4(s * lo.x, s * lo.y, s * hi.x, s * hi.y);
+            } else {
+                v.x = c0 + 0 < dim ? s * row[c0 + 0] : 0.f;
+                v.y = c0 + 1 < dim ? s * row[c0 + 1] : 0.f;
+                v.z = c0 + 2 < dim ? s * row[c0 + 2] : 0.f;
+                v.w = c0 + 3 < dim ? s * row[c0 + 3] : 0.f;
+            }
+            *reinterpret_cast<float4*>(dst + r * (static_cast<size_t>(vecs_per_row) * 4) + c0) = v;
+        }
+    }
+}
+
 template <class Index>
 static void launch_scale_rows_typed(float* dst, const float* src, const float* scale, const uint32_t* rows,
                                     long long num_nodes, int dim, int ld_dst, hipStream_t stream)
@@ -644,6 +685,15 @@ static int launch_scale_rows(float* dst, const float* src, const float* scale, c
                              int dim, int ld_dst, hipStream_t stream)
 {
     if (static_cast<long long>(num_nodes) * dim == 0) return kOk;
+    if (rows && ld_dst % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 && !force_wide_index()) {
+        long long blocks = (static_cast<long long>(num_nodes) + 255) / 256;     // one wave per 64 rows
+        if (blocks > 256 * 16) blocks = 256 * 16;
+        hipLaunchKernelGGL(scale_listed_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, dst, src,
+                           scale, rows, static_cast<unsigned>(num_nodes), static_cast<unsigned>(ld_dst / 4),
+                           static_cast<unsigned>(dim), dim % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 8 == 0);
+        EPPGCN_HIP(hipGetLastError());
+        return kOk;
+    }
     const long long elems = static_cast<long long>(num_nodes) * (ld_dst > dim ? ld_dst : dim);
     if (elems < (1ll << 32) && !force_wide_index()) launch_scale_rows_typed<unsigned>(dst, src, scale, rows, num_nodes, dim, ld_dst, stream);
     else launch_scale_rows_typed<unsigned long long>(dst, src, scale, rows, num_nodes, dim, ld_dst, stream);

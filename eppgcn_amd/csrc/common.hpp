@@ -135,6 +135,21 @@ __device__ __forceinline__ int ballot_rank(uint64_t ballot)
                                      __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(ballot), 0u));
 }
 
+// A wave looks at 64 consecutive rows (lane l at row base + l, `wanted` says whether the row needs
+// work) and leaves the wanted rows, in order, in its own 64-entry LDS list; returns how many.  The
+// barriers order the LDS traffic of the wave's lanes (the list is private to the wave).
+__device__ __forceinline__ int compact_wanted_rows(int* __restrict__ list, unsigned row, bool wanted)
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");     // earlier reads of the list are done
+    __builtin_amdgcn_wave_barrier();
+    const uint64_t m = __ballot(wanted);
+    if (wanted) list[ballot_rank(m)] = static_cast<int>(row);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    return __popcll(m);
+}
+
 // DPP controls (GFX9 encoding): row_ror:n rotates within a row of 16 lanes.
 constexpr int kDppRowRor4 = 0x124;
 constexpr int kDppRowRor8 = 0x128;

@@ -581,62 +581,35 @@ __global__ __launch_bounds__(256) void zero_rows_unless_kernel(float* __restrict
     }
 }
 
-// The same for a 16-byte aligned matrix of rows of at least 4 floats, whatever the row length: one
-// thread per 16 bytes of the flat array.  A vector lies in one row or straddles two; it is written
-// whole when no row it touches is skipped and float by float otherwise.
-template <class Index>
-__global__ __launch_bounds__(256) void zero_flat_unless_kernel(float* __restrict__ out, const uint32_t* __restrict__ skip,
-                                                               Index total_floats, Index dim)
+// The same with the work found by whole waves: a wave looks at 64 rows at a time, collects those whose bit
+// is clear (usually few: the rows of several groups or of none) and clears them VW floats per lane, so
+// the cost follows the rows that are cleared instead of the size of the matrix.
+template <int VW>
+__global__ __launch_bounds__(256) void zero_listed_rows_kernel(float* __restrict__ out, const uint32_t* __restrict__ skip,
+                                                               unsigned num_rows, unsigned vecs_per_row)
 {
-    typedef float fvec4 __attribute__((ext_vector_type(4)));
-    const Index vecs = total_floats / 4;
-    const Index stride = static_cast<Index>(gridDim.x) * blockDim.x;
-    const Index tid = static_cast<Index>(blockIdx.x) * blockDim.x + threadIdx.x;
-    for (Index j = tid; j < vecs; j += stride) {
-        const Index f0 = 4 * j;
-        const Index r0 = f0 / dim;
-        const Index in_r0 = (r0 + 1) * dim - f0;           // floats of the vector that belong to row r0
-        const Index r1 = in_r0 < 4 ? r0 + 1 : r0;
-        const bool keep0 = ((skip[r0 >> 5] >> (r0 & 31)) & 1u) != 0;
-        const bool keep1 = ((skip[r1 >> 5] >> (r1 & 31)) & 1u) != 0;
-        if (!keep0 && !keep1) {
-            fvec4 z = {};
-            __builtin_nontemporal_store(z, reinterpret_cast<fvec4*>(out) + j);
-        } else if (keep0 != keep1) {
-#pragma unroll
-            for (Index k = 0; k < 4; ++k)
-                if (!(k < in_r0 ? keep0 : keep1)) out[f0 + k] = 0.f;
+    typedef float fvec __attribute__((ext_vector_type(VW)));
+    __shared__ int lists[4][kWave];
+    int* list = lists[threadIdx.x / kWave];
+    const unsigned lane = lane_id();
+    const unsigned waves = gridDim.x * 4u;
+    const unsigned blocks64 = (num_rows + 63u) / 64u;
+    for (unsigned b = blockIdx.x * 4u + threadIdx.x / kWave; b < blocks64; b += waves) {
+        const unsigned r = b * 64u + lane;
+        const bool wanted = r < num_rows && ((skip[r >> 5] >> (r & 31)) & 1u) == 0;
+        const unsigned count = compact_wanted_rows(list, r, wanted);
+        const unsigned total = count * vecs_per_row;
+        for (unsigned t = lane; t < total; t += kWave) {
+            const unsigned k = t / vecs_per_row;
+            const size_t at = static_cast<size_t>(list[k]) * vecs_per_row + (t - k * vecs_per_row);
+            if constexpr (VW == 1) {
+                __builtin_nontemporal_store(0.f, out + at);
+            } else {
+                fvec z = {};
+                __builtin_nontemporal_store(z, reinterpret_cast<fvec*>(out) + at);
+            }
         }
-        if (vecs - j <= stride) break;                     // the next index would run past the end (and could wrap)
     }
-    const Index tail = 4 * vecs;                            // up to 3 floats of the last row
-    if (tid < total_floats - tail) {
-        const Index r = (tail + tid) / dim;
-        if (!((skip[r >> 5] >> (r & 31)) & 1u)) out[tail + tid] = 0.f;
-    }
-}
-
-template <class Index>
-static void launch_zero_rows_typed(float* out, const uint32_t* skip, long long num_rows, int dim, hipStream_t stream)
-{
-    const uintptr_t a = reinterpret_cast<uintptr_t>(out);
-    const long long floats = num_rows * dim;
-    if (dim >= 4 && a % 16 == 0) {
-        long long blocks = (floats / 4 + 255) / 256;
-        if (blocks > 256 * 64) blocks = 256 * 64;
-        if (blocks < 1) blocks = 1;
-        hipLaunchKernelGGL((zero_flat_unless_kernel<Index>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, out,
-                           skip, static_cast<Index>(floats), static_cast<Index>(dim));
-        return;
-    }
-    const int vw = (dim % 2 == 0 && a % 8 == 0) ? 2 : 1;
-    const long long total = floats / vw;
-    long long blocks = (total + 255) / 256;
-    if (blocks > 256 * 64) blocks = 256 * 64;
-    const dim3 grid(static_cast<unsigned>(blocks)), block(256);
-    const Index t = static_cast<Index>(total), v = static_cast<Index>(dim / vw);
-    if (vw == 2) hipLaunchKernelGGL((zero_rows_unless_kernel<2, Index>), grid, block, 0, stream, out, skip, t, v);
-    else hipLaunchKernelGGL((zero_rows_unless_kernel<1, Index>), grid, block, 0, stream, out, skip, t, v);
 }
 
 static bool g_force_wide_index = false;
@@ -646,8 +619,28 @@ void set_force_wide_index(bool on) { g_force_wide_index = on; }
 int launch_zero_rows_unless(float* out, const uint32_t* skip, long long num_rows, int dim, hipStream_t stream)
 {
     if (num_rows <= 0 || dim <= 0) return kOk;
-    if (num_rows * dim < (1ll << 32) && !force_wide_index()) launch_zero_rows_typed<unsigned>(out, skip, num_rows, dim, stream);
-    else launch_zero_rows_typed<unsigned long long>(out, skip, num_rows, dim, stream);
+    const uintptr_t a = reinterpret_cast<uintptr_t>(out);
+    const int vw = (dim % 4 == 0 && a % 16 == 0) ? 4 : (dim % 2 == 0 && a % 8 == 0) ? 2 : 1;
+    const int vecs_per_row = dim / vw;
+    if (num_rows < (1ll << 31) && !force_wide_index()) {
+        long long blocks = (num_rows + 255) / 256;           // one wave per 64 rows
+        if (blocks > 256 * 16) blocks = 256 * 16;
+        const dim3 grid(static_cast<unsigned>(blocks)), block(256);
+        const unsigned n = static_cast<unsigned>(num_rows), v = static_cast<unsigned>(vecs_per_row);
+        if (vw == 4) hipLaunchKernelGGL(zero_listed_rows_kernel<4>, grid, block, 0, stream, out, skip, n, v);
+        else if (vw == 2) hipLaunchKernelGGL(zero_listed_rows_kernel<2>, grid, block, 0, stream, out, skip, n, v);
+        else hipLaunchKernelGGL(zero_listed_rows_kernel<1>, grid, block, 0, stream, out, skip, n, v);
+    } else {
+        // any size: one thread per vector of the matrix
+        const unsigned long long total = static_cast<unsigned long long>(num_rows) * vecs_per_row;
+        unsigned long long blocks = (total + 255) / 256;
+        if (blocks > 256 * 64) blocks = 256 * 64;
+        const dim3 grid(static_cast<unsigned>(blocks)), block(256);
+        const unsigned long long v = static_cast<unsigned long long>(vecs_per_row);
+        if (vw == 4) hipLaunchKernelGGL((zero_rows_unless_kernel<4, unsigned long long>), grid, block, 0, stream, out, skip, total, v);
+        else if (vw == 2) hipLaunchKernelGGL((zero_rows_unless_kernel<2, unsigned long long>), grid, block, 0, stream, out, skip, total, v);
+        else hipLaunchKernelGGL((zero_rows_unless_kernel<1, unsigned long long>), grid, block, 0, stream, out, skip, total, v);
+    }
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }
