@@ -170,7 +170,7 @@ size_t eppgcn_feature_workspace_floats(int64_t num_nodes, int dim)
 int eppgcn_plan_recommended(int64_t num_nodes, int dim)
 {
     if (num_nodes <= 0 || dim <= 0) return 0;
-    return static_cast<double>(feature_workspace_floats(num_nodes, dim)) * 4.0 >= 192.0 * (1 << 20) ? 1 : 0;
+    return static_cast<double>(feature_workspace_floats(num_nodes, dim)) * 4.0 >= 4.0 * (1 << 20) ? 1 : 0;
 }
 size_t eppgcn_plan_bytes(int64_t num_parts, int64_t num_slots, int64_t num_nodes)
 {

@@ -88,9 +88,11 @@ int eppgcn_feature_workspace_pitch(int dim);
  * records, one bit per vertex, the rows that consist of a single non-empty group: the kernel
  * writes those with one plain store, so the output clear of a planned call skips them.
  * No counterpart in the reference. */
-/* 1 when a plan is expected to pay off: the [num_nodes, dim] feature table (192 MB or more) does
- * not stay resident in the last-level caches by itself.  Measured: at 268 MB the plan takes the
- * width-16 forward from 2.03 to 1.35 ms, at 67 MB it costs 5 % (its partial sums need atomics). */
+/* 1 when a plan is expected to pay off: the [num_nodes, dim] feature table has 4 MB or more.  Large
+ * tables (hundreds of MB) gain from the column-blocked order (at 268 MB the width-16 forward goes
+ * from 2.03 to 1.25 ms); small ones still gain 6-8 % from the length-sorted groups, the precomputed
+ * group flags and the selective output clear (R-MAT scale 16 ... 20); below that the calls are
+ * launch-bound and a plan changes nothing. */
 int eppgcn_plan_recommended(int64_t num_nodes, int dim);
 size_t eppgcn_plan_bytes(int64_t num_parts, int64_t num_slots, int64_t num_nodes);
 size_t eppgcn_plan_workspace_bytes(int64_t num_parts);
