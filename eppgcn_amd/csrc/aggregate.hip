@@ -22,7 +22,12 @@
 // workspace the features are scaled once per call (ws[c,:] = s[c]*in[c,:], one
 // streaming pass) and the kernel gathers pre-scaled rows and multiplies by s[r]
 // at the flush.  Without a workspace the kernel stages (id, scale) pairs and
-// weights every row by fl32(s[r]*s[c]) as the reference does.
+// weights every row by fl32(s[r]*s[c]) as the reference does.  A pruned path that
+// reads few rows (bitmap of the vertices in its edge list) scales only those.
+//
+// Output clear.  Rows summed with atomics, and rows without groups, must start
+// at zero; a row that is one non-empty group is written whole by one store.  With
+// a plan (which records those rows) only the former are cleared.
 //
 // Flush.  Groups of one row that sit in the same wave are first summed across
 // teams in registers (DPP rotations / ds_swizzle when the whole wave is one row,
