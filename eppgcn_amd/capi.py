@@ -55,7 +55,7 @@ def load():
     lib.eppgcn_plan_bytes.restype = sz
     lib.eppgcn_plan_workspace_bytes.argtypes = [i64]
     lib.eppgcn_plan_workspace_bytes.restype = sz
-    lib.eppgcn_build_plan.argtypes = [p, p, p, p, i, i64, i, i, p, sz, p, sz, p]
+    lib.eppgcn_build_plan.argtypes = [p, p, p, p, i, i64, i, i, i, p, sz, p, sz, p]
     lib.eppgcn_build_plan.restype = i
     lib.eppgcn_spmm_forward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, sz, p, p]
     lib.eppgcn_spmm_backward.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, p, sz, p, p]
@@ -265,9 +265,10 @@ def _aligned_buffer(nbytes, device):
 
 
 def build_plan(part_ptr, column_index, num_parts: int, num_slots: int, num_nodes: int, dim: int,
-               part2node=None, ids=None):
+               part2node=None, ids=None, block_shift: int = 0):
     """Column-blocked execution plan of the groups; build once per graph and group array and pass it
-    as ``plan=`` to the aggregation calls.  Forward groups: give part2node; backward path: give ids."""
+    as ``plan=`` to the aggregation calls.  Forward groups: give part2node; backward path: give ids.
+    ``block_shift``: 0 = blocks sized for the width, n = blocks of 2^n vertices (31: one block)."""
     lib = load()
     _dev(part_ptr, torch.int32, "part_ptr"); _dev(column_index, torch.int32, "column_index")
     if (part2node is None) == (ids is None):
@@ -281,7 +282,7 @@ def build_plan(part_ptr, column_index, num_parts: int, num_slots: int, num_nodes
     wbytes = lib.eppgcn_plan_workspace_bytes(int(num_parts))
     ws, wbase = _aligned_buffer(wbytes, part_ptr.device)
     _check(lib.eppgcn_build_plan(_ptr(part_ptr), _ptr(column_index), _ptr(part2node), _ptr(ids), int(num_parts),
-                                 int(num_slots), int(num_nodes), int(dim), C.c_void_p(base), nbytes,
+                                 int(num_slots), int(num_nodes), int(dim), int(block_shift), C.c_void_p(base), nbytes,
                                  C.c_void_p(wbase), wbytes, _stream()))
     torch.cuda.current_stream().synchronize()      # the workspace is released on return
     return Plan(buf, base, int(num_parts), int(num_slots), int(num_nodes))

@@ -724,8 +724,9 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
 {
     const bool prescaled = workspace != nullptr;
     int ld_in = dim;
-    // rows the kernel writes with one plain store (a plan knows them) need no clearing
-    if (single_rows && num_parts > 0) {
+    // rows the kernel writes with one plain store (a plan knows them) need no clearing; with fewer
+    // groups than half the rows most rows have no group at all and the plain fill is the faster clear
+    if (single_rows && 2ll * num_parts >= num_nodes) {
         if (int rc = launch_zero_rows_unless(out, single_rows, num_nodes, dim, stream)) return rc;
     } else {
         if (int rc = launch_zero_words(out, static_cast<size_t>(num_nodes) * dim, stream)) return rc;

@@ -80,7 +80,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 7; }
+int eppgcn_abi_version(void) { return 8; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -179,16 +179,18 @@ size_t eppgcn_plan_bytes(int64_t num_parts, int64_t num_slots, int64_t num_nodes
 size_t eppgcn_plan_workspace_bytes(int64_t num_parts) { return plan_workspace_bytes(num_parts); }
 
 int eppgcn_build_plan(const int32_t* part_pointers, const int32_t* column_index, const int32_t* part2node,
-                      const int32_t* ids, int num_parts, int64_t num_slots, int num_nodes, int dim, void* plan,
-                      size_t plan_size, void* workspace, size_t workspace_bytes, void* stream)
+                      const int32_t* ids, int num_parts, int64_t num_slots, int num_nodes, int dim, int block_shift,
+                      void* plan, size_t plan_size, void* workspace, size_t workspace_bytes, void* stream)
 {
     EPPGCN_REQUIRE(num_parts >= 0 && num_slots >= 0 && num_nodes >= 0 && dim > 0, "negative size");
+    EPPGCN_REQUIRE(block_shift >= 0 && block_shift <= 31, "block_shift must be 0 (automatic) or 1..31");
     if (num_parts == 0) return kOk;
     EPPGCN_REQUIRE(part_pointers && column_index && plan, "null pointer");
     EPPGCN_REQUIRE((part2node != nullptr) != (ids != nullptr), "give exactly one of part2node (forward) and ids (backward)");
     EPPGCN_REQUIRE(aligned(plan, 256) && workspace && aligned(workspace, 256), "plan and workspace must be 256-byte aligned");
     return launch_build_plan(part_pointers, column_index, part2node, ids, num_parts, num_slots, num_nodes,
-                             schedule_shift(dim), plan, plan_size, workspace, workspace_bytes,
+                             block_shift > 0 ? block_shift : schedule_shift(dim), plan, plan_size, workspace,
+                             workspace_bytes,
                              static_cast<hipStream_t>(stream));
 }
 

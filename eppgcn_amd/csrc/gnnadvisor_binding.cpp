@@ -105,7 +105,7 @@ Tensor aligned_bytes(size_t bytes, const Tensor& like, void** base)
 // rows: part2Node (forward groups, is_forward) or the per-edge id list (backward path);
 // num_slots < 0: read it from part_ptr[num_parts] when the plan has to be built
 const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& rows, bool is_forward, int64_t num_parts,
-                     int64_t num_slots, int num_nodes, int dim)
+                     int64_t num_slots, int num_nodes, int dim, int block_shift = 0)
 {
     if (num_parts <= 0 || g_plan_policy < 0) return nullptr;
     if (g_plan_policy == 0 && !eppgcn_plan_recommended(num_nodes, dim)) return nullptr;
@@ -134,7 +134,7 @@ const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& ro
     check(eppgcn_build_plan(part_ptr.data_ptr<int32_t>(), col.data_ptr<int32_t>(),
                             is_forward ? rows.data_ptr<int32_t>() : nullptr,
                             is_forward ? nullptr : rows.data_ptr<int32_t>(), static_cast<int>(num_parts), num_slots,
-                            num_nodes, dim_of_class(dc), base, bytes, wbase, wbytes, stream_of(part_ptr)),
+                            num_nodes, dim_of_class(dc), block_shift, base, bytes, wbase, wbytes, stream_of(part_ptr)),
           "build_plan");
     g_plans.push_front(std::move(e));
     if (g_plans.size() > kMaxPlans) g_plans.pop_back();
@@ -142,8 +142,8 @@ const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& ro
 }
 
 // Per backward path, remembered from its first use:
-//   - whether it runs with a plan: a heavily pruned path gathers from few distinct rows, which stay
-//     cached without one, so plans are built for paths that keep at least half of the edges;
+//   - whether its plan is column-blocked: a heavily pruned path gathers from few distinct rows, which
+//     stay cached in any order, so only paths that keep at least half of the edges are blocked;
 //   - the bitmap of the rows it gathers, when they are fewer than half of the vertices: the
 //     pre-scaling pass of the gradient then touches those rows only.
 // An entry is valid for exactly the tensors it was made from (same storage, same version counters);
@@ -360,9 +360,9 @@ std::vector<Tensor> ours_backward(Tensor d_output, Tensor X, Tensor W, Tensor id
         const PathChoice& choice = path_choice(partPointer, edgeList, numParts, num_nodes, &valid_len);
         if (choice.gathered.defined())
             gathered = reinterpret_cast<const uint32_t*>(choice.gathered.data_ptr<int32_t>());
-        if (choice.use_plan)
-            plan = plan_for(partPointer, edgeList, id, false, numParts, valid_len, num_nodes,
-                            static_cast<int>(d_output.size(1)));
+        // a heavily pruned path keeps its groups in one block (its few gathered rows stay cached anyway)
+        plan = plan_for(partPointer, edgeList, id, false, numParts, valid_len, num_nodes,
+                        static_cast<int>(d_output.size(1)), choice.use_plan ? 0 : 31);
     }
     check(eppgcn_ours_backward(d_input_prime.data_ptr<float>(), f32(d_output), i32(id), i32(partPointer),
                                i32(edgeList), f32(degrees), static_cast<int>(d_output.size(0)),

@@ -103,9 +103,11 @@ def prepare(graph: graphs.Graph, num_layers: int = 2, train_ratio: float = 0.1, 
         part_pointer, num_parts, v2 = capi.split_back_part(node_degs[k], e, bps)
         assert v2 == valid_len
         width = widths[min(k, len(widths) - 1)]
-        # a heavily pruned path gathers from few distinct rows, which stay cached without a plan
-        path_plan = (capi.build_plan(part_pointer, edge_list, num_parts, valid_len, n, width, ids=ids)
-                     if plan and num_parts > 0 and 2 * valid_len >= e else None)
+        # a heavily pruned path gathers from few distinct rows, which stay cached in any order: its
+        # plan keeps the groups in one block
+        path_plan = (capi.build_plan(part_pointer, edge_list, num_parts, valid_len, n, width, ids=ids,
+                                     block_shift=0 if 2 * valid_len >= e else 31)
+                     if plan and num_parts > 0 else None)
         # the pre-scaling pass of the gradient only has to cover the rows the path reads
         bitmap, distinct = capi.mark_gathered_rows(edge_list, valid_len, n)
         paths.append(BackwardPath(k + 1, ids, edge_list, part_pointer, node_degs[k], bps, num_parts,
