@@ -290,6 +290,31 @@ def test_plan_is_a_stable_column_block_reordering(api, name, ps):
         assert np.array_equal(plan.single_rows().cpu().numpy(), groups_per_row == 1)
 
 
+def test_plan_block_shift_argument(api):
+    """The per-call block size equals the tuning knob's, and 31 leaves one block: the groups keep
+    their order apart from the length classes of single-group rows."""
+    indptr, col = GRAPHS["hub"]()
+    n = indptr.size - 1
+    pp, p2n = co.build_part(5, indptr)
+    args = (dev(pp), dev(col), p2n.size, col.size, n, 16)
+    api.set_plan_shift(9)
+    try:
+        knob = api.build_plan(*args, part2node=dev(p2n))
+    finally:
+        api.set_plan_shift(0)
+    call = api.build_plan(*args, part2node=dev(p2n), block_shift=9)
+    for a, b in zip(knob.view(), call.view()):
+        assert torch.equal(a, b)
+    one = api.build_plan(*args, part2node=dev(p2n), block_shift=31)
+    ptr, row, flags, pcol = [t.cpu().numpy() for t in one.view()]
+    groups_per_row = np.bincount(p2n, minlength=n)
+    cls = np.where(groups_per_row[p2n] == 1, np.minimum(3, (np.diff(pp) - 1) >> 3), 3)
+    order = np.argsort(cls, kind="stable")
+    assert np.array_equal(row, p2n[order]) and np.array_equal(np.diff(ptr), np.diff(pp)[order])
+    with pytest.raises(api.EppgcnError):
+        api.build_plan(*args, part2node=dev(p2n), block_shift=32)
+
+
 @pytest.mark.parametrize("rounds", [0, 1, 3])
 @pytest.mark.parametrize("dim", [16, 22, 64, 256])
 @pytest.mark.parametrize("shift", [0, 3, 20])
