@@ -74,7 +74,7 @@ struct RowsArgs {
     int ld_out, out_cols, ld_x, ld_ref;
     int K, M;
     int relu_in;             // apply max(x, 0) to X on load
-    int vec_store;           // rows of out are 16-byte aligned
+    int vec_store;           // 0: scalar stores; 1: rows of out are 16-byte aligned; 2: the same, non-temporal
 };
 
 template <int VW, int MT, int CU>
@@ -151,7 +151,12 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_rows_kernel(RowsArgs a)
             for (int v = 0; v < 4; ++v)
                 if (m0 + v >= a.M) y[v] = 0.f;        // padding columns hold exact zeros
             if (a.vec_store && m0 + 4 <= a.out_cols) {
-                *reinterpret_cast<float4*>(orow + m0) = make_float4(y[0], y[1], y[2], y[3]);
+                if (a.vec_store == 2) {      // wide result rows are written once and not read back soon
+                    const floatx4 o = {y[0], y[1], y[2], y[3]};
+                    __builtin_nontemporal_store(o, reinterpret_cast<floatx4*>(orow + m0));
+                } else {
+                    *reinterpret_cast<float4*>(orow + m0) = make_float4(y[0], y[1], y[2], y[3]);
+                }
             } else {
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
@@ -225,6 +230,9 @@ int launch_dense_rows(float* out, int ld_out, int out_cols, const float* x, int 
         a.M = M - c0 > 0 ? (M - c0 < cols ? M - c0 : cols) : 0;
         a.relu_in = relu_in;
         a.vec_store = (ld_out % 4 == 0 && reinterpret_cast<uintptr_t>(a.out) % 16 == 0) ? 1 : 0;
+        // measured at 4.2 M rows: a [N, 96] result 0.63 -> 0.47 ms with non-temporal stores, [N, 16] and
+        // [N, 32] results unchanged or slower
+        if (a.vec_store && out_cols >= 64) a.vec_store = 2;
         const size_t lds = lds_per_tile * mt;
         hipError_t e;
         if (vw == 4) e = launch_rows_mt<4>(a, mt, cu, static_cast<unsigned>(blocks), lds, stream);
