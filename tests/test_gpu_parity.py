@@ -976,3 +976,41 @@ def test_ragged_random_graphs_whole_path(api):
         assert_close(got_b.cpu().numpy(), want_b, bound, "pruned backward")
 
     check()
+
+
+def test_calls_run_on_the_callers_stream(api):
+    """Work is issued on the stream the caller passes (torch's current stream here), not on the
+    default stream: two side streams (default priority) run the forward and the pruned backward
+    of different inputs at the same time with their own buffers; each result is complete after
+    synchronising its own stream only, and the path preparation on a side stream returns its counts
+    (it synchronises that stream itself)."""
+    indptr, col = GRAPHS["medium"]()
+    n = indptr.size - 1
+    s = scale_inv_sqrt(indptr)
+    rng = np.random.default_rng(21)
+    src = rng.random(n) < 0.3
+    d_col, d_s, d_indptr = dev(col), dev(s), dev(indptr)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s1):
+        pp, p2n = api.build_part(8, d_indptr, col.size)
+        degs = torch.zeros(n, dtype=torch.int32, device="cuda")
+        ids, edge_list, v = api.mark_compact(p2n, pp, d_col, dev(src), None, degs, True)
+        bpp, p, v2 = api.split_back_part(degs, col.size, 8)
+    s1.synchronize()
+    assert v == v2 == int(src[col].sum())
+    xs = [rng.standard_normal((n, 22)).astype(np.float32) for _ in range(2)]
+    outs = []
+    for x, stream in zip(xs, (s1, s2)):
+        with torch.cuda.stream(stream):
+            dx = dev(x)
+            fwd = api.spmm_forward(dx, d_col, d_s, pp, p2n, part_size=8)
+            bwd = api.ours_backward(dev((x * src[:, None]).astype(np.float32)), ids, bpp, edge_list, d_s, p, part_size=8)
+            outs.append((fwd, bwd))
+    for (fwd, bwd), x, stream in zip(outs, xs, (s1, s2)):
+        stream.synchronize()
+        bound = cf.abs_sum_bound(indptr, col, s, x)
+        assert_close(fwd.cpu().numpy(), co.spmm_f64(x, indptr, col, s), bound, "forward on a side stream")
+        assert_close(bwd.cpu().numpy(), co.spmm_f64((x * src[:, None]).astype(np.float32), indptr, col, s), bound,
+                     "pruned backward on a side stream")
+    torch.cuda.synchronize()
