@@ -5,7 +5,11 @@ compaction, split), pruned backward time, unpruned backward time, algorithmic GB
     python -m eppgcn_amd.sweep [--config cfg3_rmat20] [--ratios 0.01 0.1 0.5]
                                [--widths 16 64 256] [--groups 8 16 32 64] [--reps 5]
 
-Prints one JSON line per cell and a final summary line.  Needs the MI355X.
+Prints one JSON line per cell and a final summary line.  Needs the MI355X.  Launches are set up
+the way the extension module sets them up by itself: execution plans where the feature table has 4 MB
+or more (column-blocked for the forward groups and for paths that keep at least half of the edges,
+one block otherwise) and the gathered-rows bitmap for paths that read fewer than half of the rows;
+``--no_plans`` measures the bare kernels.
 """
 from __future__ import annotations
 
@@ -15,7 +19,7 @@ import time
 
 import torch
 
-from . import capi, graphs, workload
+from . import capi, graphs, param, workload
 
 
 def _events_ms(fn, reps):
@@ -37,14 +41,25 @@ def main():
     ap.add_argument("--widths", type=int, nargs="+", default=[16, 64, 256])
     ap.add_argument("--groups", type=int, nargs="+", default=[8, 16, 32, 64])
     ap.add_argument("--reps", type=int, default=5)
+    ap.add_argument("--no_plans", action="store_true", help="no execution plans, no gathered-rows bitmap")
     args = ap.parse_args()
 
     capi.load()
     dev = torch.device("cuda:0")
     g = graphs.make_graph(args.config, device=dev)
     n, e = g.num_nodes, g.num_edges
-    ps = max(1, int(g.avg_degree))
+    ps = max(param.MIN_AUTO_PART_SIZE, int(g.avg_degree))     # the decider's rule for the forward groups
     part_ptr, part2node = capi.build_part(ps, g.row_pointers, e)
+    fwd_plans = {}
+
+    def forward_plan(width):
+        if args.no_plans or not capi.plan_recommended(n, width):
+            return None
+        if width not in fwd_plans:
+            fwd_plans[width] = capi.build_plan(part_ptr, g.column_index, part2node.numel(), e, n, width,
+                                               part2node=part2node)
+        return fwd_plans[width]
+
     cells = []
     for ratio in args.ratios:
         mask = graphs.bernoulli_mask(n, ratio, 2, dev)
@@ -60,6 +75,8 @@ def main():
         compact_ms = _events_ms(lambda: capi.compact_back_edge(bem, g.column_index), args.reps)
         ids, edge_list, valid_len = capi.compact_back_edge(bem, g.column_index)
         valid_node = capi.count_nonzero(degs)
+        bitmap, distinct = capi.mark_gathered_rows(edge_list, valid_len, n)
+        gathered = bitmap if (2 * distinct < n and not args.no_plans) else None
         for gs in args.groups:
             split_ms = _events_ms(lambda: capi.split_back_part(degs, e, gs), args.reps)
             part_pointer, num_parts, _ = capi.split_back_part(degs, e, gs)
@@ -67,18 +84,25 @@ def main():
                 dy = graphs.normal32(7, (n, width), dev) * mask[:, None]
                 out = torch.empty_like(dy)
                 ws = capi.feature_workspace(n, width, dev)
+                plan = None
+                if not args.no_plans and num_parts > 0 and capi.plan_recommended(n, width):
+                    plan = capi.build_plan(part_pointer, edge_list, num_parts, valid_len, n, width, ids=ids,
+                                           block_shift=0 if 2 * valid_len >= e else 31)
                 capi.set_timing(True)
                 capi.clear_time()
                 for _ in range(args.reps):
-                    capi.ours_backward(dy, ids, part_pointer, edge_list, g.degrees, num_parts, gs, 1, 4, 16, out, ws)
+                    capi.ours_backward(dy, ids, part_pointer, edge_list, g.degrees, num_parts, gs, 1, 4, 16, out, ws,
+                                       plan=plan, gathered_rows=gathered)
                 pruned_ms = capi.get_time_ms(1) / args.reps
                 capi.clear_time()
                 for _ in range(args.reps):
-                    capi.spmm_forward(dy, g.column_index, g.degrees, part_ptr, part2node, ps, 32, 8, None, out, True, ws)
+                    capi.spmm_forward(dy, g.column_index, g.degrees, part_ptr, part2node, ps, 32, 8, None, out, True, ws,
+                                      plan=forward_plan(width))
                 unpruned_ms = capi.get_time_ms(1) / args.reps
                 capi.set_timing(False)
                 capi.clear_time()
                 nbytes = workload.bytes_pruned_backward(n, valid_len, num_parts, width)
+                del plan
                 cell = {"config": args.config, "ratio": ratio, "width": width, "group_size": gs,
                         "kept_edges": valid_len, "kept_rows": valid_node, "groups": num_parts,
                         "mark_ms": round(mark_ms, 4), "compact_ms": round(compact_ms, 4), "split_ms": round(split_ms, 4),
