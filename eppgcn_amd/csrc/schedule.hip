@@ -32,14 +32,17 @@ namespace eppgcn {
 static size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
 // ---------------------------------------------------------------- kernels
-// Sort key of group p: the column block of its first slot, except that all groups of a row with
-// at most `keep` groups share the key of the row's first group: such a row stays together in the
-// plan, is summed in registers and written once with plain stores, instead of leaving one
-// partial sum per column block to be combined with atomics (measured: the atomics of rows with
-// 2..16 groups cost more than the L2 hits of their later groups save).
+// Sort key of group p: the column block of its first slot, except that all groups of a short row
+// (at most `keep_slots` slots in at most kMaxRowWalk groups) share the key of the row's first group:
+// such a row stays together in the plan, is summed in registers and written once with plain stores,
+// instead of leaving one partial sum per column block to be combined with atomics (measured at group
+// size 31: the atomics of rows with 2..16 groups cost more than the L2 hits of their later groups
+// save; the bound is in slots because a row's gathers, not its groups, are what a block can speed up:
+// with groups of 4-8 slots a bound in groups spread rows of 40 slots and lost up to 2x at 256 columns).
+constexpr int kMaxRowWalk = 64;
 __global__ __launch_bounds__(256) void plan_keys_kernel(const int* __restrict__ part_ptr, const int* __restrict__ col,
                                                        const int* __restrict__ part2node, const int* __restrict__ ids,
-                                                       int num_parts, int shift, int keep, int classes,
+                                                       int num_parts, int shift, int keep_slots, int classes,
                                                        unsigned* __restrict__ keys, int* __restrict__ iota)
 {
     const int p = blockIdx.x * blockDim.x + threadIdx.x;
@@ -55,12 +58,13 @@ __global__ __launch_bounds__(256) void plan_keys_kernel(const int* __restrict__ 
         return (part2node ? part2node[j] : ids[b]) == row;
     };
     int start = p;
-    for (int k = 0; k < keep && start > 0 && same_row(start - 1); ++k) --start;
+    for (int k = 0; k < kMaxRowWalk && start > 0 && same_row(start - 1); ++k) --start;
     const bool start_found = !(start > 0 && same_row(start - 1));
     int last = p;
-    while (last + 1 < num_parts && last + 1 - start < keep && same_row(last + 1)) ++last;
+    while (last + 1 < num_parts && last + 1 - start < kMaxRowWalk && same_row(last + 1)) ++last;
     const bool end_found = !(last + 1 < num_parts && same_row(last + 1));
-    const bool short_row = start_found && end_found && last - start + 1 <= keep;
+    const bool short_row = keep_slots > 0 && start_found && end_found && last - start + 1 <= kMaxRowWalk &&
+                           part_ptr[last + 1] - part_ptr[start] <= keep_slots;
     const int key_col = short_row ? col[part_ptr[start]] : col[beg];
     unsigned key = static_cast<unsigned>(key_col) >> shift;
     if (classes) {
@@ -195,7 +199,7 @@ size_t plan_workspace_bytes(long long num_parts)
 int workspace_pitch(int dim);   // aggregate.hip
 
 static int g_force_shift = 0;
-static int g_keep_rows = 8;
+static int g_keep_rows = 8;      // in units of 32 slots: rows of up to 256 slots stay together
 static int g_length_classes = 1;
 void set_plan_length_classes(int on) { g_length_classes = on ? 1 : 0; }
 void set_schedule_shift(int shift) { g_force_shift = shift; }
@@ -256,7 +260,7 @@ int launch_build_plan(const int* part_ptr, const int* col, const int* part2node,
     }
     const unsigned blocks = static_cast<unsigned>((num_parts + 255) / 256);
     hipLaunchKernelGGL(plan_keys_kernel, dim3(blocks), dim3(256), 0, stream, part_ptr, col, part2node, ids, num_parts,
-                       shift, g_keep_rows, g_length_classes, keys_in, iota);
+                       shift, g_keep_rows * 32, g_length_classes, keys_in, iota);
     EPPGCN_HIP(hipGetLastError());
     EPPGCN_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, iota, order,
                                          static_cast<size_t>(num_parts), 0u, static_cast<unsigned>(bits), stream));

@@ -304,7 +304,8 @@ void eppgcn_set_wide_index(int on);
 /* Forces the column block size of eppgcn_build_plan to 2^shift vertices (0 = choose from the
  * feature width).  For tuning runs. */
 void eppgcn_set_plan_shift(int shift);
-/* Rows with at most this many groups stay together in a plan (default 8; 0 = block every group). */
+/* Rows of at most 32 * groups slots (and at most 64 groups) stay together in a plan (default 8, i.e.
+ * 256 slots; 0 = block every group). */
 void eppgcn_set_plan_keep_rows(int groups);
 /* Within a column block, order single-group rows by length class (1-8, 9-16, 17-24, 25+ slots) so
  * that the groups of one round take the same number of gather steps (default on). */

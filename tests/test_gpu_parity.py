@@ -267,11 +267,12 @@ def test_plan_is_a_stable_column_block_reordering(api, name, ps):
             assert np.array_equal(pcol[ptr[q]:ptr[q + 1]], col[pp[p]:pp[p + 1]])
         sizes = np.diff(pp)[order]
         assert np.array_equal(np.diff(ptr), sizes)
-        # sort key: column block of the group's first slot; rows with at most 8 groups use the key
-        # of their first group so that they stay together
+        # sort key: column block of the group's first slot; rows of at most 256 slots (in at most 64
+        # groups) use the key of their first group so that they stay together
         groups_per_row = np.bincount(p2n, minlength=n)
         row_first_group = np.concatenate([[0], np.cumsum(groups_per_row)[:-1]])
-        key_col = np.where(groups_per_row[p2n] <= 8, col[pp[row_first_group[p2n]]], col[pp[:-1]])[order]
+        short = (groups_per_row <= 64) & (np.diff(indptr) <= 256)
+        key_col = np.where(short[p2n], col[pp[row_first_group[p2n]]], col[pp[:-1]])[order]
         # second key: length class (steps of 8 slots) of rows that are a single group, 3 for the rest
         cls = np.where(groups_per_row[p2n] == 1, np.minimum(3, (np.diff(pp) - 1) >> 3), 3)[order]
         ok = False
