@@ -146,7 +146,7 @@ def main():
         capi.set_plan_keep_rows(args.plan_keep)
     t0 = time.perf_counter()
     wl = workload.prepare(g, 2, args.train_ratio, 2, args.part_size or None, args.backsize_mode, args.backsize,
-                          plan=False if (args.no_plan or args.no_workspace) else (True if args.force_plan else None),
+                          plan=False if args.no_plan else (True if args.force_plan else None),
                           fused=not args.stepwise_prep)
     torch.cuda.synchronize()
     prep_s = time.perf_counter() - t0

@@ -590,14 +590,12 @@ static hipError_t launch_slab(float* out, const float* in, const int* col, const
 #undef EPPGCN_LAUNCH
 }
 
-// Plans are only used with pre-scaled features: the per-edge-scale form is not instantiated for them.
 template <int VW, int OVW, class Groups>
 static hipError_t slab_either(bool prescaled, float* out, const float* in, const int* col, const float* scale,
                               Groups g, int num_parts, AggShape sh, hipStream_t stream)
 {
     if (prescaled) return launch_slab<VW, OVW, true>(out, in, col, scale, g, num_parts, sh, stream);
-    if constexpr (std::is_same<Groups, PlanGroups>::value) return hipErrorInvalidValue;
-    else return launch_slab<VW, OVW, false>(out, in, col, scale, g, num_parts, sh, stream);
+    return launch_slab<VW, OVW, false>(out, in, col, scale, g, num_parts, sh, stream);
 }
 
 // Row pitch of the pre-scaled workspace: rows of up to 128 bytes are padded to a power of two
@@ -775,13 +773,13 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
     return kOk;
 }
 
-// plan: nullptr, or an execution plan built for exactly these groups (used with a workspace).
+// plan: nullptr, or an execution plan built for exactly these groups.
 int aggregate_forward_groups(float* out, const float* in, const int* col, const float* scale,
                              const int* part_ptr, const int* part2node, const void* plan, int num_nodes, int dim,
                              int num_parts, int group_size, float* workspace, hipStream_t stream, double* sink,
                              double* sink2)
 {
-    if (plan && workspace && num_parts > 0) {
+    if (plan && num_parts > 0) {
         const PlanView v = plan_view(const_cast<void*>(plan), num_parts, num_nodes);
         return aggregate_dispatch(out, in, v.col, scale, PlanGroups{v.ptr, v.row, v.flags}, num_nodes, dim, num_parts,
                                   group_size, workspace, stream, sink, sink2, v.single);
@@ -797,7 +795,7 @@ int aggregate_compacted_groups(float* out, const float* in, const int* ids, cons
                                int num_parts, int group_size, float* workspace, const uint32_t* gathered_rows,
                                hipStream_t stream, double* sink, double* sink2)
 {
-    if (plan && workspace && num_parts > 0) {
+    if (plan && num_parts > 0) {
         const PlanView v = plan_view(const_cast<void*>(plan), num_parts, num_nodes);
         return aggregate_dispatch(out, in, v.col, scale, PlanGroups{v.ptr, v.row, v.flags}, num_nodes, dim, num_parts,
                                   group_size, workspace, stream, sink, sink2, v.single, gathered_rows);

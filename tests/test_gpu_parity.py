@@ -344,6 +344,10 @@ def test_planned_aggregation_exact_integer_sums(api, rounds, dim, shift):
             got = api.spmm_forward(dev(x), dcol, dev(s), dpp, dp2n, part_size=ps, plan=plan,
                                    out=torch.full((n, dim), float("nan"), device="cuda"))
             assert np.array_equal(got.cpu().numpy().astype(np.float64), want), f"forward ps={ps}"
+            # a plan also serves calls without a feature workspace (per-edge scale gather)
+            got = api.spmm_forward(dev(x), dcol, dev(s), dpp, dp2n, part_size=ps, plan=plan, workspace=None,
+                                   out=torch.full((n, dim), float("nan"), device="cuda"))
+            assert np.array_equal(got.cpu().numpy().astype(np.float64), want), f"forward ps={ps}, no workspace"
             oid, oedge, bpp, p = _gpu_path(api, indptr, col, src, 5, ps)
             if p == 0:
                 continue
@@ -354,6 +358,9 @@ def test_planned_aggregation_exact_integer_sums(api, rounds, dim, shift):
             gb = api.ours_backward(dy, oid, bpp, oedge, dev(s), p, part_size=ps, plan=bplan,
                                    out=torch.full((n, dim), float("nan"), device="cuda"))
             assert np.array_equal(gb.cpu().numpy().astype(np.float64), want_b), f"pruned ps={ps}"
+            gb = api.ours_backward(dy, oid, bpp, oedge, dev(s), p, part_size=ps, plan=bplan, workspace=None,
+                                   out=torch.full((n, dim), float("nan"), device="cuda"))
+            assert np.array_equal(gb.cpu().numpy().astype(np.float64), want_b), f"pruned ps={ps}, no workspace"
     finally:
         api.set_rounds(0)
         api.set_plan_shift(0)
@@ -374,6 +381,9 @@ def test_planned_aggregation_within_tolerance(api, name, dim):
         got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp), dev(p2n), part_size=ps, plan=plan,
                                out=torch.full((n, dim), float("nan"), device="cuda"))
         assert_close(got.cpu().numpy(), want, bound, f"{name} D={dim} ps={ps} planned")
+        got = api.spmm_forward(dev(x), dev(col), dev(s), dev(pp), dev(p2n), part_size=ps, plan=plan, workspace=None,
+                               out=torch.full((n, dim), float("nan"), device="cuda"))
+        assert_close(got.cpu().numpy(), want, bound, f"{name} D={dim} ps={ps} planned, no workspace")
 
 
 def test_forward_unit_scale_integer_features_bit_exact(api):
