@@ -35,7 +35,7 @@ def parse():
                     help="cfg1_uniform, cfg2_chunglu, cfg3_rmat20, cfg4_rmat22 (the metric's configuration), or "
                          "rmat:<scale>:<pairs per vertex> for an R-MAT graph of another size")
     ap.add_argument("--train_ratio", type=float, default=0.1)
-    ap.add_argument("--backsize_mode", default="constant", choices=["constant", "map", "threshold"])
+    ap.add_argument("--backsize_mode", default="constant", choices=["constant", "map", "threshold", "wave64"])
     ap.add_argument("--backsize", type=int, default=32)
     ap.add_argument("--part_size", type=int, default=0, help="forward group size (0 = int(avg degree))")
     ap.add_argument("--team", type=int, default=0, help="force lanes per group (0 = automatic)")

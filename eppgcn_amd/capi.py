@@ -25,7 +25,7 @@ EXPORTS = [
     "eppgcn_feature_workspace_pitch", "eppgcn_update_forward", "eppgcn_update_backward_input",
     "eppgcn_update_workspace_bytes", "eppgcn_update_backward_weight", "eppgcn_update_supported",
     "eppgcn_mark_compact_workspace_bytes", "eppgcn_mark_compact", "eppgcn_set_plan_length_classes",
-    "eppgcn_mark_gathered_rows", "eppgcn_set_wide_index",
+    "eppgcn_mark_gathered_rows", "eppgcn_set_wide_index", "eppgcn_wave64_back_part_size",
 ]
 
 _lib = None
@@ -71,6 +71,8 @@ def load():
     lib.eppgcn_count_nonzero.argtypes = [p, i64, p, C.POINTER(i64), p]
     lib.eppgcn_map_back_part_size.argtypes = [i64, i64, C.POINTER(i)]
     lib.eppgcn_threshold_back_part_size.argtypes = [i64, i64]
+    lib.eppgcn_wave64_back_part_size.argtypes = [i64, i64]
+    lib.eppgcn_wave64_back_part_size.restype = i
     lib.eppgcn_split_back_part.argtypes = [p, i, i, p, i64, p, sz, p, C.POINTER(i64), C.POINTER(i64), p]
     lib.eppgcn_build_part.argtypes = [p, i, i, p, p, i64, p, sz, p, C.POINTER(i64), p]
     lib.eppgcn_get_ginfo.argtypes = [p, i64, i64, p, C.POINTER(C.c_float), p]
@@ -446,6 +448,11 @@ def map_back_part_size(valid_node: int, valid_len: int):
 
 def threshold_back_part_size(valid_node: int, valid_len: int) -> int:
     return int(load().eppgcn_threshold_back_part_size(int(valid_node), int(valid_len)))
+
+
+def wave64_back_part_size(valid_node: int, valid_len: int) -> int:
+    """The group-size rule re-fitted for this library's kernels (16 or 32)."""
+    return int(load().eppgcn_wave64_back_part_size(int(valid_node), int(valid_len)))
 
 
 def split_back_part(node_deg, num_edges: int, part_size: int):

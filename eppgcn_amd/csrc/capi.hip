@@ -80,7 +80,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 8; }
+int eppgcn_abi_version(void) { return 9; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -310,6 +310,15 @@ int eppgcn_threshold_back_part_size(int64_t valid_node, int64_t valid_len)
     if (valid_degree < 256) return 32;
     if (valid_degree < 512) return 64;
     return 0;
+}
+
+int eppgcn_wave64_back_part_size(int64_t valid_node, int64_t valid_len)
+{
+    // measured on R-MAT scale 20 and 22, mask ratios 0.01-0.5, widths 16-256: 16 is best or within 2 % of the
+    // best up to an average kept degree of about 20, 32 above (first-layer paths with 30 kept edges per row:
+    // 8 / 16 / 32 / 64 / 128 -> 1.97 / 1.42 / 1.21 / 1.30 / 1.63 ms)
+    if (valid_node <= 0) return 16;
+    return valid_len / valid_node < 24 ? 16 : 32;
 }
 
 static int finish_split(void* workspace, hipStream_t s, int32_t* d_counts, int64_t* h_a, int64_t* h_b)

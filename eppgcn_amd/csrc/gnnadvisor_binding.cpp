@@ -492,6 +492,12 @@ int get_map_back_part_size(Tensor node_deg, int valid_len)
     return ps;
 }
 
+// The group-size rule re-fitted for the wave64 kernels (no counterpart in the reference's module).
+int get_wave64_back_part_size(Tensor node_deg, int valid_len)
+{
+    return eppgcn_wave64_back_part_size(valid_nodes(node_deg), valid_len);
+}
+
 std::vector<Tensor> split_back_part(Tensor node_deg, int num_edges, int back_part_size)
 {
     auto s = split(node_deg, num_edges, back_part_size);
@@ -564,6 +570,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("compact_back_edge", &compact_back_edge, "compact the kept edges of one layer (HIP)");
     m.def("mark_compact", &mark_compact, "marking + compaction of one layer in one pass (HIP)");
     m.def("get_map_back_part_size", &get_map_back_part_size, "backward group size from the fitted regression");
+    m.def("get_wave64_back_part_size", &get_wave64_back_part_size, "backward group size re-fitted for wave64 kernels");
     m.def("split_back_part", &split_back_part, "split kept edges into backward groups (HIP)");
     m.def("get_ginfo", &get_ginfo, "degree-distribution features of the kept path");
 }

@@ -12,6 +12,8 @@ Differences, all deliberate:
   * ``--dataset`` also accepts a synthetic graph name (``cfg1_uniform``, ``rmat:<scale>:<factor>``
     ...) when no graph file is given; the train mask is then drawn instead of read.
   * the device is the current one (the reference hard-codes device 1, gcn_main.py:69).
+  * ``--backsize_mode wave64`` (an addition) picks 16 or 32 from the kept edges per row, the rule
+    re-fitted for this library's kernels.
   * ``--degree_norm inv_sqrt`` (an addition) fills the scale vector with deg^-1/2 instead of the
     reference loader's sqrt(deg) (EPPGCN/dataset.py:117-119).
   * ``--kernel_timers`` and ``--hip_graph`` (additions) switch the per-op device timers off and
@@ -52,7 +54,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--single_spmm", default="False", help="time the forward aggregation alone", **tf)
     ap.add_argument("--verify_spmm", default="False", help="check one forward aggregation against torch", **tf)
     ap.add_argument("--backsize", type=int, default=0, help="backward group size of all layers (constant mode; 0 = 32)")
-    ap.add_argument("--backsize_mode", type=str, default="constant", choices=["map", "net", "constant"])
+    ap.add_argument("--backsize_mode", type=str, default="constant", choices=["map", "net", "constant", "wave64"])
     ap.add_argument("--degree_norm", type=str, default="sqrt", choices=["sqrt", "inv_sqrt"],
                     help="scale vector: sqrt(deg) as the reference's loader fills it, or deg^-1/2 (symmetric GCN norm)")
     ap.add_argument("--kernel_timers", default="True", **tf,

@@ -123,6 +123,8 @@ class Trainer:
             valid_len = int(info[0].item())
             if self.backsize_mode == "map":
                 part_size = self.GNNA.get_map_back_part_size(ds.node_degs[i], valid_len)
+            elif self.backsize_mode == "wave64":
+                part_size = self.GNNA.get_wave64_back_part_size(ds.node_degs[i], valid_len)
             else:
                 part_size = max(1, self.backsize)
             part_pointer, num_parts = self.GNNA.split_back_part(ds.node_degs[i], ds.num_edges, part_size)

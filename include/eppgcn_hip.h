@@ -214,6 +214,12 @@ int eppgcn_map_back_part_size(int64_t valid_node, int64_t valid_len, int* clampe
 /* Legacy threshold rule of build_back_part (EPPGCN.cpp:246-258); returns 0 when the
  * ratio is >= 512, as the reference leaves it. */
 int eppgcn_threshold_back_part_size(int64_t valid_node, int64_t valid_len);
+/* The same decision re-fitted for the wave64 kernels of this library: 16 while the path keeps fewer
+ * than 24 edges per row with kept edges, 32 above.  With partial sums carried from group to group
+ * inside a wave the group size matters far less than for the reference's kernel (within 10 % over
+ * 8..64 in every measured cell), so two values are all the fit supports.  No counterpart in the
+ * reference (its rules are EPPGCN.cpp:246-258 and :303-310). */
+int eppgcn_wave64_back_part_size(int64_t valid_node, int64_t valid_len);
 
 /* Splits the kept edges of every vertex into groups of part_size and writes the
  * group pointers: part_pointer[0..P] with part_pointer[P] = V, zero after that up

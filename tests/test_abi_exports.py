@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared_functions():
         assert hasattr(lib, name), f"{name} is declared in include/eppgcn_hip.h but not exported"
     assert sorted(capi.EXPORTS) == declared_functions()
-    assert capi.load().eppgcn_abi_version() == 8
+    assert capi.load().eppgcn_abi_version() == 9
 
 
 def test_host_only_heuristics_match_the_checker():
@@ -39,6 +39,9 @@ def test_host_only_heuristics_match_the_checker():
         raw = co.map_back_part_size(vn, vl)
         assert capi.map_back_part_size(vn, vl) == (max(raw, 1), raw < 1)
         assert capi.threshold_back_part_size(vn, vl) == co.threshold_back_part_size(vn, vl)
+    # the re-fitted rule: 16 below 24 kept edges per kept row, 32 from there on
+    assert [capi.wave64_back_part_size(vn, vl) for vn, vl in [(0, 0), (10, 0), (10, 239), (10, 240), (3, 10 ** 9)]] == \
+        [16, 16, 16, 32, 32]
 
 
 def test_product_package_never_imports_the_checker():
@@ -112,5 +115,5 @@ def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
     env = dict(os.environ, LD_LIBRARY_PATH="/opt/rocm/lib:" + os.environ.get("LD_LIBRARY_PATH", ""))
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True, env=env).stdout.split("\n")
     from oracle import c_oracle as co
-    assert out[0].split() == ["8", "32", "320", str(max(1, co.map_back_part_size(1000, 5000))), "0", "-1"]
+    assert out[0].split() == ["9", "32", "320", str(max(1, co.map_back_part_size(1000, 5000))), "0", "-1"]
     assert "dim > 0" in out[1]

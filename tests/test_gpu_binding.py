@@ -329,7 +329,7 @@ def test_driver_command_line_end_to_end(GNNA, tmp_path, capsys):
     dsmod.write_train_mask(str(tmp_path), 0.3, np.random.default_rng(2).random(n) < 0.3)
     common = ["--dataset", "toy", "--dataDir", str(tmp_path), "--dim", "24", "--hidden", "16", "--classes", "5",
               "--train_ratio", "0.3", "--num_epoches", "3", "--degree_norm", "inv_sqrt"]
-    for extra in (["--layers", "3", "--backsize_mode", "map"],
+    for extra in (["--layers", "3", "--backsize_mode", "map"], ["--layers", "2", "--backsize_mode", "wave64"],
                   ["--layers", "2", "--backsize_mode", "constant", "--backsize", "8", "--kernel_timers", "False",
                    "--manual_mode", "True", "--partSize", "4", "--verbose_mode", "True"]):
         assert gcn_main.main(common + extra) == 0
