@@ -937,7 +937,10 @@ def test_ragged_random_graphs_whole_path(api):
     from hypothesis import strategies as st
     from tests.test_oracle_fuzz import ragged_graph
 
-    @settings(max_examples=150, deadline=None, derandomize=True, database=None,
+    import os
+    examples = int(os.environ.get("EPPGCN_FUZZ_EXAMPLES", "150"))       # raise it for a longer hunt
+
+    @settings(max_examples=examples, deadline=None, derandomize=examples == 150, database=None,
               suppress_health_check=list(HealthCheck))
     @given(ragged_graph(), st.integers(1, 9), st.integers(1, 9), st.sampled_from([0.0, 0.1, 0.5, 1.0]),
            st.sampled_from([1, 3, 4, 16, 22]))

@@ -14,7 +14,7 @@ from oracle import closed_forms as cf
 
 @st.composite
 def ragged_graph(draw):
-    n = draw(st.integers(1, 40))
+    n = draw(st.one_of(st.integers(1, 40), st.integers(41, 700)))     # one wave's worth, or several
     seed = draw(st.integers(0, 2 ** 31 - 1))
     density = draw(st.sampled_from([0.0, 0.02, 0.1, 0.4, 1.0]))
     empty_rows = draw(st.sampled_from([0.0, 0.3, 0.9]))
