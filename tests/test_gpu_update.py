@@ -127,3 +127,33 @@ def test_aggregation_accepts_the_prescaled_product(api, dim):
     tb = (np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64)).astype(np.float32)
     bound = bound + co.spmm_f64(tb, indptr, col, s)
     assert_close(got.cpu().numpy(), want, bound, f"prescaled aggregation, width {dim}")
+
+
+def test_update_products_on_random_shapes(api):
+    """Property-based: any shape the kernels accept (rows 1-400, reduction length 1-1024, 1-150
+    result columns, 1-64 for the weight gradient), with and without the ReLU on load, the row
+    scale, a padded result pitch and the ReLU mask of the input gradient, stays within tolerance
+    of the float64-accumulated checker."""
+    from hypothesis import HealthCheck, given, settings
+    from hypothesis import strategies as st
+
+    @settings(max_examples=120, deadline=None, derandomize=True, database=None, suppress_health_check=list(HealthCheck))
+    @given(st.integers(1, 400), st.one_of(st.integers(1, 40), st.integers(41, 1024)), st.integers(1, 150),
+           st.booleans(), st.integers(0, 2 ** 31 - 1))
+    def check(n, k, m, relu, seed):
+        x, w, g, s = data(n, k, m, seed)
+        xa = np.maximum(x, 0) if relu else x
+        bound = np.abs(xa).astype(np.float64) @ np.abs(w).astype(np.float64)
+        ld = api.feature_workspace_pitch(m)
+        got = api.update_forward(dev(x), dev(w), scale=dev(s), relu_input=relu, ld_out=ld).cpu().numpy()
+        assert not got[:, m:].any()
+        assert_close(got[:, :m], co.update_forward(x, w, scale=s, relu_input=relu), bound * s[:, None], "forward")
+        gb = np.abs(g).astype(np.float64) @ np.abs(w).astype(np.float64).T
+        got = api.update_backward_input(dev(g), dev(w), relu_ref=dev(x) if relu else None).cpu().numpy()
+        assert_close(got, co.update_backward_input(g, w, relu_ref=x if relu else None), gb, "input gradient")
+        if m <= 64:
+            wb = np.abs(xa).astype(np.float64).T @ np.abs(g).astype(np.float64)
+            got = api.update_backward_weight(dev(x), dev(g), relu_input=relu).cpu().numpy()
+            assert_close(got, co.update_backward_weight(x, g, relu_input=relu), wb, "weight gradient")
+
+    check()
