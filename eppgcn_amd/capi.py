@@ -26,7 +26,10 @@ EXPORTS = [
     "eppgcn_update_workspace_bytes", "eppgcn_update_backward_weight", "eppgcn_update_supported",
     "eppgcn_mark_compact_workspace_bytes", "eppgcn_mark_compact", "eppgcn_set_plan_length_classes",
     "eppgcn_mark_gathered_rows", "eppgcn_set_wide_index", "eppgcn_wave64_back_part_size",
+    "eppgcn_compact_back_edge_static", "eppgcn_compact_back_edge_static_max_length",
 ]
+
+ABI_VERSION = 10      # what eppgcn_abi_version() of a matching library returns
 
 _lib = None
 
@@ -47,6 +50,9 @@ def load():
     p, i, i64, sz = C.c_void_p, C.c_int, C.c_int64, C.c_size_t
     lib.eppgcn_last_error.restype = C.c_char_p
     lib.eppgcn_abi_version.restype = i
+    if lib.eppgcn_abi_version() != ABI_VERSION:
+        raise EppgcnError(f"{LIB_PATH} has ABI version {lib.eppgcn_abi_version()}, this package expects "
+                          f"{ABI_VERSION}; rebuild it with `python -m eppgcn_amd.build`")
     lib.eppgcn_feature_workspace_floats.argtypes = [i64, i]
     lib.eppgcn_feature_workspace_floats.restype = sz
     lib.eppgcn_plan_recommended.argtypes = [i64, i]
@@ -68,6 +74,9 @@ def load():
     lib.eppgcn_split_workspace_bytes.argtypes = [i64]
     lib.eppgcn_split_workspace_bytes.restype = sz
     lib.eppgcn_compact_back_edge.argtypes = [p, p, p, p, i64, p, sz, p, C.POINTER(i64), p]
+    lib.eppgcn_compact_back_edge_static.argtypes = [p, p, p, p, i64, p, C.POINTER(i64), p]
+    lib.eppgcn_compact_back_edge_static.restype = i
+    lib.eppgcn_compact_back_edge_static_max_length.restype = i64
     lib.eppgcn_count_nonzero.argtypes = [p, i64, p, C.POINTER(i64), p]
     lib.eppgcn_map_back_part_size.argtypes = [i64, i64, C.POINTER(i)]
     lib.eppgcn_threshold_back_part_size.argtypes = [i64, i64]
@@ -404,6 +413,28 @@ def compact_back_edge(edge_mask, column_index):
     _check(lib.eppgcn_compact_back_edge(_ptr(edge_mask), _ptr(column_index), _ptr(out_id), _ptr(out_edge), length,
                                         _ptr(ws), nbytes, None, C.byref(v), _stream()))
     return out_id, out_edge, int(v.value)
+
+
+def compact_back_edge_static_max_length() -> int:
+    return int(load().eppgcn_compact_back_edge_static_max_length())
+
+
+def compact_back_edge_static(edge_mask, column_index, out_id, out_edge, d_valid_len=None, host_count=True):
+    """The compaction through the library's static device scratch: the call itself allocates
+    nothing, so the caller supplies both output tensors (int32, at least as long as edge_mask).
+    -> valid_len (None with ``host_count=False``: the count then only lands in ``d_valid_len``)."""
+    lib = load()
+    _dev(edge_mask, torch.int32, "edge_mask"); _dev(column_index, torch.int32, "column_index")
+    _dev(out_id, torch.int32, "out_id"); _dev(out_edge, torch.int32, "out_edge")
+    length = edge_mask.numel()
+    if column_index.numel() < length or out_id.numel() < length or out_edge.numel() < length:
+        raise EppgcnError("column_index, out_id and out_edge must be at least as long as edge_mask")
+    if d_valid_len is not None:
+        _dev(d_valid_len, torch.int32, "d_valid_len")
+    v = C.c_int64(0)
+    _check(lib.eppgcn_compact_back_edge_static(_ptr(edge_mask), _ptr(column_index), _ptr(out_id), _ptr(out_edge), length,
+                                               _ptr(d_valid_len), C.byref(v) if host_count else None, _stream()))
+    return int(v.value) if host_count else None
 
 
 def mark_compact(part2node, part_ptr, column_index, src_mask, ngh_mask, node_degs, is_last_layer: bool):

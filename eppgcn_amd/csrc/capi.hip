@@ -35,6 +35,8 @@ size_t split_workspace_bytes(long long);
 int launch_mask_forward(const int*, const int*, const int*, const uint8_t*, uint8_t*, int*, int*, int, long long, int,
                         hipStream_t);
 int launch_compact_mask(const int*, int*, const int*, int*, long long, void*, hipStream_t);
+long long static_compact_max_length();
+int launch_compact_mask_static(const int*, int*, const int*, int*, long long, void**, hipStream_t);
 size_t mark_compact_workspace_bytes(long long);
 int launch_mark_compact(const int*, const int*, const int*, const uint8_t*, uint8_t*, int*, int*, int*, int, long long,
                         int, void*, hipStream_t);
@@ -80,7 +82,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 9; }
+int eppgcn_abi_version(void) { return 10; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -207,6 +209,34 @@ int eppgcn_compact_back_edge(const int32_t* edge_mask, const int32_t* column_ind
     EPPGCN_REQUIRE(length == 0 || (edge_mask && column_index && out_id && out_edge), "null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (int rc = launch_compact_mask(edge_mask, out_id, column_index, out_edge, length, workspace, s)) return rc;
+    ScanState* st = static_cast<ScanState*>(workspace);
+    if (d_valid_len)
+        EPPGCN_HIP(hipMemcpyAsync(d_valid_len, st->counts, sizeof(int), hipMemcpyDeviceToDevice, s));
+    if (h_valid_len) {
+        ScanState host;
+        if (int rc = read_state(workspace, s, &host)) return rc;
+        *h_valid_len = host.counts[0];
+    }
+    return kOk;
+}
+
+int64_t eppgcn_compact_back_edge_static_max_length(void) { return static_compact_max_length(); }
+
+int eppgcn_compact_back_edge_static(const int32_t* edge_mask, const int32_t* column_index, int32_t* out_id,
+                                    int32_t* out_edge, int64_t length, int32_t* d_valid_len, int64_t* h_valid_len,
+                                    void* stream)
+{
+    EPPGCN_REQUIRE(length >= 0, "length must not be negative");
+    if (length > static_compact_max_length()) {
+        set_error("eppgcn_compact_back_edge_static: length " + std::to_string(length) + " exceeds the static scratch (" +
+                  std::to_string(static_compact_max_length()) +
+                  " slots at most); use eppgcn_compact_back_edge with a caller workspace");
+        return kErrCapacity;
+    }
+    EPPGCN_REQUIRE(length == 0 || (edge_mask && column_index && out_id && out_edge), "null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    void* workspace = nullptr;
+    if (int rc = launch_compact_mask_static(edge_mask, out_id, column_index, out_edge, length, &workspace, s)) return rc;
     ScanState* st = static_cast<ScanState*>(workspace);
     if (d_valid_len)
         EPPGCN_HIP(hipMemcpyAsync(d_valid_len, st->counts, sizeof(int), hipMemcpyDeviceToDevice, s));

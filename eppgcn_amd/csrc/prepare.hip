@@ -13,7 +13,17 @@
 // per step, until it meets a tile whose inclusive prefix is known.  Lane ranks
 // inside a wave come from a 64-bit ballot and mbcnt; no block-wide bit-sliced
 // counting and no second pass over the input.
+#include <mutex>
+
 #include "common.hpp"
+
+// Scan scratch of the allocation-free compaction entry point: one ScanState and one 64-bit tile
+// descriptor per 4096-slot tile, for inputs of up to 2^30 slots (2 MiB + 32 bytes per GPU, held
+// until the process ends).  The name is a host-side stand-in; host code only ever uses the device
+// address hipGetSymbolAddress returns for it (static_compact_scratch below).
+constexpr long long kStaticCompactMaxLength = 1ll << 30;
+constexpr size_t kStaticCompactScratchBytes = 32 + 8 * static_cast<size_t>(kStaticCompactMaxLength / 4096);
+static __device__ __align__(256) unsigned char scratch[kStaticCompactScratchBytes];
 
 namespace eppgcn {
 
@@ -697,6 +707,52 @@ int launch_compact_mask(const int* in_id, int* out_id, const int* in_edge, int* 
         EPPGCN_HIP(hipGetLastError());
     }
     return kOk;
+}
+
+// ---- allocation-free compaction: the scan workspace is the file-scope device array `scratch`
+long long static_compact_max_length() { return kStaticCompactMaxLength; }
+
+// Device address of `scratch` on the current device, looked up once per device (every GPU holds
+// its own copy of the array at its own address).
+static int static_compact_scratch(void** out)
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex lock;
+    static void* address[kMaxDevices] = {nullptr};
+    int device = 0;
+    EPPGCN_HIP(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) {
+        set_error("static scratch: device ordinal " + std::to_string(device) + " is outside 0..63");
+        return kErrInvalidArgument;
+    }
+    std::lock_guard<std::mutex> guard(lock);
+    if (!address[device]) {
+        void* p = nullptr;
+        EPPGCN_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p || reinterpret_cast<uintptr_t>(p) % 8 != 0) {
+            set_error("static scratch: hipGetSymbolAddress returned an unusable address");
+            return kErrHip;
+        }
+        address[device] = p;
+    }
+    *out = address[device];
+    return kOk;
+}
+
+// compact_mask_kernel over the static scratch; *workspace_out receives the scratch address (its
+// ScanState holds the kept length once the stream has run).  The scan state and the descriptors of
+// the tiles this call uses are cleared by init_scan's fill kernel on every call: the array keeps
+// the previous call's contents.
+int launch_compact_mask_static(const int* in_id, int* out_id, const int* in_edge, int* out_edge, long long length,
+                               void** workspace_out, hipStream_t stream)
+{
+    static_assert(kStaticCompactMaxLength % kCompactTile == 0 &&
+                      kStaticCompactScratchBytes == sizeof(ScanState) + 8 * (kStaticCompactMaxLength / kCompactTile),
+                  "the static scratch holds the scan state and one descriptor per tile");
+    void* ws = nullptr;
+    if (int rc = static_compact_scratch(&ws)) return rc;
+    *workspace_out = ws;
+    return launch_compact_mask(in_id, out_id, in_edge, out_edge, length, ws, stream);
 }
 
 size_t mark_compact_workspace_bytes(long long length)

@@ -186,6 +186,25 @@ int eppgcn_compact_back_edge(const int32_t* edge_mask, const int32_t* column_ind
                              void* workspace, size_t workspace_bytes,
                              int32_t* d_valid_len, int64_t* h_valid_len, void* stream);
 
+/* eppgcn_compact_back_edge for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): same inputs, outputs and results,
+ * but the scan scratch is a static device array inside the library instead of a caller workspace,
+ * and the call allocates nothing (no hipMalloc / hipFree, no allocating library routine).  No
+ * counterpart in the reference, whose compactor allocates and frees its scratch on every call
+ * (cuCompactor.cu:328-465).
+ *   - length may be at most eppgcn_compact_back_edge_static_max_length() = 2^30 slots; a longer
+ *     input fails with EPPGCN_ERR_CAPACITY and a message, before any device work.
+ *   - The array (2 MiB + 32 bytes) exists once per GPU the library runs on, for the life of the
+ *     process; its address on a device is looked up on the first call there (the device that is
+ *     current at the call).
+ *   - Every call on a GPU uses that GPU's one array (it is cleared at the start of each call), so
+ *     calls that overlap on one GPU - on different streams or from different threads - race and
+ *     must be serialised by the caller. */
+int64_t eppgcn_compact_back_edge_static_max_length(void);
+int eppgcn_compact_back_edge_static(const int32_t* edge_mask, const int32_t* column_index,
+                                    int32_t* out_id, int32_t* out_edge, int64_t length,
+                                    int32_t* d_valid_len, int64_t* h_valid_len, void* stream);
+
 /* Path marking and compaction of one layer in one pass over the slots: exactly the results of
  * eppgcn_mask_forward on a -1-filled edge mask followed by eppgcn_compact_back_edge (ngh_mask and
  * node_degs updated in place, out_id / out_edge with zero tails, V at d_valid_len / h_valid_len),

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared_functions():
         assert hasattr(lib, name), f"{name} is declared in include/eppgcn_hip.h but not exported"
     assert sorted(capi.EXPORTS) == declared_functions()
-    assert capi.load().eppgcn_abi_version() == 9
+    assert capi.load().eppgcn_abi_version() == capi.ABI_VERSION
 
 
 def test_host_only_heuristics_match_the_checker():
@@ -115,5 +115,5 @@ def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
     env = dict(os.environ, LD_LIBRARY_PATH="/opt/rocm/lib:" + os.environ.get("LD_LIBRARY_PATH", ""))
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True, env=env).stdout.split("\n")
     from oracle import c_oracle as co
-    assert out[0].split() == ["9", "32", "320", str(max(1, co.map_back_part_size(1000, 5000))), "0", "-1"]
+    assert out[0].split() == [str(capi.ABI_VERSION), "32", "320", str(max(1, co.map_back_part_size(1000, 5000))), "0", "-1"]
     assert "dim > 0" in out[1]
