@@ -5,7 +5,8 @@ compaction, split), pruned backward time, unpruned backward time, algorithmic GB
     python -m eppgcn_amd.sweep [--config cfg3_rmat20] [--ratios 0.01 0.1 0.5]
                                [--widths 16 64 256] [--groups 8 16 32 64] [--reps 5]
 
-Prints one JSON line per cell and a final summary line.  Needs the MI355X.  Launches are set up
+Every cell is checked before it is reported (pruned against unpruned backward within 2e-5 of the
+absolute sum); a disagreement ends the sweep.  Prints one JSON line per cell and a final summary line.  Needs the MI355X.  Launches are set up
 the way the extension module sets them up by itself: execution plans where the feature table has 4 MB
 or more (column-blocked for the forward groups and for paths that keep at least half of the edges,
 one block otherwise) and the gathered-rows bitmap for paths that read fewer than half of the rows;
@@ -101,6 +102,18 @@ def main():
                 unpruned_ms = capi.get_time_ms(1) / args.reps
                 capi.set_timing(False)
                 capi.clear_time()
+                # a timed cell is a checked cell: `out` holds the unpruned result; the pruned one sums the same
+                # terms in another order, so they agree within 2e-5 * sum |w x| (the yardstick comes from the
+                # same operator applied to |dy|)
+                pruned_out = capi.ours_backward(dy, ids, part_pointer, edge_list, g.degrees, num_parts, gs, 1, 4, 16, None,
+                                                ws, plan=plan, gathered_rows=gathered)
+                yardstick = capi.spmm_forward(dy.abs(), g.column_index, g.degrees, part_ptr, part2node, ps, 32, 8, None,
+                                              None, True, ws, plan=forward_plan(width))
+                worst = float(((pruned_out - out).abs() / (2e-5 * yardstick + 1e-30)).max())
+                if not worst <= 1.0:
+                    raise SystemExit(f"sweep: pruned and unpruned backward disagree at ratio {ratio}, width {width}, "
+                                     f"group size {gs}: max err / limit = {worst:.3f}")
+                del pruned_out, yardstick
                 nbytes = workload.bytes_pruned_backward(n, valid_len, num_parts, width)
                 del plan
                 cell = {"config": args.config, "ratio": ratio, "width": width, "group_size": gs,
@@ -109,7 +122,8 @@ def main():
                         "pruned_bwd_ms": round(pruned_ms, 4), "unpruned_bwd_ms": round(unpruned_ms, 4),
                         "pruned_GBps": round(nbytes / pruned_ms / 1e6, 1),
                         "unpruned_GBps": round(workload.bytes_forward(n, e, width) / unpruned_ms / 1e6, 1),
-                        "speedup": round(unpruned_ms / pruned_ms, 2)}
+                        "speedup": round(unpruned_ms / pruned_ms, 2),
+                        "pruned_vs_unpruned_err_over_limit": round(worst, 4)}
                 cells.append(cell)
                 print(json.dumps(cell), flush=True)
     best = {}
