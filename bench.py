@@ -7,9 +7,19 @@ at width 22 (last layer) and 16 (first layer), launched back to back through the
 every input resident in HBM.  The dense X*W products are not part of the metric.
 
 Prints ONE JSON line:  metric = the headline metric below, value = algorithmic GB/s of the epoch's
-aggregation, ms_per_step = aggregation ms per epoch, plus `roofline` for the dominant kernel
-(HIP-event time of the kernel alone) and `cpu_baseline` (the CPU checker's OpenMP restatement
-timed on the host cores on one epoch of the same workload).
+aggregation (gather-model bytes / time: every walked edge is priced as if its row came from HBM, so
+cache reuse shows up as a figure above what the memory system physically moved), ms_per_step =
+aggregation ms per epoch, plus `roofline` for the dominant launch and `cpu_baseline` (the CPU
+checker's OpenMP restatement timed on the host cores on one epoch of the same workload).
+
+`roofline` prices the dominant *call*: output clear + pre-scaling pass + aggregation kernel, i.e. all
+the work its algorithmic bytes are charged for, timed with HIP events on the launch stream
+(`call_ms`; the three parts are also timed apart by the library's own events).  `kernel_only_frac`
+is the aggregation kernel alone; `hbm_frac` is the HBM traffic rocprofv3 measured for the same call
+(committed summary under profiles/, used only while the kernel sources still hash to what was
+profiled) over the same time; `compulsory_frac` is the lower bound with perfect reuse over it.
+Before anything is timed every launch is checked against the same operator without plan and
+workspace (different kernel instantiation, different summation order).
 """
 from __future__ import annotations
 
@@ -55,6 +65,11 @@ def parse():
     ap.add_argument("--train_epochs", type=int, default=100)
     ap.add_argument("--copy_probe", action="store_true",
                     help="also launch a plain 1 GiB device copy 3 times (calibrates byte counters under rocprofv3)")
+    ap.add_argument("--gather_probe", action="store_true",
+                    help="also run the aggregation kernel 3 times each over permutation graphs with 64- and 128-byte "
+                         "rows: every row of a 2^22-row table is gathered exactly once, so the bytes read are known "
+                         "(calibrates FETCH_SIZE for row gathers under rocprofv3)")
+    ap.add_argument("--no_check", action="store_true", help="skip the result check of the timed launches")
     ap.add_argument("--verbose", action="store_true")
     return ap.parse_args()
 
@@ -198,6 +213,8 @@ def main():
         for _, fn, _ in kernels:
             fn()
 
+    checked = None if args.no_check else check_launches(g, wl, kernels, (x16, x22, dy22, dy16), (out16, out22))
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -209,21 +226,27 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     value = bytes_epoch / (ms_per_step * 1e-3) / 1e9
 
-    # per-kernel time: the library's own HIP events on the launch stream, around the
-    # aggregation kernel alone (the output clear is outside the bracket)
-    capi.set_timing(True)
+    # per launch: the whole call (output clear + pre-scaling pass + aggregation kernel) between two HIP
+    # events on the launch stream, calls issued back to back; and, from the library's own events on the
+    # same stream, the three parts apart (with those enabled every part is followed by a host wait,
+    # so they are taken in a pass of their own)
     per_kernel = {}
     reps = max(3, min(args.steps, 10))
     for name, fn, nbytes in kernels:
+        call_ms = _event_ms(fn, reps)
         which = 0 if name.startswith("fwd") else 1
+        capi.set_timing(True)
         capi.clear_time()
         for _ in range(reps):
             fn()
-        ms = capi.get_time_ms(which) / reps
-        per_kernel[name] = {"ms": round(ms, 4), "alg_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1),
-                            "pct_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS * 100, 2)}
-    capi.set_timing(False)
-    capi.clear_time()
+        ms, clear_ms, scale_ms = (capi.get_time_ms(w) / reps for w in (which, 3, 4))
+        capi.set_timing(False)
+        capi.clear_time()
+        per_kernel[name] = {"call_ms": round(call_ms, 4), "kernel_ms": round(ms, 4), "clear_ms": round(clear_ms, 4),
+                            "prescale_ms": round(scale_ms, 4), "alg_bytes": nbytes,
+                            "alg_GBps": round(nbytes / call_ms / 1e6, 1),
+                            "pct_peak": round(nbytes / call_ms / 1e6 / PEAK_HBM_GBS * 100, 2),
+                            "kernel_only_pct_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS * 100, 2)}
     if args.copy_probe:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
@@ -231,11 +254,25 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    dominant = max(per_kernel, key=lambda k: per_kernel[k]["ms"])
+    if args.gather_probe:
+        gather_probe(dev)
+    dominant = max(per_kernel, key=lambda k: per_kernel[k]["call_ms"])
     dk = per_kernel[dominant]
-    roofline = {"bound": "hbm", "kernel": dominant, "achieved": dk["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": round(dk["GBps"] / PEAK_HBM_GBS, 4), "traffic": measured_traffic(args.config, dominant),
-                "kernel_ms": dk["ms"], "alg_bytes_per_launch": dk["alg_bytes"]}
+    dim = 22 if "d22" in dominant else 16
+    compulsory = workload.bytes_compulsory(n, e, dim)
+    traffic, traffic_note = measured_traffic(args.config, dominant)
+    sec = dk["call_ms"] * 1e-3
+    roofline = {"bound": "hbm", "kernel": dominant,
+                "launch": "whole call: output clear + pre-scaling pass + aggregation kernel",
+                "achieved": dk["alg_GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(dk["alg_GBps"] / PEAK_HBM_GBS, 4), "traffic": traffic, "traffic_source": traffic_note,
+                "achieved_is": "algorithmic (gather-model) bytes / call time; rows served from cache count as moved",
+                "call_ms": dk["call_ms"], "kernel_ms": dk["kernel_ms"], "clear_ms": dk["clear_ms"],
+                "prescale_ms": dk["prescale_ms"], "alg_bytes_per_launch": dk["alg_bytes"],
+                "kernel_only_frac": round(dk["alg_bytes"] / (dk["kernel_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                "hbm_frac": None if traffic is None else round(traffic / sec / 1e9 / PEAK_HBM_GBS, 4),
+                "compulsory_bytes": compulsory,
+                "compulsory_frac": round(compulsory / sec / 1e9 / PEAK_HBM_GBS, 4)}
 
     result = {
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -251,9 +288,16 @@ def main():
                    "column_blocked_plan": bool(wl.plans)},
         "agg_ms_per_epoch": round(ms_per_step, 4), "alg_bytes_per_epoch": bytes_epoch,
         "pct_of_peak_hbm": round(value / PEAK_HBM_GBS * 100, 2),
+        "value_is": "algorithmic (gather-model) bytes of the epoch / wall time; not measured HBM traffic",
         "per_kernel": per_kernel, "path_preparation_s": round(prep_s, 3),
+        "result_check": checked,
         "roofline": roofline,
     }
+    traffic_epoch = [measured_traffic(args.config, k)[0] for k in per_kernel]
+    if all(t is not None for t in traffic_epoch):
+        result["measured_hbm_bytes_per_epoch"] = sum(traffic_epoch)
+        result["measured_hbm_GBps"] = round(sum(traffic_epoch) / (ms_per_step * 1e-3) / 1e9, 1)
+        result["measured_hbm_pct_of_peak"] = round(result["measured_hbm_GBps"] / PEAK_HBM_GBS * 100, 2)
 
     # the same epoch as the training pipeline issues it: the forward tables arrive scaled and padded
     # from the dense update (built outside the timed region here), so only the backward launches
@@ -279,17 +323,99 @@ def main():
     print(json.dumps(result), flush=True)
 
 
+PROFILED_SOURCES = ("aggregate.hip", "common.hpp", "schedule.hip", "prepare.hip")
+
+
+def kernel_source_hash():
+    """sha256 (first 16 hex digits) over the sources that decide what an aggregation call moves: the
+    kernels, the plan builder and the clear kernels.  A counter summary under profiles/ names the
+    hash it was taken with."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in PROFILED_SOURCES:
+        with open(os.path.join(ROOT, "eppgcn_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def measured_traffic(config, kernel):
-    """HBM bytes per launch of `kernel` from the committed rocprofv3 counter summary (FETCH_SIZE +
-    WRITE_SIZE of the same bench command), or None when no summary covers this workload."""
+    """(HBM bytes per call of `kernel`, where they come from) from the committed rocprofv3 counter
+    summary of the same bench command: calibrated FETCH_SIZE + WRITE_SIZE of the call's kernels.
+    (None, reason) when no summary covers this workload or the kernel sources have changed since it
+    was taken - a stale counter must not pose as a measurement."""
     import glob
     import re
-    for path in glob.glob(os.path.join(ROOT, "profiles", "*.md")):
-        m = re.search(r"traffic_bytes %s %s = ([0-9.e+]+)" % (re.escape(config), re.escape(kernel)),
-                      open(path).read())
-        if m:
-            return float(m.group(1))
-    return None
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
+        text = open(path).read()
+        m = re.search(r"traffic_bytes %s %s = ([0-9.e+]+)" % (re.escape(config), re.escape(kernel)), text)
+        if not m:
+            continue
+        h = re.search(r"kernel_source_sha256 = ([0-9a-f]+)", text)
+        rel = os.path.relpath(path, ROOT)
+        if not h or h.group(1) != kernel_source_hash():
+            return None, f"{rel} was taken from other kernel sources ({h.group(1) if h else 'no hash'} != {kernel_source_hash()})"
+        return float(m.group(1)), rel
+    return None, "no counter summary under profiles/ covers this workload"
+
+
+def gather_probe(dev):
+    """Aggregation over a permutation graph: row r gathers exactly row perm[r] of a 2^22-row table that
+    arrives pre-scaled, so one launch reads every table row once (64-byte rows at width 16, 128-byte
+    rows at width 32) plus 16 bytes of indices and scale per row, and writes the output once.  Under
+    rocprofv3 --pmc these launches (the only ones over `ForwardGroups` at these widths) give the
+    factor between FETCH_SIZE and the bytes a row gather really moves."""
+    import torch
+    from eppgcn_amd import capi
+    n = 1 << 22
+    gen = torch.Generator(device=dev).manual_seed(5)
+    col = torch.randperm(n, device=dev, generator=gen).int()
+    part_ptr = torch.arange(n + 1, dtype=torch.int32, device=dev)
+    part2node = torch.arange(n, dtype=torch.int32, device=dev)
+    ones = torch.ones(n, device=dev)
+    for dim in (16, 32):
+        table = torch.empty(n, capi.feature_workspace_pitch(dim), device=dev).normal_()
+        out = torch.empty(n, dim, device=dev)
+        for _ in range(3):
+            capi.spmm_forward(None, col, ones, part_ptr, part2node, 1, 32, 8, None, out, workspace=table.view(-1),
+                              prescaled_dim=dim)
+        torch.cuda.synchronize()
+        assert torch.equal(out, table[col.long()][:, :dim])
+        del table, out
+
+
+def check_launches(g, wl, kernels, inputs, outputs):
+    """Every timed launch (plan + feature workspace + gathered-rows bitmap) against the same operator
+    without plan and workspace - another kernel instantiation, per-edge scale gather, CSR order - within
+    2e-5 * sum |w x| per element (the yardstick is the operator applied to |x|).  Raises on a mismatch:
+    a number must never be printed for a kernel whose results are off."""
+    import torch
+    from eppgcn_amd import capi
+    x16, x22, dy22, dy16 = inputs
+    out16, out22 = outputs
+    fwd = lambda x: capi.spmm_forward(x, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 32, 8,
+                                      g.row_pointers, None, workspace=None)
+    p_last, p_first = wl.paths[1], wl.paths[0]
+    bwd = lambda dy, p: capi.ours_backward(dy, p.ids, p.part_pointer, p.edge_list, g.degrees, p.num_parts, p.part_size,
+                                           p.layer, 4, 16, None, workspace=None)
+    plain = {"fwd_agg_d16": lambda: fwd(x16), "fwd_agg_d22": lambda: fwd(x22),
+             "bwd_agg_d22_last": lambda: bwd(dy22, p_last), "bwd_agg_d16_first": lambda: bwd(dy16, p_first)}
+    source = {"fwd_agg_d16": (x16, out16), "fwd_agg_d22": (x22, out22), "bwd_agg_d22_last": (dy22, out22),
+              "bwd_agg_d16_first": (dy16, out16)}
+    worst = {}
+    for name, fn, _ in kernels:
+        x, out = source[name]
+        out.fill_(float("nan"))
+        fn()
+        want = plain[name]()
+        yardstick = fwd(x.abs())
+        ratio = float(((out - want).abs() / (2e-5 * yardstick + 1e-30)).max())
+        if not ratio <= 1.0:
+            raise SystemExit(f"bench.py: {name} differs from the unplanned, unscaled operator: "
+                             f"max err / (2e-5 * sum|w x|) = {ratio:.3f}")
+        worst[name] = round(ratio, 4)
+        del want, yardstick
+    return {"against": "same operator without plan and workspace", "tolerance": "2e-5 * sum|w x| per element",
+            "max_err_over_tolerance": worst}
 
 
 def cpu_baseline(args, g, wl, x16, x22, dy22, dy16, bytes_epoch):

@@ -27,9 +27,10 @@ EXPORTS = [
     "eppgcn_mark_compact_workspace_bytes", "eppgcn_mark_compact", "eppgcn_set_plan_length_classes",
     "eppgcn_mark_gathered_rows", "eppgcn_set_wide_index", "eppgcn_wave64_back_part_size",
     "eppgcn_compact_back_edge_static", "eppgcn_compact_back_edge_static_max_length",
+    "eppgcn_auto_back_part_size", "eppgcn_scan_status", "eppgcn_build_plan_status",
 ]
 
-ABI_VERSION = 10      # what eppgcn_abi_version() of a matching library returns
+ABI_VERSION = 11      # what eppgcn_abi_version() of a matching library returns
 
 _lib = None
 
@@ -82,6 +83,12 @@ def load():
     lib.eppgcn_threshold_back_part_size.argtypes = [i64, i64]
     lib.eppgcn_wave64_back_part_size.argtypes = [i64, i64]
     lib.eppgcn_wave64_back_part_size.restype = i
+    lib.eppgcn_auto_back_part_size.argtypes = [i64, i64, C.POINTER(i)]
+    lib.eppgcn_auto_back_part_size.restype = i
+    lib.eppgcn_scan_status.argtypes = [p, p]
+    lib.eppgcn_scan_status.restype = i
+    lib.eppgcn_build_plan_status.argtypes = [p, i, p]
+    lib.eppgcn_build_plan_status.restype = i
     lib.eppgcn_split_back_part.argtypes = [p, i, i, p, i64, p, sz, p, C.POINTER(i64), C.POINTER(i64), p]
     lib.eppgcn_build_part.argtypes = [p, i, i, p, p, i64, p, sz, p, C.POINTER(i64), p]
     lib.eppgcn_get_ginfo.argtypes = [p, i64, i64, p, C.POINTER(C.c_float), p]
@@ -295,7 +302,8 @@ def build_plan(part_ptr, column_index, num_parts: int, num_slots: int, num_nodes
     _check(lib.eppgcn_build_plan(_ptr(part_ptr), _ptr(column_index), _ptr(part2node), _ptr(ids), int(num_parts),
                                  int(num_slots), int(num_nodes), int(dim), int(block_shift), C.c_void_p(base), nbytes,
                                  C.c_void_p(wbase), wbytes, _stream()))
-    torch.cuda.current_stream().synchronize()      # the workspace is released on return
+    # synchronises (the workspace is released on return) and refuses a plan whose scan stalled
+    _check(lib.eppgcn_build_plan_status(C.c_void_p(wbase), int(num_parts), _stream()))
     return Plan(buf, base, int(num_parts), int(num_slots), int(num_nodes))
 
 
@@ -484,6 +492,19 @@ def threshold_back_part_size(valid_node: int, valid_len: int) -> int:
 def wave64_back_part_size(valid_node: int, valid_len: int) -> int:
     """The group-size rule re-fitted for this library's kernels (16 or 32)."""
     return int(load().eppgcn_wave64_back_part_size(int(valid_node), int(valid_len)))
+
+
+def auto_back_part_size(valid_node: int, valid_len: int):
+    """The reference's `map` mode made safe for large paths -> (group size, fell_back): the fitted
+    regression while it gives at least 1, the wave64 rule otherwise."""
+    c = C.c_int(0)
+    ps = load().eppgcn_auto_back_part_size(int(valid_node), int(valid_len), C.byref(c))
+    return int(ps), bool(c.value)
+
+
+def scan_status(workspace) -> None:
+    """Raises if the last scan-based call over ``workspace`` stalled or overflowed (synchronises)."""
+    _check(load().eppgcn_scan_status(_ptr(workspace), _stream()))
 
 
 def split_back_part(node_deg, num_edges: int, part_size: int):

@@ -724,17 +724,22 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
     int ld_in = dim;
     // rows the kernel writes with one plain store (a plan knows them) need no clearing; with fewer
     // groups than half the rows most rows have no group at all and the plain fill is the faster clear
-    if (single_rows && 2ll * num_parts >= num_nodes) {
-        if (int rc = launch_zero_rows_unless(out, single_rows, num_nodes, dim, stream)) return rc;
-    } else {
-        if (int rc = launch_zero_words(out, static_cast<size_t>(num_nodes) * dim, stream)) return rc;
+    {
+        KernelTimer timer(stream, phase_sink(0));
+        if (single_rows && 2ll * num_parts >= num_nodes) {
+            if (int rc = launch_zero_rows_unless(out, single_rows, num_nodes, dim, stream)) return rc;
+        } else {
+            if (int rc = launch_zero_words(out, static_cast<size_t>(num_nodes) * dim, stream)) return rc;
+        }
     }
     if (num_parts == 0) return kOk;
     if (prescaled) {
         // in == nullptr: the caller (the dense update) already wrote the scaled, padded rows
         ld_in = workspace == in ? dim : workspace_pitch(dim);
-        if (in)
+        if (in) {
+            KernelTimer timer(stream, phase_sink(1));
             if (int rc = launch_scale_rows(workspace, in, scale, gathered_rows, num_nodes, dim, ld_in, stream)) return rc;
+        }
         in = workspace;
     }
     KernelTimer timer(stream, sink, sink2);   // brackets the aggregation kernel alone

@@ -16,6 +16,7 @@ int aggregate_forward_groups(float*, const float*, const int*, const float*, con
 int aggregate_compacted_groups(float*, const float*, const int*, const int*, const int*, const float*, const void*,
                                int, int, int, int, float*, const uint32_t*, hipStream_t, double*, double*);
 size_t plan_workspace_bytes(long long);
+size_t plan_scan_state_offset(long long);
 int schedule_shift(int);
 void set_schedule_shift(int);
 void set_plan_keep_rows(int);
@@ -60,7 +61,10 @@ static bool g_timing = false;
 static double g_for_agg_ms = 0.0, g_back_agg_ms = 0.0, g_mask_ms = 0.0;
 static double g_layer_back_ms[kMaxTimedLayers] = {0};
 
+static double g_phase_ms[2] = {0.0, 0.0};       // output clears, pre-scaling passes of the aggregation calls
+
 bool timing_enabled() { return g_timing; }
+double* phase_sink(int which) { return &g_phase_ms[which & 1]; }
 
 static int read_state(void* workspace, hipStream_t stream, ScanState* host)
 {
@@ -82,7 +86,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 10; }
+int eppgcn_abi_version(void) { return 11; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -351,6 +355,37 @@ int eppgcn_wave64_back_part_size(int64_t valid_node, int64_t valid_len)
     return valid_len / valid_node < 24 ? 16 : 32;
 }
 
+int eppgcn_auto_back_part_size(int64_t valid_node, int64_t valid_len, int* fell_back)
+{
+    int clamped = 0;
+    const int fitted = eppgcn_map_back_part_size(valid_node, valid_len, &clamped);
+    if (fell_back) *fell_back = clamped;
+    return clamped ? eppgcn_wave64_back_part_size(valid_node, valid_len) : fitted;
+}
+
+int eppgcn_scan_status(const void* workspace, void* stream)
+{
+    EPPGCN_REQUIRE(workspace && aligned(workspace, 8), "workspace must be 8-byte aligned");
+    ScanState host;
+    if (int rc = read_state(const_cast<void*>(workspace), static_cast<hipStream_t>(stream), &host)) return rc;
+    if (host.overflow) {
+        set_error("group pointers did not fit the given capacity (need " + std::to_string(host.counts[0] + 1) +
+                  " entries)");
+        return kErrCapacity;
+    }
+    return kOk;
+}
+
+int eppgcn_build_plan_status(const void* workspace, int num_parts, void* stream)
+{
+    EPPGCN_REQUIRE(num_parts >= 0, "negative size");
+    if (num_parts == 0) return kOk;
+    EPPGCN_REQUIRE(workspace && aligned(workspace, 256), "workspace must be 256-byte aligned");
+    ScanState host;
+    return read_state(static_cast<char*>(const_cast<void*>(workspace)) + plan_scan_state_offset(num_parts),
+                      static_cast<hipStream_t>(stream), &host);
+}
+
 static int finish_split(void* workspace, hipStream_t s, int32_t* d_counts, int64_t* h_a, int64_t* h_b)
 {
     ScanState* st = static_cast<ScanState*>(workspace);
@@ -439,6 +474,7 @@ void eppgcn_clear_time(void)
     g_for_agg_ms = 0.0;
     g_back_agg_ms = 0.0;
     for (double& v : g_layer_back_ms) v = 0.0;
+    g_phase_ms[0] = g_phase_ms[1] = 0.0;
 }
 
 double eppgcn_get_time_ms(int which)
@@ -446,6 +482,7 @@ double eppgcn_get_time_ms(int which)
     if (which == 0) return g_for_agg_ms;
     if (which == 1) return g_back_agg_ms;
     if (which == 2) return g_mask_ms;
+    if (which == 3 || which == 4) return g_phase_ms[which - 3];
     if (which > 100 && which <= 100 + kMaxTimedLayers) return g_layer_back_ms[which - 101];
     return -1.0;
 }

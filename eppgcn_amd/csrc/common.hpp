@@ -96,6 +96,9 @@ inline PlanView plan_view(void* plan, long long num_parts, long long num_nodes)
 // asynchronous).  When enabled the destructor synchronises on the stop event and
 // adds the elapsed milliseconds to the sinks.
 bool timing_enabled();
+// Accumulators (ms) of the passes an aggregation call runs before its kernel: 0 = output clear,
+// 1 = pre-scaling of the input into the feature workspace.
+double* phase_sink(int which);
 struct KernelTimer {
     hipStream_t stream;
     double* sink;

@@ -15,7 +15,9 @@
 //     exact for any edge count;
 //   - split_back_part's part_pointer has num_edges + 1 entries, so the terminator
 //     is always in bounds;
-//   - get_map_back_part_size never returns less than 1;
+//   - get_map_back_part_size never returns less than 1: where the fitted regression drops below 1
+//     (large paths) it returns the group size of the rule fitted for the wave64 kernels;
+//   - get_ginfo also accepts a CPU tensor, as the reference's host loop does;
 //   - the module keeps, per group array it has seen, a column-blocked execution plan for the
 //     aggregation kernels (built on first use, about 4 bytes per edge, the 8 most recently used
 //     kept); it affects speed only.
@@ -77,6 +79,11 @@ Tensor workspace(size_t bytes, const Tensor& like)
 // training run passes unchanged every epoch.  Entries are keyed by storage address, length,
 // tensor version and block-size class, and hold references to the key tensors so that an
 // address cannot be reused for other data while its entry lives.
+// Staleness rule: an entry is invalidated by writes that bump torch's version counter (ordinary
+// in-place tensor operations).  A writer that bypasses the counter - `.data` / detach() in-place
+// operations, a raw-pointer kernel of another extension, this library's own C ABI writing into the
+// same storage - leaves the cached plan describing the old groups; after such a write call
+// clear_plans() before the next layer operation.
 struct PlanEntry {
     const void* part_ptr;
     const void* col;
@@ -136,6 +143,8 @@ const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& ro
                             is_forward ? nullptr : rows.data_ptr<int32_t>(), static_cast<int>(num_parts), num_slots,
                             num_nodes, dim_of_class(dc), block_shift, base, bytes, wbase, wbytes, stream_of(part_ptr)),
           "build_plan");
+    // once per group array: wait for the build and refuse a plan whose look-back scan stalled
+    check(eppgcn_build_plan_status(wbase, static_cast<int>(num_parts), stream_of(part_ptr)), "build_plan");
     g_plans.push_front(std::move(e));
     if (g_plans.size() > kMaxPlans) g_plans.pop_back();
     return g_plans.front().plan_ptr;
@@ -484,11 +493,11 @@ std::vector<Tensor> mark_compact(Tensor id, Tensor partPointer, Tensor edgeList,
 
 int get_map_back_part_size(Tensor node_deg, int valid_len)
 {
-    int clamped = 0;
-    const int ps = eppgcn_map_back_part_size(valid_nodes(node_deg), valid_len, &clamped);
-    if (clamped)
-        TORCH_WARN_ONCE("get_map_back_part_size: the fitted regression gives a group size below 1 for this graph; "
-                        "using 1 (pass a constant group size instead)");
+    int fell_back = 0;
+    const int ps = eppgcn_auto_back_part_size(valid_nodes(node_deg), valid_len, &fell_back);
+    if (fell_back)
+        TORCH_WARN_ONCE("get_map_back_part_size: the fitted regression gives a group size below 1 for this path (it "
+                        "was fitted on small graphs); using the rule fitted for the wave64 kernels instead: ", ps);
     return ps;
 }
 
@@ -525,6 +534,10 @@ std::vector<Tensor> build_back_part(Tensor edge_mask, Tensor column_index, Tenso
 
 Tensor get_ginfo(Tensor node_deg, int valid_len)
 {
+    // the reference reads node_deg on the host (EPPGCN.cpp:351-386) and its caller passes a CPU tensor
+    TORCH_CHECK(node_deg.scalar_type() == torch::kInt32, "node_deg must be int32");
+    if (!node_deg.is_cuda()) node_deg = node_deg.to(torch::kCUDA);
+    node_deg = node_deg.contiguous();
     CHECK_I32(node_deg);
     auto hist = torch::empty({10}, node_deg.options());
     auto re = torch::zeros({10}, torch::kFloat32);

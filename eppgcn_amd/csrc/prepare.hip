@@ -416,10 +416,11 @@ __global__ __launch_bounds__(256) void ginfo_hist_kernel(const int* __restrict__
 // Vertex i with g_i slots (g_i = kept degree, or CSR degree) yields q_i = ceil(g_i/ps)
 // groups; group j of vertex i starts at G_i + j*ps where G_i is the exclusive sum
 // of g.  One look-back scan carries (sum q, sum g) packed as q*2^31 + g.  The
-// tile's groups are then written by all threads together: output slot o finds its
-// vertex by binary search over the tile's q offsets in LDS, so a hub vertex with
-// a hundred thousand groups costs its tile a longer loop, not one thread a longer
-// life.
+// tile's groups are then written in two ways: a vertex with at most kSmallGroups
+// groups by the thread that owns it, every other vertex - collected on a list in
+// LDS - by a whole wave, 64 groups per step with coalesced stores, so a hub vertex
+// with a hundred thousand groups costs its tile a longer loop, not one thread a
+// longer life.
 constexpr int kSplitBlock = 256;
 constexpr int kSplitItems = 8;
 constexpr int kSplitTile = kSplitBlock * kSplitItems;

@@ -196,6 +196,12 @@ size_t plan_workspace_bytes(long long num_parts)
            align256(temp) + 256;
 }
 
+// where launch_build_plan keeps the state of its look-back scan inside the workspace
+size_t plan_scan_state_offset(long long num_parts)
+{
+    return 5 * align256(sizeof(int) * (static_cast<size_t>(num_parts > 0 ? num_parts : 0) + 1));
+}
+
 int workspace_pitch(int dim);   // aggregate.hip
 
 static int g_force_shift = 0;
@@ -246,7 +252,7 @@ int launch_build_plan(const int* part_ptr, const int* col, const int* part2node,
     int* iota = reinterpret_cast<int*>(base + 2 * slab);
     int* order = reinterpret_cast<int*>(base + 3 * slab);
     int* sizes = reinterpret_cast<int*>(base + 4 * slab);
-    ScanState* st = reinterpret_cast<ScanState*>(base + 5 * slab);
+    ScanState* st = reinterpret_cast<ScanState*>(base + plan_scan_state_offset(num_parts));
     uint64_t* desc = reinterpret_cast<uint64_t*>(st + 1);
     void* temp = base + 5 * slab + scan_state_bytes(num_parts);
     int bits = 1;

@@ -94,8 +94,11 @@ class custom_dataset(torch.nn.Module):
         self.avg_edgeSpan = float(np.mean(np.abs(src - dst))) if src.size else 0.0
         self.row_pointers, self.column_index = csr_from_directed_pairs(
             torch.from_numpy(src).to(device), torch.from_numpy(dst).to(device), n)
-        self.num_edges = int(self.column_index.numel())
-        self.avg_degree = self.num_edges / max(1, n)
+        self.num_edges = int(self.column_index.numel())     # CSR entries (the reference: input lines)
+        self.raw_num_edges = int(src.size)
+        # the decider's automatic group size reads avg_degree, which the reference computes from the
+        # number of input lines, repeated pairs included (EPPGCN/dataset.py:73,100)
+        self.avg_degree = self.raw_num_edges / max(1, n)
         self.degrees = graphs.scale_vector(self.row_pointers, scale_mode)
         if verbose:
             print(f"# nodes: {n}\n# avg_degree: {self.avg_degree:.2f}\n# avg_edgeSpan: {int(self.avg_edgeSpan)}")

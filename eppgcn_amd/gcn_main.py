@@ -112,7 +112,9 @@ def _single_spmm(tr, epochs, verify):
     return True
 
 
-def main(argv=None) -> int:
+def main(argv=None, report: dict = None) -> int:
+    """``report``: a dict that receives the figures of the run (the printed lines as numbers), for
+    callers that run several configurations in one process."""
     args = build_parser().parse_args(argv)
     print("||" + args.dataset + "   " + str(args.train_ratio) + "   " + str(args.layers))
     if args.backsize_mode == "net":
@@ -142,6 +144,8 @@ def main(argv=None) -> int:
         print()
         return 0
     res = tr.run(args.num_epoches, warmup=10, kernel_timing=args.kernel_timers == "True")
+    if report is not None:
+        report.update(res, num_nodes=ds.num_nodes, num_edges=ds.num_edges, forward_group_size=tr.inputInfo.partSize)
     tr.GNNA.print_time()
     for key in ("for_time", "loss_time", "back_time", "build_time"):
         print("{}: {:.6f}".format(key, res[key]))

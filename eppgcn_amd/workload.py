@@ -48,13 +48,13 @@ class Workload:
 
 
 def choose_back_part_size(mode: str, constant: int, valid_node: int, valid_len: int) -> int:
-    """Backward group size: 'constant', 'map' (fitted regression, EPPGCN/GCNConv/EPPGCN.cpp:298-325,
-    clamped to >= 1), 'threshold' (legacy rule of build_back_part, :246-258) or 'wave64' (the rule
+    """Backward group size: 'constant', 'map' (fitted regression, EPPGCN/GCNConv/EPPGCN.cpp:298-325;
+    the wave64 rule where the regression drops below 1), 'threshold' (legacy rule of build_back_part, :246-258) or 'wave64' (the rule
     re-fitted for this library's kernels)."""
     if mode == "constant":
         return max(1, int(constant))
     if mode == "map":
-        return capi.map_back_part_size(valid_node, valid_len)[0]
+        return capi.auto_back_part_size(valid_node, valid_len)[0]
     if mode == "threshold":
         return capi.threshold_back_part_size(valid_node, valid_len) or 64
     if mode == "wave64":

@@ -17,7 +17,10 @@
  *     per vertex (torch.bool layout).
  *   - Calls are asynchronous on `stream` unless a host result (h_*) is
  *     requested; a function that fills an h_* argument synchronises the stream
- *     first, as the reference's compactors do.
+ *     first, as the reference's compactors do.  Device-side failures of the
+ *     scan-based functions (a stalled look-back, a capacity overflow) are only
+ *     reported by such a synchronising call, or by eppgcn_scan_status /
+ *     eppgcn_build_plan_status.
  *   - Scan-based functions need a workspace of at least the number of bytes the
  *     matching *_workspace_bytes() call returns, 8-byte aligned.  The library
  *     itself allocates no device memory.
@@ -104,6 +107,11 @@ int eppgcn_build_plan(const int32_t* part_pointers, const int32_t* column_index,
                       const int32_t* part2node, const int32_t* ids, int num_parts, int64_t num_slots,
                       int num_nodes, int dim, int block_shift, void* plan, size_t plan_bytes,
                       void* workspace, size_t workspace_bytes, void* stream);
+/* eppgcn_build_plan is asynchronous and contains a look-back scan.  This call synchronises `stream`
+ * and returns 0 or EPPGCN_ERR_SCAN_STALLED for the build that last used `workspace` with this
+ * num_parts (a stalled scan leaves a corrupt plan, which must not be used).  Call it once after the
+ * build, before the workspace is released. */
+int eppgcn_build_plan_status(const void* workspace, int num_parts, void* stream);
 
 /* Forward neighbour-group aggregation:
  *   out[r,:] = sum_{e in groups of r} fl32(degrees[r]*degrees[col[e]]) * in[col[e],:]
@@ -175,6 +183,15 @@ int eppgcn_mask_forward(const int32_t* part2node, const int32_t* part_pointers,
 size_t eppgcn_compact_workspace_bytes(int64_t length);
 size_t eppgcn_split_workspace_bytes(int64_t num_nodes);
 
+/* Status of the last scan-based call that used `workspace` (eppgcn_compact_back_edge,
+ * eppgcn_mark_compact, eppgcn_split_back_part, eppgcn_build_part): synchronises `stream`, then
+ * returns 0, EPPGCN_ERR_SCAN_STALLED (a look-back wait hit its spin limit: the outputs of that call
+ * are invalid) or EPPGCN_ERR_CAPACITY (the group pointers did not fit).  The scan-based calls check
+ * this themselves only when a host result (h_*) is requested; a caller that takes every count on
+ * the device (all h_* NULL) gets return code 0 from them whatever happened on the device and must
+ * call this once before it trusts the outputs. */
+int eppgcn_scan_status(const void* workspace, void* stream);
+
 /* Stable two-array compaction of the slots with edge_mask[e] != -1:
  *   out_id[k] = edge_mask[e_k], out_edge[k] = column_index[e_k], k < V; both
  * outputs (length entries each) are zero from V on.  V is left in device memory at
@@ -239,6 +256,14 @@ int eppgcn_threshold_back_part_size(int64_t valid_node, int64_t valid_len);
  * 8..64 in every measured cell), so two values are all the fit supports.  No counterpart in the
  * reference (its rules are EPPGCN.cpp:246-258 and :303-310). */
 int eppgcn_wave64_back_part_size(int64_t valid_node, int64_t valid_len);
+
+/* The group size a caller of the reference's `map` mode should use with this library: the fitted
+ * regression (eppgcn_map_back_part_size) while it yields at least 1, otherwise - on large paths,
+ * where the regression, which was fitted on small graphs, goes negative (-143 at 10^6 rows with 10^8
+ * kept edges) - the wave64 rule above instead of a clamp to 1 (which would cut a path of 10^8 kept
+ * edges into 10^8 one-slot groups).  *fell_back (may be NULL) is set when the wave64 rule was used.
+ * Stands in for get_map_back_part_size (EPPGCN.cpp:298-325) in drivers. */
+int eppgcn_auto_back_part_size(int64_t valid_node, int64_t valid_len, int* fell_back);
 
 /* Splits the kept edges of every vertex into groups of part_size and writes the
  * group pointers: part_pointer[0..P] with part_pointer[P] = V, zero after that up
@@ -314,7 +339,9 @@ void eppgcn_set_timing(int enabled);
 void eppgcn_print_time(void);
 void eppgcn_clear_time(void);
 /* which: 0 forward aggregation, 1 backward aggregation (all layers), 2 path marking,
- * 100+k backward aggregation of layer k (1-based, k <= 16).  Milliseconds. */
+ * 3 the output clears and 4 the pre-scaling passes of the aggregation calls (0 and 1 cover the
+ * aggregation kernels alone, as the reference's timers do), 100+k backward aggregation of layer k
+ * (1-based, k <= 16).  Milliseconds. */
 double eppgcn_get_time_ms(int which);
 
 /* Forces the number of lanes per neighbour group in the aggregation kernels

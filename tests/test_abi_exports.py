@@ -42,6 +42,11 @@ def test_host_only_heuristics_match_the_checker():
     # the re-fitted rule: 16 below 24 kept edges per kept row, 32 from there on
     assert [capi.wave64_back_part_size(vn, vl) for vn, vl in [(0, 0), (10, 0), (10, 239), (10, 240), (3, 10 ** 9)]] == \
         [16, 16, 16, 32, 32]
+    # the safe form of the `map` mode: the regression while it is usable, the wave64 rule where it is not
+    assert capi.auto_back_part_size(1000, 5000) == (co.map_back_part_size(1000, 5000), False)
+    assert co.map_back_part_size(10 ** 6, 10 ** 8) < 1 and capi.auto_back_part_size(10 ** 6, 10 ** 8) == (32, True)
+    assert capi.auto_back_part_size(4 * 10 ** 6, 4 * 10 ** 7) == (16, True)
+    assert capi.auto_back_part_size(0, 0) == (16, True)
 
 
 def test_product_package_never_imports_the_checker():
@@ -73,10 +78,13 @@ def test_argument_errors_are_reported_before_any_device_work():
         (lib.eppgcn_spmm_forward(one, p0, p0, one, one, one, one, 8, 4, 2, 1, 1, 1, p0, 0, p0, p0), "null feature"),
         (lib.eppgcn_spmm_forward(one, one, p0, one, one, one, one, 8, 0, 2, 1, 1, 1, p0, 0, p0, p0), "dim > 0"),
     ]
+    cases += [(lib.eppgcn_scan_status(p0, p0), "workspace"), (lib.eppgcn_build_plan_status(p0, 5, p0), "workspace"),
+              (lib.eppgcn_build_plan_status(one, -1, p0), "negative")]
     for rc, needle in cases:
         assert rc == -1
     # the message belongs to the last failing call
-    assert b"dim > 0" in lib.eppgcn_last_error()
+    assert b"negative" in lib.eppgcn_last_error()
+    assert lib.eppgcn_build_plan_status(p0, 0, p0) == 0
     assert lib.eppgcn_update_supported(96, 16) == 7 and lib.eppgcn_update_supported(2000, 16) == 6
     assert lib.eppgcn_update_supported(16, 100) == 3 and lib.eppgcn_update_supported(0, 4) == 0
     assert lib.eppgcn_feature_workspace_pitch(16) == 16 and lib.eppgcn_feature_workspace_pitch(22) == 32

@@ -349,10 +349,11 @@ def test_driver_command_line_end_to_end(GNNA, tmp_path, capsys):
         gcn_main.main(["--dataset", "no_such_graph", "--dataDir", str(tmp_path)])
 
 
-@pytest.mark.parametrize("num_layers", [3, 4])
+@pytest.mark.parametrize("num_layers", [3, 4, 5, 6])
 def test_deeper_models_follow_the_mask_chain(GNNA, num_layers):
-    """3 and 4 layers (the reference sweeps 3-6): the marking of layer i feeds layer i+1's source
-    mask and edge_masks[L-1-i]; gradients of every weight equal the float64 dense model's."""
+    """3 to 6 layers (the depths the reference sweeps, EPPGCN/bench_EPPGCN.py:36): the marking of
+    layer i feeds layer i+1's source mask and edge_masks[L-1-i]; gradients of every weight equal the
+    float64 dense model's."""
     from eppgcn_amd import graphs, train
     indptr, col = random_symmetric_csr(500, 1400, 41)
     n = indptr.size - 1
@@ -383,6 +384,80 @@ def test_deeper_models_follow_the_mask_chain(GNNA, num_layers):
     # the kept path grows from the last layer (train rows only) towards the first
     kept = [b.numParts for b in tr.back_props]
     assert all(kept[i] >= kept[i + 1] for i in range(num_layers - 1))
+    # and every layer's compacted path is the closed form of the chain (EPPGCN/gcn_main.py:130-139):
+    # step i keeps the slots whose column is in its source mask; the next source mask is the rows of
+    # the current one that have slots, plus their neighbours
+    row = cf.row_index(indptr)
+    src = mask.copy()
+    for i in range(num_layers):
+        prop = tr.back_props[num_layers - 1 - i]
+        keep = src[col]
+        v = int(keep.sum())
+        assert int(prop.partPointer[prop.numParts]) == v
+        assert np.array_equal(prop.id[:v].cpu().numpy(), row[keep]) and np.array_equal(prop.edgeList[:v].cpu().numpy(), col[keep])
+        nxt = np.zeros(n, bool)
+        sel = src[row]
+        nxt[row[sel]] = True
+        nxt[col[sel]] = True
+        src = nxt
+
+
+def test_group_size_rules_on_device_degrees(GNNA):
+    """get_wave64_back_part_size / get_map_back_part_size on kept degrees that live on the device: the
+    wave64 rule is 16 below 24 kept edges per kept row and 32 from there on; the fitted regression
+    (EPPGCN/GCNConv/EPPGCN.cpp:303-310) is returned while it is at least 1 and replaced by the wave64
+    rule where it goes negative (large paths), never by a clamp to 1."""
+    from eppgcn_amd import capi, graphs, workload
+    g = graphs.make_graph("cfg3_rmat20", device="cuda")
+    wl = workload.prepare(g, 2, 0.1, 2, plan=False)
+    for path in wl.paths:
+        vn = int((path.node_degs != 0).sum())
+        assert vn == path.valid_node
+        want = 16 if path.valid_len // vn < 24 else 32
+        assert GNNA.get_wave64_back_part_size(path.node_degs, path.valid_len) == want
+        fitted = co.map_back_part_size(vn, path.valid_len)
+        assert fitted >= 1, "the regression is positive at this size"
+        assert GNNA.get_map_back_part_size(path.node_degs, path.valid_len) == fitted
+        assert capi.auto_back_part_size(vn, path.valid_len) == (fitted, False)
+    # a path the regression was never fitted for: 10^6 kept rows of 100 kept edges each -> -143
+    degs = torch.full((1_000_000,), 100, dtype=torch.int32, device="cuda")
+    assert co.map_back_part_size(1_000_000, 100_000_000) < 1
+    assert capi.map_back_part_size(1_000_000, 100_000_000) == (1, True)
+    assert GNNA.get_map_back_part_size(degs, 100_000_000) == 32      # (warns once per process)
+    assert capi.auto_back_part_size(1_000_000, 100_000_000) == (32, True)
+    degs[::2] = 0                                  # half of the rows keep nothing: 5 * 10^5 rows, 10 per row
+    degs[1::2] = 10
+    assert GNNA.get_wave64_back_part_size(degs, 5_000_000) == 16
+    # get_ginfo takes the kept degrees from the host as well, as the reference's caller passes them
+    assert torch.equal(GNNA.get_ginfo(degs.cpu(), 5_000_000), GNNA.get_ginfo(degs, 5_000_000))
+
+
+def test_sweep_driver_runs_every_depth_in_one_process(GNNA, tmp_path, capsys):
+    """The datasets x ratios x depths sweep (EPPGCN/bench_EPPGCN.py:17-61) over the driver: a dataset
+    from files in the reference's layout and a synthetic one, depths 3-6, one report line each."""
+    import json
+    from eppgcn_amd import bench_eppgcn, dataset as ds_mod
+    indptr, col = random_symmetric_csr(400, 1500, 77)
+    folder = tmp_path / "toy"
+    folder.mkdir()
+    rows = cf.row_index(indptr)
+    np.savetxt(folder / "toy_snap", np.stack([rows, col], 1), fmt="%d")
+    ds_mod.write_train_mask(str(folder), 0.3, np.random.default_rng(1).random(400) < 0.3)
+    rc = bench_eppgcn.main(["--dataRoot", str(tmp_path), "--datasets", "toy,12,5", "cfg1_uniform", "absent,8,3",
+                            "--ratios", "0.3", "--layers", "3", "4", "5", "6", "--num_epoches", "3",
+                            "--groupsize_model", "regression_equation"])
+    assert rc == 0
+    out = capsys.readouterr().out
+    lines = [json.loads(l) for l in out.splitlines() if l.startswith("{")]
+    assert len(lines) == 12
+    ok = [l for l in lines if l["status"] == "ok"]
+    assert [(l["dataset"], l["layers"]) for l in ok] == [(d, k) for d in ("toy", "cfg1_uniform") for k in (3, 4, 5, 6)]
+    assert all(l["status"] == "skipped" for l in lines if l["dataset"] == "absent")
+    for l in ok:
+        assert l["Time"] > 0 and len(l["backward_group_sizes"]) == l["layers"] and min(l["backward_group_sizes"]) >= 1
+    assert out.count("||toy   0.3   ") == 4 and out.count("Time: ") == 8
+    assert bench_eppgcn.main(["--datasets", "cfg1_uniform", "--ratios", "0.1", "--layers", "3", "--num_epoches", "1",
+                              "--groupsize_model", "SAGPG"]) == 1
 
 
 def test_module_mark_compact_equals_the_two_reference_steps(GNNA):

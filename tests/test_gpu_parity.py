@@ -133,6 +133,40 @@ def test_split_all_zero_and_capacity_error(api):
         api.split_back_part(dev(degs), 100, 1)     # 15000 groups cannot fit 101 entries
 
 
+def test_scan_status_reports_what_asynchronous_calls_cannot(api):
+    """With every count taken on the device (no h_* argument) the scan-based calls return before the
+    device has run; eppgcn_scan_status is how such a caller learns of a capacity overflow."""
+    import ctypes as C
+    lib = api.load()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ptr = lambda t: C.c_void_p(t.data_ptr())
+    n = 50000
+    degs = torch.full((n,), 3, dtype=torch.int32, device="cuda")
+    nbytes = lib.eppgcn_split_workspace_bytes(n)
+    ws = torch.empty((nbytes + 7) // 8, dtype=torch.int64, device="cuda")
+    counts = torch.zeros(2, dtype=torch.int32, device="cuda")
+    roomy = torch.empty(3 * n + 1, dtype=torch.int32, device="cuda")
+    assert lib.eppgcn_split_back_part(ptr(degs), n, 1, ptr(roomy), roomy.numel(), ptr(ws), nbytes, ptr(counts),
+                                      None, None, stream) == 0
+    assert lib.eppgcn_scan_status(ptr(ws), stream) == 0
+    assert counts.tolist() == [3 * n, 3 * n] and int(roomy[-1]) == 3 * n
+    tight = torch.empty(n, dtype=torch.int32, device="cuda")             # 3n + 1 entries are needed
+    assert lib.eppgcn_split_back_part(ptr(degs), n, 1, ptr(tight), tight.numel(), ptr(ws), nbytes, ptr(counts),
+                                      None, None, stream) == 0
+    assert lib.eppgcn_scan_status(ptr(ws), stream) == -4 and b"capacity" in lib.eppgcn_last_error()
+    # a compaction that took its count on the device only
+    mask = torch.where(torch.arange(100000, device="cuda") % 3 == 0, 7, -1).int()
+    col = torch.arange(100000, dtype=torch.int32, device="cuda")
+    oid, oedge = torch.empty_like(mask), torch.empty_like(col)
+    cbytes = lib.eppgcn_compact_workspace_bytes(mask.numel())
+    cws = torch.empty((cbytes + 7) // 8, dtype=torch.int64, device="cuda")
+    kept = torch.zeros(1, dtype=torch.int32, device="cuda")
+    assert lib.eppgcn_compact_back_edge(ptr(mask), ptr(col), ptr(oid), ptr(oedge), mask.numel(), ptr(cws), cbytes,
+                                        ptr(kept), None, stream) == 0
+    assert lib.eppgcn_scan_status(ptr(cws), stream) == 0 and int(kept) == 33334
+    assert torch.equal(oedge[:33334], col[::3])
+
+
 def test_heuristics_and_ginfo(api):
     for vn, vl in [(1000, 5000), (100000, 1000000), (419000, 13_400_000), (7, 7)]:
         ps, clamped = api.map_back_part_size(vn, vl)
