@@ -18,12 +18,10 @@
 // The re-ordering changes no result, only which groups run together.  It depends on the graph
 // and the groups alone: a caller builds it once and passes it to every aggregation call.
 //
-// The stable sort of (block, group index) pairs is rocPRIM's device radix sort, a library
-// routine in a preparation step, as the reference uses thrust for its scans; everything else
-// (keys, look-back scan of the group sizes, flags, column copy) is written here.
+// Everything is written here: the keys, a stable least-significant-digit radix sort of the
+// (key, group index) pairs (8 bits per pass: tile histograms, one look-back scan, stable scatter with
+// ballot-based ranks), the look-back scan of the group sizes, the flags and the column copy.
 #include <cstring>
-
-#include <rocprim/device/device_radix_sort.hpp>
 
 #include "common.hpp"
 
@@ -43,11 +41,10 @@ constexpr int kMaxRowWalk = 64;
 __global__ __launch_bounds__(256) void plan_keys_kernel(const int* __restrict__ part_ptr, const int* __restrict__ col,
                                                        const int* __restrict__ part2node, const int* __restrict__ ids,
                                                        int num_parts, int shift, int keep_slots, int classes,
-                                                       unsigned* __restrict__ keys, int* __restrict__ iota)
+                                                       unsigned* __restrict__ keys)
 {
     const int p = blockIdx.x * blockDim.x + threadIdx.x;
     if (p >= num_parts) return;
-    iota[p] = p;
     const int beg = part_ptr[p];
     const int end = part_ptr[p + 1];
     if (end <= beg) { keys[p] = 0u; return; }
@@ -134,6 +131,91 @@ __global__ __launch_bounds__(kScanBlock) void exclusive_scan_kernel(const int* _
     if (tile == num_tiles - 1 && threadIdx.x == kScanBlock - 1) out[n] = run;
 }
 
+// ---------------------------------------------------------------- stable radix sort of (key, index) pairs
+// One pass sorts by the 8-bit digit (key >> shift) & 255 and keeps the order of equal digits, so
+// passes from the least significant digit upwards sort by the whole key, equal keys staying in index
+// order.  A tile is kSortTile consecutive elements, element (round r, thread t) of tile T being
+// T * kSortTile + r * 256 + t, so that (round, wave, lane) order is index order.
+//   radix_hist_kernel     hist[d * tiles + T] = elements of tile T with digit d
+//   exclusive_scan_kernel over hist (digit-major): where (digit d, tile T) starts in the output
+//   radix_scatter_kernel  rank of an element among the equal digits of its wave from eight ballots,
+//                         counts per (round, wave, digit) in LDS, prefix over (round, wave) per digit
+constexpr int kSortBlock = 256;
+constexpr int kSortRounds = 8;
+constexpr int kSortTile = kSortBlock * kSortRounds;
+constexpr int kDigits = 256;
+
+__global__ __launch_bounds__(kSortBlock) void radix_hist_kernel(const unsigned* __restrict__ keys, int n, int shift,
+                                                                int num_tiles, int* __restrict__ hist)
+{
+    __shared__ int s_hist[kDigits];
+    s_hist[threadIdx.x] = 0;
+    __syncthreads();
+    const long long base = static_cast<long long>(blockIdx.x) * kSortTile;
+#pragma unroll
+    for (int r = 0; r < kSortRounds; ++r) {
+        const long long i = base + r * kSortBlock + threadIdx.x;
+        if (i < n) atomicAdd(&s_hist[(keys[i] >> shift) & (kDigits - 1)], 1);
+    }
+    __syncthreads();
+    hist[static_cast<long long>(threadIdx.x) * num_tiles + blockIdx.x] = s_hist[threadIdx.x];
+}
+
+// vals_in == nullptr: the value of element i is i (first pass)
+__global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(const unsigned* __restrict__ keys_in,
+                                                                   const int* __restrict__ vals_in,
+                                                                   unsigned* __restrict__ keys_out,
+                                                                   int* __restrict__ vals_out, int n, int shift,
+                                                                   int num_tiles, const int* __restrict__ offsets)
+{
+    constexpr int kWaves = kSortBlock / kWave;
+    __shared__ int s_count[kSortRounds * kWaves][kDigits];      // per (round, wave): elements of each digit
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < kSortRounds * kWaves * kDigits; i += kSortBlock) (&s_count[0][0])[i] = 0;
+    __syncthreads();
+    const long long base = static_cast<long long>(blockIdx.x) * kSortTile;
+    unsigned key[kSortRounds];
+    int rank[kSortRounds];
+#pragma unroll
+    for (int r = 0; r < kSortRounds; ++r) {
+        const long long i = base + r * kSortBlock + threadIdx.x;
+        const bool valid = i < n;
+        key[r] = valid ? keys_in[i] : 0u;
+        const unsigned d = (key[r] >> shift) & (kDigits - 1);
+        // lanes of the wave holding the same digit: intersect the ballots of the eight digit bits
+        uint64_t peers = __ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const uint64_t set = __ballot(((d >> b) & 1u) != 0);
+            peers &= ((d >> b) & 1u) ? set : ~set;
+        }
+        rank[r] = __popcll(peers & ((1ull << lane) - 1ull));
+        if (valid && rank[r] == 0) s_count[r * kWaves + wave][d] = __popcll(peers);
+    }
+    __syncthreads();
+    {   // thread d: exclusive prefix of digit d over the (round, wave) pairs, on top of the tile's global offset
+        int run = offsets[static_cast<long long>(threadIdx.x) * num_tiles + blockIdx.x];
+#pragma unroll
+        for (int q = 0; q < kSortRounds * kWaves; ++q) {
+            const int c = s_count[q][threadIdx.x];
+            s_count[q][threadIdx.x] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kSortRounds; ++r) {
+        const long long i = base + r * kSortBlock + threadIdx.x;
+        if (i < n) {
+            const unsigned d = (key[r] >> shift) & (kDigits - 1);
+            const int dst = s_count[r * kWaves + wave][d] + rank[r];
+            keys_out[dst] = key[r];
+            vals_out[dst] = vals_in ? vals_in[i] : static_cast<int>(i);
+        }
+    }
+}
+
 // row, flags and the column copy of every plan entry; a team of 8 lanes per group.
 __global__ __launch_bounds__(256) void plan_fill_kernel(const int* __restrict__ part_ptr, const int* __restrict__ col,
                                                        const int* __restrict__ part2node, const int* __restrict__ ids,
@@ -172,28 +254,26 @@ __global__ __launch_bounds__(256) void plan_fill_kernel(const int* __restrict__ 
 }
 
 // ---------------------------------------------------------------- host
-static hipError_t sort_temp_bytes(int num_parts, int bits, size_t* bytes)
-{
-    *bytes = 0;
-    return rocprim::radix_sort_pairs(nullptr, *bytes, static_cast<unsigned*>(nullptr), static_cast<unsigned*>(nullptr),
-                                     static_cast<int*>(nullptr), static_cast<int*>(nullptr),
-                                     static_cast<size_t>(num_parts), 0u, static_cast<unsigned>(bits));
-}
-
 static size_t scan_state_bytes(long long n)
 {
     const long long tiles = (n + kScanTile - 1) / kScanTile;
     return align256(sizeof(ScanState) + sizeof(uint64_t) * static_cast<size_t>(tiles > 0 ? tiles : 1));
 }
 
-// workspace layout: keys_in | keys_out | iota | order | sizes | scan state | rocPRIM temporary storage
+static long long sort_tiles(long long n) { return (n + kSortTile - 1) / kSortTile; }
+// histogram | its exclusive scan (one more entry) | state of that scan
+static size_t sort_temp_bytes(long long n)
+{
+    const long long entries = sort_tiles(n) * kDigits;
+    return 2 * align256(sizeof(int) * static_cast<size_t>(entries + 1)) + scan_state_bytes(entries);
+}
+
+// workspace layout: keys_in | keys_out | order (scratch) | order | sizes | scan state | sort temporaries
 size_t plan_workspace_bytes(long long num_parts)
 {
     if (num_parts <= 0) return 256;
-    size_t temp = 0;
-    if (sort_temp_bytes(static_cast<int>(num_parts), 32, &temp) != hipSuccess) temp = 0;
     return 5 * align256(sizeof(int) * (static_cast<size_t>(num_parts) + 1)) + scan_state_bytes(num_parts) +
-           align256(temp) + 256;
+           sort_temp_bytes(num_parts) + 256;
 }
 
 // where launch_build_plan keeps the state of its look-back scan inside the workspace
@@ -236,6 +316,51 @@ __global__ void plan_scan_init_kernel(ScanState* st, uint64_t* desc, int num_til
     }
 }
 
+// out[0..n] = exclusive prefix sums of in[0..n) (out[n] = total), with the scan state at `state`
+static int launch_exclusive_scan(const int* in, int* out, long long n, void* state, hipStream_t stream)
+{
+    ScanState* st = static_cast<ScanState*>(state);
+    uint64_t* desc = reinterpret_cast<uint64_t*>(st + 1);
+    const int tiles = static_cast<int>((n + kScanTile - 1) / kScanTile);
+    hipLaunchKernelGGL(plan_scan_init_kernel, dim3((tiles + 255) / 256), dim3(256), 0, stream, st, desc, tiles);
+    EPPGCN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(exclusive_scan_kernel, dim3(tiles), dim3(kScanBlock), 0, stream, in, out, static_cast<int>(n),
+                       tiles, st, desc);
+    EPPGCN_HIP(hipGetLastError());
+    return kOk;
+}
+
+// Sorts the pairs (keys[i], i) by the low `bits` bits of the key, stably; the sorted indices end up in
+// `order`.  keys_a is overwritten; keys_b, vals_tmp and temp are scratch.
+static int stable_sort_by_key(unsigned* keys_a, unsigned* keys_b, int* vals_tmp, int* order, int n, int bits, void* temp,
+                              hipStream_t stream)
+{
+    const int tiles = static_cast<int>(sort_tiles(n));
+    const long long entries = static_cast<long long>(tiles) * kDigits;
+    char* t = static_cast<char*>(temp);
+    int* hist = reinterpret_cast<int*>(t);
+    int* offsets = reinterpret_cast<int*>(t + align256(sizeof(int) * static_cast<size_t>(entries + 1)));
+    void* state = t + 2 * align256(sizeof(int) * static_cast<size_t>(entries + 1));
+    const int passes = bits <= 8 ? 1 : (bits + 7) / 8;
+    // the last pass must write `order`: with an even number of passes the first one writes the temporary
+    unsigned* kin = keys_a;
+    unsigned* kout = keys_b;
+    const int* vin = nullptr;
+    for (int pass = 0; pass < passes; ++pass) {
+        int* vout = ((passes - pass) % 2 == 1) ? order : vals_tmp;
+        const int shift = pass * 8;
+        hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(kSortBlock), 0, stream, kin, n, shift, tiles, hist);
+        EPPGCN_HIP(hipGetLastError());
+        if (int rc = launch_exclusive_scan(hist, offsets, entries, state, stream)) return rc;
+        hipLaunchKernelGGL(radix_scatter_kernel, dim3(tiles), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, shift,
+                           tiles, offsets);
+        EPPGCN_HIP(hipGetLastError());
+        unsigned* tk = kin; kin = kout; kout = tk;
+        vin = vout;
+    }
+    return kOk;
+}
+
 int launch_build_plan(const int* part_ptr, const int* col, const int* part2node, const int* ids, int num_parts,
                       long long num_slots, int num_nodes, int shift, void* plan, size_t plan_size, void* workspace,
                       size_t workspace_bytes, hipStream_t stream)
@@ -249,37 +374,29 @@ int launch_build_plan(const int* part_ptr, const int* col, const int* part2node,
     char* base = static_cast<char*>(workspace);
     unsigned* keys_in = reinterpret_cast<unsigned*>(base);
     unsigned* keys_out = reinterpret_cast<unsigned*>(base + slab);
-    int* iota = reinterpret_cast<int*>(base + 2 * slab);
+    int* order_tmp = reinterpret_cast<int*>(base + 2 * slab);
     int* order = reinterpret_cast<int*>(base + 3 * slab);
     int* sizes = reinterpret_cast<int*>(base + 4 * slab);
     ScanState* st = reinterpret_cast<ScanState*>(base + plan_scan_state_offset(num_parts));
-    uint64_t* desc = reinterpret_cast<uint64_t*>(st + 1);
     void* temp = base + 5 * slab + scan_state_bytes(num_parts);
     int bits = 1;
     while (bits < 30 && (static_cast<long long>(num_nodes) >> shift) >= (1ll << bits)) ++bits;
     if (g_length_classes) bits += 2;
-    size_t temp_bytes = 0;
-    EPPGCN_HIP(sort_temp_bytes(num_parts, bits, &temp_bytes));
+    const size_t temp_bytes = sort_temp_bytes(num_parts);
     if (5 * slab + scan_state_bytes(num_parts) + temp_bytes > workspace_bytes) {
         set_error("build_plan: workspace smaller than eppgcn_plan_workspace_bytes(num_parts)");
         return kErrInvalidArgument;
     }
     const unsigned blocks = static_cast<unsigned>((num_parts + 255) / 256);
     hipLaunchKernelGGL(plan_keys_kernel, dim3(blocks), dim3(256), 0, stream, part_ptr, col, part2node, ids, num_parts,
-                       shift, g_keep_rows * 32, g_length_classes, keys_in, iota);
+                       shift, g_keep_rows * 32, g_length_classes, keys_in);
     EPPGCN_HIP(hipGetLastError());
-    EPPGCN_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, iota, order,
-                                         static_cast<size_t>(num_parts), 0u, static_cast<unsigned>(bits), stream));
+    if (int rc = stable_sort_by_key(keys_in, keys_out, order_tmp, order, num_parts, bits, temp, stream)) return rc;
     hipLaunchKernelGGL(plan_sizes_kernel, dim3(blocks), dim3(256), 0, stream, part_ptr, order, num_parts, sizes);
-    EPPGCN_HIP(hipGetLastError());
-    const int tiles = (num_parts + kScanTile - 1) / kScanTile;
-    hipLaunchKernelGGL(plan_scan_init_kernel, dim3((tiles + 255) / 256), dim3(256), 0, stream, st, desc, tiles);
     EPPGCN_HIP(hipGetLastError());
     PlanView v = plan_view(plan, num_parts, num_nodes);
     if (int rc = launch_zero_words(v.single, plan_single_words(num_nodes), stream)) return rc;
-    hipLaunchKernelGGL(exclusive_scan_kernel, dim3(tiles), dim3(kScanBlock), 0, stream, sizes, v.ptr, num_parts, tiles,
-                       st, desc);
-    EPPGCN_HIP(hipGetLastError());
+    if (int rc = launch_exclusive_scan(sizes, v.ptr, num_parts, st, stream)) return rc;
     const long long threads = static_cast<long long>(num_parts) * 8;
     hipLaunchKernelGGL(plan_fill_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream,
                        part_ptr, col, part2node, ids, order, num_parts, v);

@@ -5,10 +5,10 @@
   (column-blocked, or one block for heavily pruned paths) and the gathered-rows bitmap that
   ``eppgcn_amd.sweep`` and the extension module use.  Per cell: the compacted path against its closed
   form (bit-exact), integer data pruned == unpruned == int64 ``index_add_`` (bit-exact), float data
-  with the symmetric normalisation within rel. tol. 1e-5 of a float64 ``index_add_`` on the device.
+  with the symmetric normalisation within rel. tol. 1e-5 of a float64 sparse product on the device.
 * Headline configuration (R-MAT scale 22): s = deg^-1/2, N(0,1) features, both forward widths and
   both pruned paths through the pre-scaled feature workspace (128-byte rows at width 22) with plans and
-  the gathered-rows bitmap - i.e. exactly what ``bench.py`` times - against float64 ``index_add_``.
+  the gathered-rows bitmap - i.e. exactly what ``bench.py`` times - against a float64 sparse product.
 
 Tolerance: |got - want| <= 1e-5 * sum_j |w_ij x_j| per output element (a forward error bound of the
 sum, the right yardstick for sums that cancel), written out in ``_assert_within``.
@@ -33,17 +33,16 @@ def api():
 
 
 # ----------------------------------------------------------------------------- float64 references on the device
-def _weighted_sums(row, col, w, x, rows_out, chunk=1 << 23):
-    """(sum_e w_e x[col_e], sum_e |w_e x[col_e]|) per output row in float64, by ``index_add_`` over
-    slot chunks (so that the E x D float64 intermediates stay small)."""
-    dim = x.shape[1]
-    want = torch.zeros(rows_out, dim, dtype=torch.float64, device=x.device)
-    bound = torch.zeros_like(want)
-    for lo in range(0, row.numel(), chunk):
-        hi = min(row.numel(), lo + chunk)
-        t = x[col[lo:hi]].double() * w[lo:hi, None]
-        want.index_add_(0, row[lo:hi], t)
-        bound.index_add_(0, row[lo:hi], t.abs_())
+def _weighted_sums(row_pointers, col, w, x):
+    """(sum_e w_e x[col_e], sum_e |w_e x[col_e]|) per output row in float64: the textbook sparse
+    product A @ x of a float64 CSR matrix with the edge weights as values (torch.sparse.mm, i.e. the
+    vendor's SpMM - an implementation that shares nothing with the kernels under test)."""
+    n = row_pointers.numel() - 1
+    crow = row_pointers.long()
+    a = torch.sparse_csr_tensor(crow, col, w, size=(n, n))
+    want = torch.sparse.mm(a, x.double())
+    a_abs = torch.sparse_csr_tensor(crow, col, w.abs(), size=(n, n))
+    bound = torch.sparse.mm(a_abs, x.double().abs())
     return want, bound
 
 
@@ -129,7 +128,7 @@ class _Rmat20:
             self.refs.clear()                     # one (ratio, width) at a time: [N, 256] float64 is 2 GB
             mask = self.path(ratio)[0]
             dy = self.graphs.normal32(7, (self.n, width), "cuda") * mask[:, None]
-            want, bound = _weighted_sums(self.row, self.col, self.w, dy, self.n)
+            want, bound = _weighted_sums(self.g.row_pointers, self.col, self.w, dy)
             self.refs[key] = (dy, want, bound)
         return self.refs[key]
 
@@ -214,7 +213,7 @@ def test_headline_size_benched_numeric_path_within_tolerance(api):
     for dim, path, src in ((16, wl.paths[0], wl.ngh_masks[0]), (22, wl.paths[1], wl.train_mask)):
         ws = api.feature_workspace(n, dim, "cuda")
         x = graphs.normal32(1, (n, dim), "cuda", dim)
-        want, bound = _weighted_sums(row, col, w, x, n)
+        want, bound = _weighted_sums(g.row_pointers, col, w, x)
         out = torch.full((n, dim), float("nan"), device="cuda")
         got = api.spmm_forward(x, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 32, 8,
                                g.row_pointers, out, workspace=ws, plan=wl.plans[dim])
@@ -230,7 +229,7 @@ def test_headline_size_benched_numeric_path_within_tolerance(api):
         del table, want, bound
 
         dy = graphs.normal32(2, (n, dim), "cuda", dim) * src[:, None]
-        want, bound = _weighted_sums(row, col, w, dy, n)
+        want, bound = _weighted_sums(g.row_pointers, col, w, dy)
         out.fill_(float("nan"))
         ws.fill_(float("nan"))                   # rows the scaling pass skips must never be gathered
         got = api.ours_backward(dy, path.ids, path.part_pointer, path.edge_list, g.degrees, path.num_parts,

@@ -279,11 +279,23 @@ def test_plan_is_a_stable_column_block_reordering(api, name, ps):
     first slot with the original order kept inside a block, with rows, column ids and adjacency
     flags that describe the original groups."""
     indptr, col = GRAPHS[name]()
+    # default block sizes (one block for these small graphs at width 16) and forced small blocks; blocks of
+    # 4 vertices make sort keys of up to 15 bits, i.e. two passes of the radix sort
+    _check_plan_order(api, indptr, col, ps, ((16, 0), (256, 0), (16, 9), (16, 12), (16, 2)))
+
+
+def test_plan_sort_with_three_radix_passes(api):
+    """300 000 vertices in blocks of 2: 18 block bits + 2 class bits = three 8-bit passes, the last of
+    which has to land in the final buffer; ties must stay in group order."""
+    indptr, col = random_symmetric_csr(300000, 500000, 29)
+    _check_plan_order(api, indptr, col, 16, ((16, 1), (16, 5)))
+
+
+def _check_plan_order(api, indptr, col, ps, cases):
     n = indptr.size - 1
     pp, p2n = co.build_part(ps, indptr)
     P = p2n.size
-    # default block sizes (one block for these small graphs at width 16) and forced small blocks
-    for dim, forced in ((16, 0), (256, 0), (16, 9), (16, 12)):
+    for dim, forced in cases:
         api.set_plan_shift(forced)
         try:
             plan = api.build_plan(dev(pp), dev(col), P, col.size, n, dim, part2node=dev(p2n))
