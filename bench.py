@@ -54,8 +54,9 @@ def parse():
     ap.add_argument("--plan_keep", type=int, default=-1, help="rows with at most this many groups stay together")
     ap.add_argument("--force_plan", action="store_true", help="use execution plans even for small feature tables")
     ap.add_argument("--no_length_classes", action="store_true", help="plans without the length-class key")
-    ap.add_argument("--stepwise_prep", action="store_true",
-                    help="prepare the backward paths with the reference's separate marking and compaction steps")
+    ap.add_argument("--fused_prep", action="store_true",
+                    help="prepare the backward paths with the one-pass marking + compaction instead of the "
+                         "reference's separate steps (same results, same time, no edge masks)")
     ap.add_argument("--no_plan", action="store_true",
                     help="process the groups in CSR order instead of the column-blocked execution plan")
     ap.add_argument("--no_workspace", action="store_true",
@@ -162,7 +163,7 @@ def main():
     t0 = time.perf_counter()
     wl = workload.prepare(g, 2, args.train_ratio, 2, args.part_size or None, args.backsize_mode, args.backsize,
                           plan=False if args.no_plan else (True if args.force_plan else None),
-                          fused=not args.stepwise_prep)
+                          fused=args.fused_prep)
     torch.cuda.synchronize()
     prep_s = time.perf_counter() - t0
     n, e = g.num_nodes, g.num_edges

@@ -410,6 +410,30 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
                 for (int j = 0; j < VW; ++j) acc[k].v[j] *= s_row;
         }
 
+        // ---- a round of complete rows (every group is all of its row, nothing carried in): each team
+        // stores its sum and the run bookkeeping below is skipped.  Plans order single-group rows next to
+        // each other, so on graphs of low degree most rounds take this path.
+        if (!carry_valid && __all(!active || (flags & 15) == 0)) {
+            if (live) {
+                float* dst = out + static_cast<size_t>(row) * ld_out;
+#pragma unroll
+                for (int k = 0; k < CPL; ++k) {
+                    const int c0 = (tl + k * TS) * VW;
+#pragma unroll
+                    for (int piece = 0; piece < VW / OVW; ++piece) {
+                        const int c = c0 + piece * OVW;
+                        if (c < width_out) {
+                            Vec<OVW> o;
+#pragma unroll
+                            for (int j = 0; j < OVW; ++j) o.v[j] = acc[k].v[piece * OVW + j];
+                            o.store(dst + c);
+                        }
+                    }
+                }
+            }
+            continue;
+        }
+
         // ---- combine with the carried run, reduce across teams, flush or carry on
         bool prev = live && (flags & 1) != 0;
         const bool next = live && (flags & 2) != 0;
