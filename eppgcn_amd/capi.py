@@ -27,10 +27,10 @@ EXPORTS = [
     "eppgcn_mark_compact_workspace_bytes", "eppgcn_mark_compact", "eppgcn_set_plan_length_classes",
     "eppgcn_mark_gathered_rows", "eppgcn_set_wide_index", "eppgcn_wave64_back_part_size",
     "eppgcn_compact_back_edge_static", "eppgcn_compact_back_edge_static_max_length",
-    "eppgcn_auto_back_part_size", "eppgcn_scan_status", "eppgcn_build_plan_status",
+    "eppgcn_auto_back_part_size", "eppgcn_scan_status", "eppgcn_build_plan_status", "eppgcn_set_scan_test_mode",
 ]
 
-ABI_VERSION = 11      # what eppgcn_abi_version() of a matching library returns
+ABI_VERSION = 12      # what eppgcn_abi_version() of a matching library returns
 
 _lib = None
 
@@ -102,6 +102,8 @@ def load():
     lib.eppgcn_set_team_size.restype = None
     lib.eppgcn_set_rounds.argtypes = [i]
     lib.eppgcn_set_rounds.restype = None
+    lib.eppgcn_set_scan_test_mode.argtypes = [C.c_uint, i]
+    lib.eppgcn_set_scan_test_mode.restype = None
     lib.eppgcn_set_wide_index.argtypes = [i]
     lib.eppgcn_set_wide_index.restype = None
     lib.eppgcn_set_plan_shift.argtypes = [i]
@@ -578,6 +580,11 @@ def set_rounds(rounds: int):
 def set_wide_index(on: bool):
     """Forces the 64-bit instantiations of the clear and pre-scaling kernels (for tests)."""
     load().eppgcn_set_wide_index(int(bool(on)))
+
+
+def set_scan_test_mode(spin_limit: int = 0, mute_first_tile: bool = False):
+    """Test knob: bounded look-back waits that are certain to give up (see the header); (0, False) = normal."""
+    load().eppgcn_set_scan_test_mode(int(spin_limit), int(bool(mute_first_tile)))
 
 
 def set_plan_length_classes(on: bool):

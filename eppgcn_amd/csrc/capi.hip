@@ -17,6 +17,7 @@ int aggregate_compacted_groups(float*, const float*, const int*, const int*, con
                                int, int, int, int, float*, const uint32_t*, hipStream_t, double*, double*);
 size_t plan_workspace_bytes(long long);
 size_t plan_scan_state_offset(long long);
+size_t plan_sort_state_offset(long long);
 int schedule_shift(int);
 void set_schedule_shift(int);
 void set_plan_keep_rows(int);
@@ -86,7 +87,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 11; }
+int eppgcn_abi_version(void) { return 12; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -382,8 +383,9 @@ int eppgcn_build_plan_status(const void* workspace, int num_parts, void* stream)
     if (num_parts == 0) return kOk;
     EPPGCN_REQUIRE(workspace && aligned(workspace, 256), "workspace must be 256-byte aligned");
     ScanState host;
-    return read_state(static_cast<char*>(const_cast<void*>(workspace)) + plan_scan_state_offset(num_parts),
-                      static_cast<hipStream_t>(stream), &host);
+    char* base = static_cast<char*>(const_cast<void*>(workspace));
+    if (int rc = read_state(base + plan_sort_state_offset(num_parts), static_cast<hipStream_t>(stream), &host)) return rc;
+    return read_state(base + plan_scan_state_offset(num_parts), static_cast<hipStream_t>(stream), &host);
 }
 
 static int finish_split(void* workspace, hipStream_t s, int32_t* d_counts, int64_t* h_a, int64_t* h_b)
@@ -490,6 +492,7 @@ double eppgcn_get_time_ms(int which)
 void eppgcn_set_team_size(int lanes) { set_agg_force_team(lanes); }
 void eppgcn_set_rounds(int rounds) { set_agg_force_rounds(rounds); }
 void eppgcn_set_wide_index(int on) { set_force_wide_index(on != 0); }
+void eppgcn_set_scan_test_mode(unsigned spin_limit, int mute_first_tile) { set_scan_test_mode(spin_limit, mute_first_tile); }
 void eppgcn_set_plan_shift(int shift) { set_schedule_shift(shift); }
 void eppgcn_set_plan_keep_rows(int groups) { set_plan_keep_rows(groups); }
 void eppgcn_set_plan_length_classes(int on) { set_plan_length_classes(on); }

@@ -232,11 +232,17 @@ constexpr unsigned kSpinLimit = 1u << 22;   // polls before a wait is declared s
 
 struct ScanState {
     int counter;        // next tile id to hand out
-    int error;          // set to 1 when a look-back wait hit kSpinLimit
+    int error;          // set to 1 when a look-back wait hit its spin limit
     int counts[2];      // results the last tile publishes (meaning depends on the kernel)
     int overflow;       // set to 1 when an output would not fit its capacity
-    int pad[3];
+    unsigned spin_limit;     // polls before a wait is declared stalled (0 = kSpinLimit)
+    int mute_first_tile;     // test mode: tile 0 never publishes, so every look-back ends in a bounded stall
+    int pad;
 };
+// What the scan-init kernels write into the two fields above (host globals behind a test knob).
+unsigned scan_spin_limit();
+int scan_mute_first_tile();
+void set_scan_test_mode(unsigned spin_limit, int mute_first_tile);
 static_assert(sizeof(ScanState) == 32, "descriptor array starts 32 bytes into the workspace");
 
 __device__ __forceinline__ void tile_store(uint64_t* desc, int tile, uint64_t v)
@@ -262,15 +268,16 @@ __device__ __forceinline__ int acquire_tile(ScanState* st, int* s_tile)
 // Executed by one full wave.  Publishes this tile's aggregate, walks back over
 // the predecessors 64 at a time until a tile with a known inclusive prefix is
 // found, publishes this tile's inclusive prefix and returns its exclusive prefix
-// to every lane.  Every wait is bounded: after kSpinLimit polls the error flag is
+// to every lane.  Every wait is bounded: after the spin limit the error flag is
 // raised and the walk continues with what it has, so the kernel always drains.
 __device__ __forceinline__ uint64_t tile_lookback(uint64_t* desc, ScanState* st, int tile, uint64_t aggregate)
 {
     const int lane = lane_id();
     if (tile == 0) {
-        if (lane == 0) tile_store(desc, 0, kTilePrefix | aggregate);
+        if (lane == 0 && !st->mute_first_tile) tile_store(desc, 0, kTilePrefix | aggregate);
         return 0;
     }
+    const unsigned spin_limit = st->spin_limit ? st->spin_limit : kSpinLimit;
     if (lane == 0) tile_store(desc, tile, kTileAggregate | aggregate);
     uint64_t exclusive = 0;
     int base = tile - 1;
@@ -283,7 +290,7 @@ __device__ __forceinline__ uint64_t tile_lookback(uint64_t* desc, ScanState* st,
             if (t >= 0) d = tile_load(desc, t);
             const bool ready = (d >> 62) != 0;
             if (__all(ready)) break;
-            if (++spins >= kSpinLimit) { stalled = true; break; }
+            if (++spins >= spin_limit) { stalled = true; break; }
             __builtin_amdgcn_s_sleep(1);
         }
         const uint64_t has_prefix = __ballot((d >> 62) == 2);

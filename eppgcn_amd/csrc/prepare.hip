@@ -28,7 +28,7 @@ static __device__ __align__(256) unsigned char scratch[kStaticCompactScratchByte
 namespace eppgcn {
 
 // ================================================================ scan state init
-__global__ void scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles)
+__global__ void scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles, unsigned spin_limit, int mute_first_tile)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < num_tiles) desc[i] = kTileEmpty;
@@ -38,7 +38,21 @@ __global__ void scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles)
         st->counts[0] = 0;
         st->counts[1] = 0;
         st->overflow = 0;
+        st->spin_limit = spin_limit;
+        st->mute_first_tile = mute_first_tile;
     }
+}
+
+// Test knob for the stall path: with tile 0 muted every look-back runs into its (then tiny) spin limit,
+// raises the error flag and carries on, so the kernels still drain and the host sees EPPGCN_ERR_SCAN_STALLED.
+static unsigned g_scan_spin_limit = 0;
+static int g_scan_mute_first_tile = 0;
+unsigned scan_spin_limit() { return g_scan_spin_limit; }
+int scan_mute_first_tile() { return g_scan_mute_first_tile; }
+void set_scan_test_mode(unsigned spin_limit, int mute_first_tile)
+{
+    g_scan_spin_limit = spin_limit;
+    g_scan_mute_first_tile = mute_first_tile ? 1 : 0;
 }
 
 // ================================================================ path marking
@@ -670,7 +684,8 @@ static int init_scan(void* workspace, int num_tiles, hipStream_t stream)
     ScanState* st = static_cast<ScanState*>(workspace);
     uint64_t* desc = reinterpret_cast<uint64_t*>(st + 1);
     const int n = num_tiles > 0 ? num_tiles : 1;
-    hipLaunchKernelGGL(scan_init_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, st, desc, num_tiles);
+    hipLaunchKernelGGL(scan_init_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, st, desc, num_tiles,
+                       scan_spin_limit(), scan_mute_first_tile());
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }

@@ -282,6 +282,14 @@ size_t plan_scan_state_offset(long long num_parts)
     return 5 * align256(sizeof(int) * (static_cast<size_t>(num_parts > 0 ? num_parts : 0) + 1));
 }
 
+// ... and the state of the scans inside its radix sort (one state for all passes; the stall flag survives them)
+size_t plan_sort_state_offset(long long num_parts)
+{
+    const long long entries = sort_tiles(num_parts > 0 ? num_parts : 0) * kDigits;
+    return plan_scan_state_offset(num_parts) + scan_state_bytes(num_parts) +
+           2 * align256(sizeof(int) * static_cast<size_t>(entries + 1));
+}
+
 int workspace_pitch(int dim);   // aggregate.hip
 
 static int g_force_shift = 0;
@@ -304,25 +312,31 @@ int schedule_shift(int dim)
     return shift;
 }
 
-__global__ void plan_scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles)
+// keep_error: a later scan over the same state must not wipe the stall flag of an earlier one
+__global__ void plan_scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles, bool keep_error,
+                                      unsigned spin_limit, int mute_first_tile)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < num_tiles) desc[i] = kTileEmpty;
     if (i == 0) {
         st->counter = 0;
-        st->error = 0;
+        st->spin_limit = spin_limit;
+        st->mute_first_tile = mute_first_tile;
+        if (!keep_error) st->error = 0;
         st->counts[0] = st->counts[1] = 0;
         st->overflow = 0;
     }
 }
 
 // out[0..n] = exclusive prefix sums of in[0..n) (out[n] = total), with the scan state at `state`
-static int launch_exclusive_scan(const int* in, int* out, long long n, void* state, hipStream_t stream)
+static int launch_exclusive_scan(const int* in, int* out, long long n, void* state, hipStream_t stream,
+                                 bool keep_error = false)
 {
     ScanState* st = static_cast<ScanState*>(state);
     uint64_t* desc = reinterpret_cast<uint64_t*>(st + 1);
     const int tiles = static_cast<int>((n + kScanTile - 1) / kScanTile);
-    hipLaunchKernelGGL(plan_scan_init_kernel, dim3((tiles + 255) / 256), dim3(256), 0, stream, st, desc, tiles);
+    hipLaunchKernelGGL(plan_scan_init_kernel, dim3((tiles + 255) / 256), dim3(256), 0, stream, st, desc, tiles, keep_error,
+                       scan_spin_limit(), scan_mute_first_tile());
     EPPGCN_HIP(hipGetLastError());
     hipLaunchKernelGGL(exclusive_scan_kernel, dim3(tiles), dim3(kScanBlock), 0, stream, in, out, static_cast<int>(n),
                        tiles, st, desc);
@@ -351,7 +365,7 @@ static int stable_sort_by_key(unsigned* keys_a, unsigned* keys_b, int* vals_tmp,
         const int shift = pass * 8;
         hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(kSortBlock), 0, stream, kin, n, shift, tiles, hist);
         EPPGCN_HIP(hipGetLastError());
-        if (int rc = launch_exclusive_scan(hist, offsets, entries, state, stream)) return rc;
+        if (int rc = launch_exclusive_scan(hist, offsets, entries, state, stream, pass > 0)) return rc;
         hipLaunchKernelGGL(radix_scatter_kernel, dim3(tiles), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, shift,
                            tiles, offsets);
         EPPGCN_HIP(hipGetLastError());

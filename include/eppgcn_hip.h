@@ -353,6 +353,12 @@ void eppgcn_set_rounds(int rounds);
 /* The output-clear and pre-scaling kernels index with 32 bits while the matrices have fewer than 2^32
  * elements; 1 forces their 64-bit instantiations at any size.  For tests. */
 void eppgcn_set_wide_index(int on);
+/* For tests of the stall path of the look-back scans: spin_limit > 0 replaces the number of polls after
+ * which a waiting tile gives up (default 2^22); mute_first_tile != 0 makes tile 0 of every scan keep its
+ * result to itself, so that every later tile runs into the limit, raises the stall flag and carries on
+ * with what it has - the kernels still finish, the results are invalid, and the calls that read the
+ * status return EPPGCN_ERR_SCAN_STALLED.  (0, 0) restores normal operation. */
+void eppgcn_set_scan_test_mode(unsigned spin_limit, int mute_first_tile);
 /* Forces the column block size of eppgcn_build_plan to 2^shift vertices (0 = choose from the
  * feature width).  For tuning runs. */
 void eppgcn_set_plan_shift(int shift);

@@ -167,6 +167,41 @@ def test_scan_status_reports_what_asynchronous_calls_cannot(api):
     assert torch.equal(oedge[:33334], col[::3])
 
 
+def test_stalled_scans_are_reported_and_the_kernels_still_finish(api):
+    """Failure handling of the look-back scans, forced from the host: tile 0 keeps its result to itself and
+    the spin limit is tiny, so every waiting tile gives up after a few polls, flags the stall and goes on -
+    no kernel hangs, and every call that reads the status reports EPPGCN_ERR_SCAN_STALLED (-3)."""
+    import ctypes as C
+    lib = api.load()
+    n = 300000
+    mask = torch.where(torch.arange(n, device="cuda") % 3 == 0, 5, -1).int()
+    col = torch.arange(n, dtype=torch.int32, device="cuda")
+    degs = torch.full((n,), 2, dtype=torch.int32, device="cuda")
+    indptr, cols = GRAPHS["medium"]()
+    pp, p2n = co.build_part(4, indptr)
+    api.set_scan_test_mode(8, True)
+    try:
+        for call in (lambda: api.compact_back_edge(mask, col), lambda: api.split_back_part(degs, 2 * n, 1),
+                     lambda: api.build_part(2, dev(indptr)),
+                     lambda: api.build_plan(dev(pp), dev(cols), p2n.size, cols.size, indptr.size - 1, 16, part2node=dev(p2n)),
+                     lambda: api.compact_back_edge_static(mask, col, torch.empty_like(mask), torch.empty_like(col))):
+            with pytest.raises(api.EppgcnError, match="-3"):
+                call()
+        # the asynchronous form returns 0; the status call tells
+        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        nbytes = lib.eppgcn_compact_workspace_bytes(n)
+        ws = torch.empty((nbytes + 7) // 8, dtype=torch.int64, device="cuda")
+        oid, oedge = torch.empty_like(mask), torch.empty_like(col)
+        kept = torch.zeros(1, dtype=torch.int32, device="cuda")
+        p = lambda t: C.c_void_p(t.data_ptr())
+        assert lib.eppgcn_compact_back_edge(p(mask), p(col), p(oid), p(oedge), n, p(ws), nbytes, p(kept), None, stream) == 0
+        assert lib.eppgcn_scan_status(p(ws), stream) == -3 and b"stalled" in lib.eppgcn_last_error()
+    finally:
+        api.set_scan_test_mode(0, False)
+    oid, oedge, v = api.compact_back_edge(mask, col)          # and normal operation is back
+    assert v == 100000 and torch.equal(oedge[:v], col[::3])
+
+
 def test_heuristics_and_ginfo(api):
     for vn, vl in [(1000, 5000), (100000, 1000000), (419000, 13_400_000), (7, 7)]:
         ps, clamped = api.map_back_part_size(vn, vl)
