@@ -235,13 +235,14 @@ struct ScanState {
     int error;          // set to 1 when a look-back wait hit its spin limit
     int counts[2];      // results the last tile publishes (meaning depends on the kernel)
     int overflow;       // set to 1 when an output would not fit its capacity
-    unsigned spin_limit;     // polls before a wait is declared stalled (0 = kSpinLimit)
-    int mute_first_tile;     // test mode: tile 0 never publishes, so every look-back ends in a bounded stall
-    int pad;
+    int pad[3];
 };
-// What the scan-init kernels write into the two fields above (host globals behind a test knob).
-unsigned scan_spin_limit();
-int scan_mute_first_tile();
+// Scan mode, a kernel argument of every scan kernel (it stays in scalar registers: the ScanState line is
+// hammered by the tile-id atomics, so nothing else is read from it per tile): the low 31 bits are the
+// number of polls before a wait is declared stalled (0 = kSpinLimit); the top bit is the test mode in
+// which tile 0 never publishes, so that every look-back ends in a bounded stall.  The host value sits
+// behind a test knob.
+unsigned scan_mode();
 void set_scan_test_mode(unsigned spin_limit, int mute_first_tile);
 static_assert(sizeof(ScanState) == 32, "descriptor array starts 32 bytes into the workspace");
 
@@ -270,14 +271,15 @@ __device__ __forceinline__ int acquire_tile(ScanState* st, int* s_tile)
 // found, publishes this tile's inclusive prefix and returns its exclusive prefix
 // to every lane.  Every wait is bounded: after the spin limit the error flag is
 // raised and the walk continues with what it has, so the kernel always drains.
-__device__ __forceinline__ uint64_t tile_lookback(uint64_t* desc, ScanState* st, int tile, uint64_t aggregate)
+__device__ __forceinline__ uint64_t tile_lookback(uint64_t* desc, ScanState* st, int tile, uint64_t aggregate,
+                                                  unsigned mode)
 {
     const int lane = lane_id();
     if (tile == 0) {
-        if (lane == 0 && !st->mute_first_tile) tile_store(desc, 0, kTilePrefix | aggregate);
+        if (lane == 0 && (mode >> 31) == 0) tile_store(desc, 0, kTilePrefix | aggregate);
         return 0;
     }
-    const unsigned spin_limit = st->spin_limit ? st->spin_limit : kSpinLimit;
+    const unsigned spin_limit = (mode & 0x7fffffffu) ? (mode & 0x7fffffffu) : kSpinLimit;
     if (lane == 0) tile_store(desc, tile, kTileAggregate | aggregate);
     uint64_t exclusive = 0;
     int base = tile - 1;

@@ -28,7 +28,7 @@ static __device__ __align__(256) unsigned char scratch[kStaticCompactScratchByte
 namespace eppgcn {
 
 // ================================================================ scan state init
-__global__ void scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles, unsigned spin_limit, int mute_first_tile)
+__global__ void scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < num_tiles) desc[i] = kTileEmpty;
@@ -38,21 +38,16 @@ __global__ void scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles, u
         st->counts[0] = 0;
         st->counts[1] = 0;
         st->overflow = 0;
-        st->spin_limit = spin_limit;
-        st->mute_first_tile = mute_first_tile;
     }
 }
 
 // Test knob for the stall path: with tile 0 muted every look-back runs into its (then tiny) spin limit,
 // raises the error flag and carries on, so the kernels still drain and the host sees EPPGCN_ERR_SCAN_STALLED.
-static unsigned g_scan_spin_limit = 0;
-static int g_scan_mute_first_tile = 0;
-unsigned scan_spin_limit() { return g_scan_spin_limit; }
-int scan_mute_first_tile() { return g_scan_mute_first_tile; }
+static unsigned g_scan_mode = 0;
+unsigned scan_mode() { return g_scan_mode; }
 void set_scan_test_mode(unsigned spin_limit, int mute_first_tile)
 {
-    g_scan_spin_limit = spin_limit;
-    g_scan_mute_first_tile = mute_first_tile ? 1 : 0;
+    g_scan_mode = (spin_limit & 0x7fffffffu) | (mute_first_tile ? 0x80000000u : 0u);
 }
 
 // ================================================================ path marking
@@ -140,7 +135,7 @@ static_assert(kCompactItems * (kCompactBlock / kWave) == kWave, "one wave scans 
 
 __global__ __launch_bounds__(kCompactBlock) void compact_mask_kernel(
     const int* __restrict__ in_id, const int* __restrict__ in_edge, int* __restrict__ out_id,
-    int* __restrict__ out_edge, int length, int num_tiles, ScanState* st, uint64_t* desc)
+    int* __restrict__ out_edge, int length, int num_tiles, ScanState* st, uint64_t* desc, unsigned mode)
 {
     __shared__ int s_tile;
     __shared__ int s_count[kWave];
@@ -168,7 +163,7 @@ __global__ __launch_bounds__(kCompactBlock) void compact_mask_kernel(
         const int incl = wave_inclusive_scan(c);
         const int total = __shfl(incl, kWave - 1, kWave);
         s_count[lane] = incl - c;
-        const uint64_t excl = tile_lookback(desc, st, tile, static_cast<uint64_t>(total));
+        const uint64_t excl = tile_lookback(desc, st, tile, static_cast<uint64_t>(total), mode);
         if (lane == 0) {
             s_prefix = static_cast<int>(excl);
             if (tile == num_tiles - 1) st->counts[0] = static_cast<int>(excl) + total;
@@ -221,7 +216,7 @@ __global__ __launch_bounds__(kCompactBlock) void mark_compact_kernel(
     const int* __restrict__ part2node, const int* __restrict__ part_ptr, const int* __restrict__ col,
     const uint8_t* __restrict__ src_mask, uint8_t* __restrict__ ngh_mask, int* __restrict__ node_degs,
     int* __restrict__ out_id, int* __restrict__ out_edge, int num_parts, int length, int num_tiles, int is_last,
-    const int* __restrict__ tile_first, ScanState* st, uint64_t* desc)
+    const int* __restrict__ tile_first, ScanState* st, uint64_t* desc, unsigned mode)
 {
     __shared__ int s_tile;
     __shared__ int s_count[kWave];
@@ -328,7 +323,7 @@ __global__ __launch_bounds__(kCompactBlock) void mark_compact_kernel(
         const int incl = wave_inclusive_scan(cnt);
         const int total = __shfl(incl, kWave - 1, kWave);
         s_count[lane] = incl - cnt;
-        const uint64_t excl = tile_lookback(desc, st, tile, static_cast<uint64_t>(total));
+        const uint64_t excl = tile_lookback(desc, st, tile, static_cast<uint64_t>(total), mode);
         if (lane == 0) {
             s_prefix = static_cast<int>(excl);
             if (tile == num_tiles - 1) st->counts[0] = static_cast<int>(excl) + total;
@@ -443,7 +438,7 @@ constexpr int kSmallGroups = 4;     // groups per vertex up to which the owning 
 template <bool kFromRowPtr>
 __global__ __launch_bounds__(kSplitBlock) void split_groups_kernel(
     const int* __restrict__ src, int num_nodes, int part_size, int* __restrict__ part_ptr_out,
-    int* __restrict__ part2node_out, long long capacity, int num_tiles, ScanState* st, uint64_t* desc)
+    int* __restrict__ part2node_out, long long capacity, int num_tiles, ScanState* st, uint64_t* desc, unsigned mode)
 {
     __shared__ int s_tile;
     __shared__ int s_q[kSplitTile + 1];
@@ -482,7 +477,7 @@ __global__ __launch_bounds__(kSplitBlock) void split_groups_kernel(
         tile_total += s_wave[w];
     }
     if (wave == 0) {
-        const uint64_t excl = tile_lookback(desc, st, tile, tile_total);
+        const uint64_t excl = tile_lookback(desc, st, tile, tile_total, mode);
         if (lane == 0) s_tile_excl = excl;
     }
     // tile-relative q offsets and absolute g offsets of this thread's vertices
@@ -684,8 +679,7 @@ static int init_scan(void* workspace, int num_tiles, hipStream_t stream)
     ScanState* st = static_cast<ScanState*>(workspace);
     uint64_t* desc = reinterpret_cast<uint64_t*>(st + 1);
     const int n = num_tiles > 0 ? num_tiles : 1;
-    hipLaunchKernelGGL(scan_init_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, st, desc, num_tiles,
-                       scan_spin_limit(), scan_mute_first_tile());
+    hipLaunchKernelGGL(scan_init_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, st, desc, num_tiles);
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }
@@ -714,7 +708,7 @@ int launch_compact_mask(const int* in_id, int* out_id, const int* in_edge, int* 
     if (int rc = init_scan(workspace, num_tiles, stream)) return rc;
     if (num_tiles > 0) {
         hipLaunchKernelGGL(compact_mask_kernel, dim3(num_tiles), dim3(kCompactBlock), 0, stream, in_id, in_edge,
-                           out_id, out_edge, static_cast<int>(length), num_tiles, st, desc);
+                           out_id, out_edge, static_cast<int>(length), num_tiles, st, desc, scan_mode());
         EPPGCN_HIP(hipGetLastError());
         long long blocks = (length + 1023) / 1024;
         if (blocks > 2048) blocks = 2048;
@@ -799,7 +793,7 @@ int launch_mark_compact(const int* part2node, const int* part_ptr, const int* co
     EPPGCN_HIP(hipGetLastError());
     hipLaunchKernelGGL(mark_compact_kernel, dim3(num_tiles), dim3(kCompactBlock), 0, stream, part2node, part_ptr, col,
                        src_mask, ngh_mask, node_degs, out_id, out_edge, num_parts, static_cast<int>(length), num_tiles,
-                       is_last, tile_first, st, desc);
+                       is_last, tile_first, st, desc, scan_mode());
     EPPGCN_HIP(hipGetLastError());
     long long blocks = (length + 1023) / 1024;
     if (blocks > 2048) blocks = 2048;
@@ -824,10 +818,10 @@ int launch_split(bool from_row_ptr, const int* src, int num_nodes, int part_size
     }
     if (from_row_ptr)
         hipLaunchKernelGGL((split_groups_kernel<true>), dim3(num_tiles), dim3(kSplitBlock), 0, stream, src, num_nodes,
-                           part_size, part_ptr_out, part2node_out, capacity, num_tiles, st, desc);
+                           part_size, part_ptr_out, part2node_out, capacity, num_tiles, st, desc, scan_mode());
     else
         hipLaunchKernelGGL((split_groups_kernel<false>), dim3(num_tiles), dim3(kSplitBlock), 0, stream, src, num_nodes,
-                           part_size, part_ptr_out, part2node_out, capacity, num_tiles, st, desc);
+                           part_size, part_ptr_out, part2node_out, capacity, num_tiles, st, desc, scan_mode());
     EPPGCN_HIP(hipGetLastError());
     if (zero_tail) {
         long long blocks = (capacity + 1023) / 1024;

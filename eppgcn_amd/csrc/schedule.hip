@@ -91,7 +91,7 @@ constexpr int kScanItems = 8;
 constexpr int kScanTile = kScanBlock * kScanItems;
 
 __global__ __launch_bounds__(kScanBlock) void exclusive_scan_kernel(const int* __restrict__ in, int* __restrict__ out,
-                                                                   int n, int num_tiles, ScanState* st, uint64_t* desc)
+                                                                   int n, int num_tiles, ScanState* st, uint64_t* desc, unsigned mode)
 {
     __shared__ int s_tile;
     __shared__ int s_wave[kScanBlock / kWave];
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kScanBlock) void exclusive_scan_kernel(const int* _
         total += s_wave[w];
     }
     if (wave == 0) {
-        const uint64_t excl = tile_lookback(desc, st, tile, static_cast<uint64_t>(total));
+        const uint64_t excl = tile_lookback(desc, st, tile, static_cast<uint64_t>(total), mode);
         if (lane == 0) s_excl = static_cast<int>(excl);
     }
     __syncthreads();
@@ -313,15 +313,12 @@ int schedule_shift(int dim)
 }
 
 // keep_error: a later scan over the same state must not wipe the stall flag of an earlier one
-__global__ void plan_scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles, bool keep_error,
-                                      unsigned spin_limit, int mute_first_tile)
+__global__ void plan_scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles, bool keep_error)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < num_tiles) desc[i] = kTileEmpty;
     if (i == 0) {
         st->counter = 0;
-        st->spin_limit = spin_limit;
-        st->mute_first_tile = mute_first_tile;
         if (!keep_error) st->error = 0;
         st->counts[0] = st->counts[1] = 0;
         st->overflow = 0;
@@ -335,11 +332,10 @@ static int launch_exclusive_scan(const int* in, int* out, long long n, void* sta
     ScanState* st = static_cast<ScanState*>(state);
     uint64_t* desc = reinterpret_cast<uint64_t*>(st + 1);
     const int tiles = static_cast<int>((n + kScanTile - 1) / kScanTile);
-    hipLaunchKernelGGL(plan_scan_init_kernel, dim3((tiles + 255) / 256), dim3(256), 0, stream, st, desc, tiles, keep_error,
-                       scan_spin_limit(), scan_mute_first_tile());
+    hipLaunchKernelGGL(plan_scan_init_kernel, dim3((tiles + 255) / 256), dim3(256), 0, stream, st, desc, tiles, keep_error);
     EPPGCN_HIP(hipGetLastError());
     hipLaunchKernelGGL(exclusive_scan_kernel, dim3(tiles), dim3(kScanBlock), 0, stream, in, out, static_cast<int>(n),
-                       tiles, st, desc);
+                       tiles, st, desc, scan_mode());
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }
