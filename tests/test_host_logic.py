@@ -122,3 +122,46 @@ def test_driver_command_line_takes_the_reference_flags(capsys):
     assert gcn_main.main(["--backsize_mode", "net"]) == 2
     out = capsys.readouterr()
     assert out.out.startswith("||amazon0601   0.1   2") and "net" in out.err
+
+
+def test_sweep_driver_formats_the_reference_flags():
+    """The datasets x ratios x depths sweep hands the driver the flags the reference's script formats
+    (EPPGCN/bench_EPPGCN.py:41-59): automatic forward group size, `map` for the fitted regression,
+    constant 32 for `fixed_value`, `net` for the predictor (which the driver refuses)."""
+    from eppgcn_amd import bench_eppgcn as sweep, gcn_main
+    args = sweep.build_parser().parse_args([])
+    assert [d[0] for d in args.datasets] == ["cora", "citeseer", "pubmed", "youtube", "amazon", "corafull", "catalog",
+                                             "twitter", "google", "dblp"]
+    assert (args.ratios, args.layers, args.hidden) == ([0.1, 0.3, 0.5, 0.8], [3, 4, 5, 6], [16])
+    assert sweep.parse_dataset("pubmed") == ("pubmed", 500, 3)
+    assert sweep.parse_dataset("mygraph") == ("mygraph", 96, 22) and sweep.parse_dataset("g,8,3") == ("g", 8, 3)
+    with pytest.raises(Exception):
+        sweep.parse_dataset("g,8")
+    for model, mode, size in (("regression_equation", "map", 0), ("fixed_value", "constant", 32), ("SAGPG", "net", 0)):
+        args = sweep.build_parser().parse_args(["--groupsize_model", model, "--dataRoot", "/nowhere"])
+        argv = sweep.driver_arguments(args, "cora", 1433, 7, 16, 0.3, 5)
+        ns = gcn_main.build_parser().parse_args(argv)          # every flag is one the driver knows
+        assert (ns.dataset, ns.dim, ns.classes, ns.hidden, ns.layers, ns.train_ratio) == ("cora", 1433, 7, 16, 5, 0.3)
+        assert (ns.backsize_mode, ns.backsize, ns.manual_mode, ns.partSize) == (mode, size, "False", 0)
+        assert ns.dataDir == "/nowhere"
+
+
+def test_counter_summary_is_only_used_for_the_sources_it_was_taken_from(tmp_path, monkeypatch):
+    """bench.py reports measured traffic from a committed rocprofv3 summary only while the kernel sources
+    still hash to what the summary names; otherwise the field is null with the reason."""
+    import bench
+    h = bench.kernel_source_hash()
+    assert len(h) == 16 and h == bench.kernel_source_hash()
+    prof = tmp_path / "profiles"
+    prof.mkdir()
+    monkeypatch.setattr(bench, "ROOT", str(tmp_path))
+    monkeypatch.setattr(bench, "kernel_source_hash", lambda: h)
+    assert bench.measured_traffic("cfgX", "fwd")[0] is None
+    (prof / "a.md").write_text(f"    kernel_source_sha256 = {h}\n    traffic_bytes cfgX fwd = 1.5e+09\n")
+    assert bench.measured_traffic("cfgX", "fwd") == (1.5e9, "profiles/a.md")
+    assert bench.measured_traffic("cfgX", "bwd")[0] is None
+    (prof / "a.md").write_text("    kernel_source_sha256 = 0123456789abcdef\n    traffic_bytes cfgX fwd = 1.5e+09\n")
+    value, why = bench.measured_traffic("cfgX", "fwd")
+    assert value is None and "other kernel sources" in why
+    (prof / "a.md").write_text("    traffic_bytes cfgX fwd = 1.5e+09\n")
+    assert bench.measured_traffic("cfgX", "fwd")[0] is None
