@@ -59,6 +59,8 @@ def parse():
                          "reference's separate steps (same results, same time, no edge masks)")
     ap.add_argument("--no_plan", action="store_true",
                     help="process the groups in CSR order instead of the column-blocked execution plan")
+    ap.add_argument("--no_stream", action="store_true",
+                    help="keep planned launches on the group kernel instead of the plan's stream form")
     ap.add_argument("--no_workspace", action="store_true",
                     help="aggregate without the feature workspace (per-edge scale gather, no scratch)")
     ap.add_argument("--no_cpu_baseline", action="store_true")
@@ -101,16 +103,16 @@ def pipeline_figures(g, wl, kernels, x16, x22, out16, out22, args):
     w0 = graphs.uniform_weights(3, 96, 16).to(dev)
     w1 = graphs.uniform_weights(4, 16, 22).to(dev)
     x96 = graphs.normal32(1, (n, 96), dev, 5)
-    t16 = capi.update_forward(x96, w0, scale=g.degrees, ld_out=capi.feature_workspace_pitch(16))
-    t22 = capi.update_forward(x16, w1, scale=g.degrees, relu_input=True, ld_out=capi.feature_workspace_pitch(22))
+    t16 = capi.update_forward_table(x96, w0, g.degrees, plan=wl.plans.get(16))
+    t22 = capi.update_forward_table(x16, w1, g.degrees, relu_input=True, plan=wl.plans.get(22))
 
     def fwd16():
         capi.spmm_forward(None, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 32, 8,
-                          g.row_pointers, out16, workspace=t16.view(-1), plan=wl.plans.get(16), prescaled_dim=16)
+                          g.row_pointers, out16, workspace=t16, plan=wl.plans.get(16), prescaled_dim=16)
 
     def fwd22():
         capi.spmm_forward(None, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 16, 8,
-                          g.row_pointers, out22, workspace=t22.view(-1), plan=wl.plans.get(22), prescaled_dim=22)
+                          g.row_pointers, out22, workspace=t22, plan=wl.plans.get(22), prescaled_dim=22)
 
     def step():
         fwd16(); fwd22(); kernels[2][1](); kernels[3][1]()
@@ -118,10 +120,10 @@ def pipeline_figures(g, wl, kernels, x16, x22, out16, out22, args):
     fig = {"agg_ms_per_epoch_forward_prescaled": round(_event_ms(step, reps), 4)}
     f32 = 4
     dense = [
-        ("x96_w0_scaled_table", lambda: capi.update_forward(x96, w0, scale=g.degrees, ld_out=16, out=t16),
+        ("x96_w0_scaled_table", lambda: capi.update_forward_table(x96, w0, g.degrees, table=t16),
          n * (96 + 16 + 1) * f32),
-        ("relu_y1_w1_scaled_table", lambda: capi.update_forward(x16, w1, scale=g.degrees, relu_input=True, ld_out=32,
-                                                                out=t22), n * (16 + 32 + 1) * f32),
+        ("relu_y1_w1_scaled_table", lambda: capi.update_forward_table(x16, w1, g.degrees, relu_input=True, table=t22),
+         n * (16 + 32 + 1) * f32),
         ("g1_w1t_relu_masked", lambda: capi.update_backward_input(x22, w1, relu_ref=x16), n * (22 + 16 + 16) * f32),
         ("x96t_g0_weight_grad", lambda: capi.update_backward_weight(x96, x16), n * (96 + 16) * f32),
         ("relu_y1t_g1_weight_grad", lambda: capi.update_backward_weight(x16, x22, relu_input=True), n * (16 + 22) * f32),
@@ -176,9 +178,14 @@ def main():
     dy22 = graphs.normal32(1, (n, 22), dev, 2) * wl.train_mask[:, None]
     dy16 = graphs.normal32(1, (n, 16), dev, 3) * wl.ngh_masks[0][:, None]
     out16, out22 = torch.empty_like(x16), torch.empty_like(x22)
-    ws16, ws22 = ((capi.feature_workspace(n, 16, dev), capi.feature_workspace(n, 22, dev))
-                  if not args.no_workspace else (None, None))
     p_last, p_first = wl.paths[1], wl.paths[0]
+    # one workspace per width, shared by the forward and the backward launch of that width: the pre-scaled
+    # table and, behind it, room for the partial sums of either plan's stream form
+    ws16, ws22 = ((capi.feature_workspace(n, 16, dev, (wl.plans.get(16), p_first.plan)),
+                   capi.feature_workspace(n, 22, dev, (wl.plans.get(22), p_last.plan)))
+                  if not args.no_workspace else (None, None))
+    if args.no_stream:
+        capi.set_stream_mode(False)
     if args.team:
         capi.set_team_size(args.team)
     if args.rounds:
@@ -286,7 +293,8 @@ def main():
                    "kept_edges": [p.valid_len for p in wl.paths],
                    "backward_groups": [p.num_parts for p in wl.paths], "max_degree": g.stats()["max_degree"],
                    "feature_workspace": not args.no_workspace,
-                   "column_blocked_plan": bool(wl.plans)},
+                   "column_blocked_plan": bool(wl.plans),
+                   "stream_form": bool(wl.plans) and not args.no_stream and not args.no_workspace},
         "agg_ms_per_epoch": round(ms_per_step, 4), "alg_bytes_per_epoch": bytes_epoch,
         "pct_of_peak_hbm": round(value / PEAK_HBM_GBS * 100, 2),
         "value_is": "algorithmic (gather-model) bytes of the epoch / wall time; not measured HBM traffic",
@@ -374,13 +382,14 @@ def gather_probe(dev):
     part2node = torch.arange(n, dtype=torch.int32, device=dev)
     ones = torch.ones(n, device=dev)
     for dim in (16, 32):
-        table = torch.empty(n, capi.feature_workspace_pitch(dim), device=dev).normal_()
+        table = torch.empty(n, capi.feature_workspace_pitch(dim), device=dev).normal_()     # n is a multiple of 4096
+        rows = capi.feature_workspace_rows(n, dev)
         out = torch.empty(n, dim, device=dev)
         for _ in range(3):
             capi.spmm_forward(None, col, ones, part_ptr, part2node, 1, 32, 8, None, out, workspace=table.view(-1),
                               prescaled_dim=dim)
         torch.cuda.synchronize()
-        assert torch.equal(out, table[col.long()][:, :dim])
+        assert torch.equal(out, table[rows[col.long()]][:, :dim])
         del table, out
 
 

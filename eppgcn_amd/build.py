@@ -20,7 +20,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 OBJ_DIR = os.path.join(HERE, "csrc", "_obj")
 HIP_LIB = os.path.join(LIB_DIR, "libeppgcn_hip.so")
-HIP_SOURCES = ["aggregate.hip", "prepare.hip", "schedule.hip", "update.hip", "capi.hip"]
+HIP_SOURCES = ["aggregate.hip", "stream.hip", "prepare.hip", "schedule.hip", "update.hip", "capi.hip"]
 HIP_HEADERS = ["common.hpp", os.path.join(ROOT, "include", "eppgcn_hip.h")]
 ARCH = "gfx950"
 

@@ -27,10 +27,12 @@ EXPORTS = [
     "eppgcn_mark_compact_workspace_bytes", "eppgcn_mark_compact", "eppgcn_set_plan_length_classes",
     "eppgcn_mark_gathered_rows", "eppgcn_set_wide_index", "eppgcn_wave64_back_part_size",
     "eppgcn_compact_back_edge_static", "eppgcn_compact_back_edge_static_max_length",
-    "eppgcn_auto_back_part_size", "eppgcn_scan_status", "eppgcn_build_plan_status", "eppgcn_set_scan_test_mode",
+    "eppgcn_auto_back_part_size", "eppgcn_scan_status", "eppgcn_plan_status", "eppgcn_set_scan_test_mode",
+    "eppgcn_plan_workspace_floats", "eppgcn_set_stream_mode", "eppgcn_last_call_used_stream",
+    "eppgcn_update_forward_table", "eppgcn_feature_workspace_row",
 ]
 
-ABI_VERSION = 12      # what eppgcn_abi_version() of a matching library returns
+ABI_VERSION = 13      # what eppgcn_abi_version() of a matching library returns
 
 _lib = None
 
@@ -60,7 +62,7 @@ def load():
     lib.eppgcn_plan_recommended.restype = i
     lib.eppgcn_plan_bytes.argtypes = [i64, i64, i64]
     lib.eppgcn_plan_bytes.restype = sz
-    lib.eppgcn_plan_workspace_bytes.argtypes = [i64]
+    lib.eppgcn_plan_workspace_bytes.argtypes = [i64, i64]
     lib.eppgcn_plan_workspace_bytes.restype = sz
     lib.eppgcn_build_plan.argtypes = [p, p, p, p, i, i64, i, i, i, p, sz, p, sz, p]
     lib.eppgcn_build_plan.restype = i
@@ -87,8 +89,13 @@ def load():
     lib.eppgcn_auto_back_part_size.restype = i
     lib.eppgcn_scan_status.argtypes = [p, p]
     lib.eppgcn_scan_status.restype = i
-    lib.eppgcn_build_plan_status.argtypes = [p, i, p]
-    lib.eppgcn_build_plan_status.restype = i
+    lib.eppgcn_plan_status.argtypes = [p, i, i64, i, C.POINTER(i64), p]
+    lib.eppgcn_plan_status.restype = i
+    lib.eppgcn_plan_workspace_floats.argtypes = [p, i64, i]
+    lib.eppgcn_plan_workspace_floats.restype = sz
+    lib.eppgcn_set_stream_mode.argtypes = [i]
+    lib.eppgcn_set_stream_mode.restype = None
+    lib.eppgcn_last_call_used_stream.restype = i
     lib.eppgcn_split_back_part.argtypes = [p, i, i, p, i64, p, sz, p, C.POINTER(i64), C.POINTER(i64), p]
     lib.eppgcn_build_part.argtypes = [p, i, i, p, p, i64, p, sz, p, C.POINTER(i64), p]
     lib.eppgcn_get_ginfo.argtypes = [p, i64, i64, p, C.POINTER(C.c_float), p]
@@ -121,6 +128,10 @@ def load():
     lib.eppgcn_update_supported.argtypes = [i, i]
     lib.eppgcn_update_supported.restype = i
     lib.eppgcn_update_forward.argtypes = [p, i, p, p, p, i, i64, i, i, p]
+    lib.eppgcn_update_forward_table.argtypes = [p, sz, p, p, p, i, i64, i, i, p]
+    lib.eppgcn_update_forward_table.restype = i
+    lib.eppgcn_feature_workspace_row.argtypes = [i64]
+    lib.eppgcn_feature_workspace_row.restype = i64
     lib.eppgcn_update_backward_input.argtypes = [p, p, p, p, i64, i, i, p]
     lib.eppgcn_update_workspace_bytes.argtypes = [i64, i, i]
     lib.eppgcn_update_workspace_bytes.restype = sz
@@ -197,6 +208,33 @@ def update_forward(x, w, scale=None, relu_input=False, ld_out=None, out=None):
     return out
 
 
+def update_forward_table(x, w, scale, relu_input=False, table=None, plan=None):
+    """scale[r] * act(x) @ w written as the pre-scaled feature workspace of the aggregation calls (their
+    ``feats=None`` form): padded rows in the workspace's row order.  ``plan``: leave room for the partial
+    sums of that plan's stream form behind the table."""
+    lib = load()
+    _dev(x, torch.float32, "x"); _dev(w, torch.float32, "w"); _dev(scale, torch.float32, "scale")
+    n, k = x.shape
+    if w.dim() != 2 or w.shape[0] != k:
+        raise EppgcnError("w must be [in_dim, out_dim]")
+    m = w.shape[1]
+    if scale.numel() != n:
+        raise EppgcnError("scale must have one entry per row")
+    if table is None:
+        table = feature_workspace(n, m, x.device, plan)
+    elif table.numel() < lib.eppgcn_feature_workspace_floats(n, m):
+        raise EppgcnError("table is too small")
+    _check(lib.eppgcn_update_forward_table(_ptr(table), table.numel(), _ptr(x), _ptr(w), _ptr(scale), int(bool(relu_input)), n, k, m,
+                                           _stream()))
+    return table
+
+
+def feature_workspace_rows(num_nodes: int, device) -> torch.Tensor:
+    """int64[num_nodes]: the row of a separate feature workspace that holds each vertex."""
+    r = torch.arange(int(num_nodes), dtype=torch.int64, device=device)
+    return r ^ ((r >> 5) & 4095)
+
+
 def update_backward_input(g, w, relu_ref=None):
     """(g @ w.T), zeroed where relu_ref <= 0 -> [N, in_dim]."""
     lib = load()
@@ -230,29 +268,54 @@ def update_backward_weight(x, g, relu_input=False):
     return d_w
 
 
-def _feature_workspace(workspace, feats):
+def _feature_workspace(workspace, feats, plan=None):
     """None -> per-edge scale gather (no scratch); True -> allocate; a tensor -> use it (it may be
     `feats` itself, which is then overwritten with the scaled features)."""
     if workspace is None or workspace is False:
         return None
     if workspace is True:
-        return feature_workspace(feats.shape[0], feats.shape[1], feats.device)
+        return feature_workspace(feats.shape[0], feats.shape[1], feats.device, plan)
     _dev(workspace, torch.float32, "workspace")
     return workspace
 
 
-def feature_workspace(num_nodes: int, dim: int, device):
-    """A scratch tensor large enough for the pre-scaled, padded copy of [num_nodes, dim] features."""
-    return torch.empty(load().eppgcn_feature_workspace_floats(int(num_nodes), int(dim)), dtype=torch.float32,
-                       device=device)
+def feature_workspace(num_nodes: int, dim: int, device, plan=None):
+    """A scratch tensor large enough for the pre-scaled, padded copy of [num_nodes, dim] features and,
+    with ``plan``, for the partial sums of a call through the plan's stream form behind it."""
+    lib = load()
+    floats = lib.eppgcn_feature_workspace_floats(int(num_nodes), int(dim))
+    plans = [] if plan is None else [plan] if isinstance(plan, Plan) else list(plan)     # several: room for any of them
+    for pl in plans:
+        if pl is not None:
+            floats = max(floats, lib.eppgcn_plan_workspace_floats(C.c_void_p(pl.base_ptr), int(num_nodes), int(dim)))
+    return torch.empty(floats, dtype=torch.float32, device=device)
+
+
+def last_call_used_stream() -> bool:
+    """Whether this thread's last aggregation call ran the stream form of its plan."""
+    return bool(load().eppgcn_last_call_used_stream())
+
+
+def set_stream_mode(on: bool):
+    """False keeps planned calls on the group kernel (comparisons); True (default) allows the stream form."""
+    load().eppgcn_set_stream_mode(int(bool(on)))
+
+
+STREAM_WAVE = 512      # slots a wave of the stream kernel takes
+STREAM_CHUNK = 32      # piece ends are counted per chunk of this many slots
 
 
 class Plan:
     """A column-blocked execution plan (device buffer + the sizes it was built for)."""
 
-    def __init__(self, buffer, base_ptr, num_parts, num_slots, num_nodes):
+    def __init__(self, buffer, base_ptr, num_parts, num_slots, num_nodes, partial_rows=0):
         self.buffer, self.base_ptr, self.num_parts, self.num_slots = buffer, base_ptr, num_parts, num_slots
         self.num_nodes = num_nodes
+        self.partial_rows = partial_rows      # partial sums of a call through the stream form (0: no stream form)
+
+    @property
+    def padded_slots(self):
+        return (self.num_slots + STREAM_WAVE - 1) // STREAM_WAVE * STREAM_WAVE
 
     def _offsets(self):
         def al(x):
@@ -263,13 +326,33 @@ class Plan:
         o4 = o3 + al(4 * ((self.num_nodes + 31) // 32))
         return off, o1, o2, o3, o4
 
-    def view(self):
-        """(ptr, row, flags, col) as torch tensors, for tests."""
+    def view(self, raw_col=False):
+        """(ptr, row, flags, col) as torch tensors, for tests.  ``raw_col``: keep bit 31 of the column ids,
+        which marks the last slot of every piece."""
         p, s = self.num_parts, self.num_slots
         off, o1, o2, o3, o4 = self._offsets()
         raw = self.buffer.view(torch.uint8)
+        col = raw[o4: o4 + 4 * s].view(torch.int32)
         return (raw[off: off + 4 * (p + 1)].view(torch.int32), raw[o1: o1 + 4 * p].view(torch.int32),
-                raw[o2: o2 + p], raw[o4: o4 + 4 * s].view(torch.int32))
+                raw[o2: o2 + p], col if raw_col else col & 0x7fffffff)
+
+    def stream_view(self):
+        """The stream form as a dict of torch tensors (header, col with padding, erow, cev, wtail, touched, frow,
+        fptr), for tests."""
+        def al(x):
+            return (x + 255) // 256 * 256
+        p, n, sp = self.num_parts, self.num_nodes, self.padded_slots
+        *_, o4 = self._offsets()
+        raw = self.buffer.view(torch.uint8)
+        words = (n + 31) // 32
+        o = o4 + al(4 * sp)
+        out = {"col": raw[o4: o4 + 4 * sp].view(torch.int32), "header": raw[o: o + 64].view(torch.int32)}
+        o += al(64)
+        for name, count in (("erow", p), ("cev", sp // STREAM_CHUNK + 1), ("wtail", sp // STREAM_WAVE),
+                            ("touched", words), ("frow", n), ("fptr", n + 1)):
+            out[name] = raw[o: o + 4 * count].view(torch.int32)
+            o += al(4 * count)
+        return out
 
     def single_rows(self):
         """bool[num_nodes]: rows recorded as one non-empty group (skipped by the output clear), for tests."""
@@ -299,14 +382,17 @@ def build_plan(part_ptr, column_index, num_parts: int, num_slots: int, num_nodes
         raise EppgcnError("column_index is shorter than num_slots")
     nbytes = lib.eppgcn_plan_bytes(int(num_parts), int(num_slots), int(num_nodes))
     buf, base = _aligned_buffer(nbytes, part_ptr.device)
-    wbytes = lib.eppgcn_plan_workspace_bytes(int(num_parts))
+    wbytes = lib.eppgcn_plan_workspace_bytes(int(num_parts), int(num_slots))
     ws, wbase = _aligned_buffer(wbytes, part_ptr.device)
     _check(lib.eppgcn_build_plan(_ptr(part_ptr), _ptr(column_index), _ptr(part2node), _ptr(ids), int(num_parts),
                                  int(num_slots), int(num_nodes), int(dim), int(block_shift), C.c_void_p(base), nbytes,
                                  C.c_void_p(wbase), wbytes, _stream()))
-    # synchronises (the workspace is released on return) and refuses a plan whose scan stalled
-    _check(lib.eppgcn_build_plan_status(C.c_void_p(wbase), int(num_parts), _stream()))
-    return Plan(buf, base, int(num_parts), int(num_slots), int(num_nodes))
+    # synchronises (the workspace is released on return), refuses a plan whose scan stalled and lets the
+    # library know the plan's stream form
+    partial = C.c_int64(0)
+    _check(lib.eppgcn_plan_status(C.c_void_p(base), int(num_parts), int(num_slots), int(num_nodes), C.byref(partial),
+                                  _stream()))
+    return Plan(buf, base, int(num_parts), int(num_slots), int(num_nodes), int(partial.value))
 
 
 def plan_recommended(num_nodes: int, dim: int) -> bool:
@@ -348,7 +434,7 @@ def spmm_forward(feats, column_index, degrees, part_ptr, part2node, part_size=32
     if out is None:
         out = torch.empty_like(feats)
     fn = lib.eppgcn_spmm_backward if backward else lib.eppgcn_spmm_forward
-    ws = workspace if feats is None else _feature_workspace(workspace, feats)
+    ws = workspace if feats is None else _feature_workspace(workspace, feats, plan)
     _check(fn(_ptr(out), _ptr(feats), _ptr(row_pointers), _ptr(column_index), _ptr(degrees), _ptr(part_ptr),
               _ptr(part2node), n, dim, num_parts, part_size, dim_worker, warp_per_block, _ptr(ws),
               0 if ws is None else ws.numel(), _plan_ptr(plan, num_parts, n), _stream()))
@@ -380,7 +466,7 @@ def ours_backward(d_output, ids, part_pointer, edge_list, degrees, num_parts, pa
         raise EppgcnError("part_pointer needs num_parts + 1 entries")
     if out is None:
         out = torch.empty_like(d_output)
-    ws = _feature_workspace(workspace, d_output)
+    ws = _feature_workspace(workspace, d_output, plan)
     _check(lib.eppgcn_ours_backward(_ptr(out), _ptr(d_output), _ptr(ids), _ptr(part_pointer), _ptr(edge_list),
                                     _ptr(degrees), n, dim, int(num_parts), part_size, layer, blockx, blocky,
                                     _ptr(ws), 0 if ws is None else ws.numel(),

@@ -158,13 +158,15 @@ template <class Index>
 __global__ __launch_bounds__(256) void scale_rows_kernel(float* __restrict__ dst, const float* __restrict__ src,
                                                          const float* __restrict__ scale,
                                                          const uint32_t* __restrict__ rows, Index total_vecs,
-                                                         Index vecs_per_row, Index dim, bool pairs)
+                                                         Index vecs_per_row, Index dim, bool pairs, unsigned swz_mask)
 {
     const Index stride = static_cast<Index>(gridDim.x) * blockDim.x;
     for (Index i = static_cast<Index>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs; i += stride) {
         const Index r = i / vecs_per_row;
         if (row_wanted(rows, r)) {
             const Index c0 = (i - r * vecs_per_row) * 4;
+            // row r of the table lives at swizzled_row(r) (the mask is 0 for a table in vertex order)
+            const size_t at = static_cast<size_t>(swizzled_row(static_cast<unsigned>(r), swz_mask)) * vecs_per_row * 4 + c0;
             const float s = scale[r];
             const float* row = src + static_cast<size_t>(r) * dim;
             float4 v;
@@ -178,7 +180,7 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(float* __restrict__ dst
                 v.z = c0 + 2 < dim ? s * row[c0 + 2] : 0.f;
                 v.w = c0 + 3 < dim ? s * row[c0 + 3] : 0.f;
             }
-            *reinterpret_cast<float4*>(dst + static_cast<size_t>(i) * 4) = v;
+            *reinterpret_cast<float4*>(dst + at) = v;
         }
         if (total_vecs - i <= stride) break;      // the next index would run past the end (and could wrap)
     }
@@ -203,7 +205,7 @@ template <class Index>
 __global__ __launch_bounds__(256) void scale_rows_flat4_kernel(float4* dst, const float4* src,
                                                                const float* __restrict__ scale,
                                                                const uint32_t* __restrict__ rows, Index total_vecs,
-                                                               Index vecs_per_row)
+                                                               Index vecs_per_row, unsigned swz_mask)
 {
     const Index stride = static_cast<Index>(gridDim.x) * blockDim.x;
     for (Index i = static_cast<Index>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs; i += stride) {
@@ -212,7 +214,7 @@ __global__ __launch_bounds__(256) void scale_rows_flat4_kernel(float4* dst, cons
             const float s = scale[r];
             float4 v = src[i];
             v.x *= s; v.y *= s; v.z *= s; v.w *= s;
-            dst[i] = v;
+            dst[static_cast<size_t>(swizzled_row(static_cast<unsigned>(r), swz_mask)) * vecs_per_row + (i - r * vecs_per_row)] = v;
         }
         if (total_vecs - i <= stride) break;
     }
@@ -237,7 +239,7 @@ template <int VW, int OVW, int TS, int CPL, int U, bool kPrescaled, class Groups
 __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
     float* __restrict__ out, const float* __restrict__ in, const int* __restrict__ col,
     const float* __restrict__ scale, Groups groups, int num_parts, int rounds, int chunks, int ld_in, int width_out,
-    int ld_out)
+    int ld_out, unsigned swz_mask)
 {
     constexpr int TPW = kWave / TS;                  // teams (= groups) per wave and round
     constexpr int kPasses = kStageCap / kWave;       // load instructions per staging pass
@@ -345,7 +347,7 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
 #pragma unroll
                         for (int r = 0; r < kPasses / 2; ++r) {
                             const int i = lane + (half * (kPasses / 2) + r) * kWave;
-                            sc[r] = i < cn_new ? scale[c[r]] : 0.f;
+                            sc[r] = i < cn_new ? scale[c[r] & kStreamIdMask] : 0.f;
                         }
 #pragma unroll
                         for (int r = 0; r < kPasses / 2; ++r) {
@@ -377,9 +379,10 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
                 for (int u = 0; u < U; ++u) {
                     const bool ok = i + u < hi;
                     const int word = stage_index(ok ? i + u - win_beg : 0);
-                    const int c = my_col[word];
+                    const int c = my_col[word] & kStreamIdMask;     // a plan's ids carry a flag in bit 31
                     if constexpr (!kPrescaled) w[u] = ok ? s_row * my_scale[word] : 0.f;
-                    const float* src = in + static_cast<size_t>(c) * ld_in;
+                    // a separate pre-scaled table holds its rows in swizzled order (mask 0: vertex order)
+                    const float* src = in + static_cast<size_t>(kPrescaled ? swizzled_row(c, swz_mask) : c) * ld_in;
 #pragma unroll
                     for (int k = 0; k < CPL; ++k) {
                         const int ch = tl + k * TS;
@@ -553,6 +556,7 @@ struct AggShape {
     int ld_in;       // input row pitch (floats)
     int width_out;   // output columns written
     int ld_out;      // output row pitch (floats)
+    unsigned swz_mask;   // kRowSwizzleMask when the input is a separate pre-scaled table, else 0
 };
 
 template <int VW, int OVW, int TS, int CPL, int U, bool kPrescaled, class Groups>
@@ -581,7 +585,7 @@ static hipError_t launch_one(float* out, const float* in, const int* col, const 
     const long long grid = (num_parts + groups_per_block - 1) / groups_per_block;
     hipLaunchKernelGGL((aggregate_kernel<VW, OVW, TS, CPL, U, kPrescaled, Groups>),
                        dim3(static_cast<unsigned>(grid)), dim3(kAggBlock), 0, stream, out, in, col, scale, g,
-                       num_parts, rounds, sh.chunks, sh.ld_in, sh.width_out, sh.ld_out);
+                       num_parts, rounds, sh.chunks, sh.ld_in, sh.width_out, sh.ld_out, sh.swz_mask);
     return hipGetLastError();
 }
 
@@ -635,9 +639,10 @@ int workspace_pitch(int dim)
     return (dim + 7) / 8 * 8;
 }
 
+// a separate table holds its rows in swizzled order, whole blocks of 4096 rows
 size_t feature_workspace_floats(long long num_nodes, int dim)
 {
-    return static_cast<size_t>(num_nodes) * static_cast<size_t>(workspace_pitch(dim));
+    return static_cast<size_t>(swizzle_padded_rows(num_nodes)) * static_cast<size_t>(workspace_pitch(dim));
 }
 
 // Restricted form of the pass for a sparse row set: a wave looks at 64 rows at a time, collects those
@@ -647,7 +652,8 @@ size_t feature_workspace_floats(long long num_nodes, int dim)
 __global__ __launch_bounds__(256) void scale_listed_rows_kernel(float* __restrict__ dst, const float* __restrict__ src,
                                                                 const float* __restrict__ scale,
                                                                 const uint32_t* __restrict__ rows, unsigned num_rows,
-                                                                unsigned vecs_per_row, unsigned dim, bool pairs)
+                                                                unsigned vecs_per_row, unsigned dim, bool pairs,
+                                                                unsigned swz_mask)
 {
     __shared__ int lists[4][kWave];
     int* list = lists[threadIdx.x / kWave];
@@ -676,40 +682,46 @@ __global__ __launch_bounds__(256) void scale_listed_rows_kernel(float* __restric
                 v.z = c0 + 2 < dim ? s * row[c0 + 2] : 0.f;
                 v.w = c0 + 3 < dim ? s * row[c0 + 3] : 0.f;
             }
-            *reinterpret_cast<float4*>(dst + r * (static_cast<size_t>(vecs_per_row) * 4) + c0) = v;
+            *reinterpret_cast<float4*>(dst + static_cast<size_t>(swizzled_row(static_cast<unsigned>(r), swz_mask)) *
+                                                 (static_cast<size_t>(vecs_per_row) * 4) + c0) = v;
         }
     }
 }
 
 template <class Index>
 static void launch_scale_rows_typed(float* dst, const float* src, const float* scale, const uint32_t* rows,
-                                    long long num_nodes, int dim, int ld_dst, hipStream_t stream)
+                                    long long num_nodes, int dim, int ld_dst, unsigned swz_mask, hipStream_t stream)
 {
     auto grid_for = [](long long threads) {
         long long blocks = (threads + 255) / 256;
         if (blocks > 256 * 32) blocks = 256 * 32;
         return dim3(static_cast<unsigned>(blocks < 1 ? 1 : blocks));
     };
-    if (dst == src || ld_dst == dim) {
+    const bool in_place = dst == src;
+    if (in_place || ld_dst == dim) {
         const long long total = num_nodes * dim;
         if (dim % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0) {
             hipLaunchKernelGGL((scale_rows_flat4_kernel<Index>), grid_for(total / 4), dim3(256), 0, stream,
                                reinterpret_cast<float4*>(dst), reinterpret_cast<const float4*>(src), scale, rows,
-                               static_cast<Index>(total / 4), static_cast<Index>(dim / 4));
+                               static_cast<Index>(total / 4), static_cast<Index>(dim / 4), in_place ? 0u : swz_mask);
             return;
         }
-        hipLaunchKernelGGL((scale_rows_flat_kernel<Index>), grid_for(total), dim3(256), 0, stream, dst, src, scale, rows,
-                           static_cast<Index>(total), static_cast<Index>(dim));
-    } else {
-        const long long vecs = num_nodes * (ld_dst / 4);
-        hipLaunchKernelGGL((scale_rows_kernel<Index>), grid_for(vecs), dim3(256), 0, stream, dst, src, scale, rows,
-                           static_cast<Index>(vecs), static_cast<Index>(ld_dst / 4), static_cast<Index>(dim),
-                           dim % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 8 == 0);
+        if (in_place || swz_mask == 0) {
+            hipLaunchKernelGGL((scale_rows_flat_kernel<Index>), grid_for(total), dim3(256), 0, stream, dst, src, scale, rows,
+                               static_cast<Index>(total), static_cast<Index>(dim));
+            return;
+        }
+        // a separate table without padding whose source is not 16-byte aligned: the general kernel below
     }
+    const long long vecs = num_nodes * (ld_dst / 4);
+    hipLaunchKernelGGL((scale_rows_kernel<Index>), grid_for(vecs), dim3(256), 0, stream, dst, src, scale, rows,
+                       static_cast<Index>(vecs), static_cast<Index>(ld_dst / 4), static_cast<Index>(dim),
+                       dim % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 8 == 0, swz_mask);
 }
 
+// swz_mask: kRowSwizzleMask for a separate table (rows in swizzled order), 0 for one in vertex order
 static int launch_scale_rows(float* dst, const float* src, const float* scale, const uint32_t* rows, int num_nodes,
-                             int dim, int ld_dst, hipStream_t stream)
+                             int dim, int ld_dst, unsigned swz_mask, hipStream_t stream)
 {
     if (static_cast<long long>(num_nodes) * dim == 0) return kOk;
     if (rows && ld_dst % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 && !force_wide_index()) {
@@ -717,13 +729,14 @@ static int launch_scale_rows(float* dst, const float* src, const float* scale, c
         if (blocks > 256 * 16) blocks = 256 * 16;
         hipLaunchKernelGGL(scale_listed_rows_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, dst, src,
                            scale, rows, static_cast<unsigned>(num_nodes), static_cast<unsigned>(ld_dst / 4),
-                           static_cast<unsigned>(dim), dim % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 8 == 0);
+                           static_cast<unsigned>(dim), dim % 2 == 0 && reinterpret_cast<uintptr_t>(src) % 8 == 0,
+                           dst == src ? 0u : swz_mask);
         EPPGCN_HIP(hipGetLastError());
         return kOk;
     }
-    const long long elems = static_cast<long long>(num_nodes) * (ld_dst > dim ? ld_dst : dim);
-    if (elems < (1ll << 32) && !force_wide_index()) launch_scale_rows_typed<unsigned>(dst, src, scale, rows, num_nodes, dim, ld_dst, stream);
-    else launch_scale_rows_typed<unsigned long long>(dst, src, scale, rows, num_nodes, dim, ld_dst, stream);
+    const long long elems = swizzle_padded_rows(num_nodes) * (ld_dst > dim ? ld_dst : dim);
+    if (elems < (1ll << 32) && !force_wide_index()) launch_scale_rows_typed<unsigned>(dst, src, scale, rows, num_nodes, dim, ld_dst, swz_mask, stream);
+    else launch_scale_rows_typed<unsigned long long>(dst, src, scale, rows, num_nodes, dim, ld_dst, swz_mask, stream);
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }
@@ -738,6 +751,53 @@ static int vector_width(int pitch, int width, const void* p)
 
 // workspace: nullptr (per-edge scale gather), the input pointer itself (scaled in place, pitch dim)
 // or a separate buffer of feature_workspace_floats() floats (padded pitch).
+bool stream_covers(int num_nodes, int dim, int ld_in, const float* table);                     // stream.hip
+int launch_aggregate_stream(float* out, float* partial, const float* table, const int* scol, const StreamView& sv,
+                            const StreamInfo& info, const float* scale, int num_nodes, int dim, int ld_in,
+                            hipStream_t stream);
+
+// The stream form of the plan is used when the host knows it (eppgcn_plan_status has read its header), the
+// rows are gathered from a separate pre-scaled workspace, the shape fits the stream kernel and the workspace has
+// room for the partial sums behind the table.
+static bool stream_usable(const StreamInfo* info, const float* in, const float* workspace, size_t workspace_floats,
+                          int num_nodes, int dim, int num_parts)
+{
+    if (!info || !workspace || workspace == in) return false;
+    if (!info->header.valid || info->num_parts != num_parts || info->num_nodes != num_nodes) return false;
+    const int ld = workspace_pitch(dim);
+    if (!stream_covers(num_nodes, dim, ld, workspace)) return false;
+    return workspace_floats >= (static_cast<size_t>(swizzle_padded_rows(num_nodes)) + static_cast<size_t>(info->header.num_partials)) * ld;
+}
+
+// which kernel family the calling thread's last planned aggregation call ran (1 = stream form)
+static thread_local int g_last_used_stream = 0;
+int last_call_used_stream() { return g_last_used_stream; }
+
+static int aggregate_stream_call(float* out, const float* in, const int* scol, const float* scale, const StreamInfo& info,
+                                 const void* plan, int num_nodes, int dim, float* workspace, hipStream_t stream,
+                                 double* sink, double* sink2, const uint32_t* gathered_rows)
+{
+    const StreamView sv = stream_view(const_cast<void*>(plan), info.num_parts, info.num_slots, info.num_nodes);
+    const int ld = workspace_pitch(dim);
+    g_last_used_stream = 1;
+    // only rows without any slot are left to a clear: every other row is written by the stream kernel or the fix-up
+    if (info.header.empty_rows > 0) {
+        KernelTimer timer(stream, phase_sink(0));
+        if (2ll * info.header.empty_rows <= num_nodes) {
+            if (int rc = launch_zero_rows_unless(out, sv.touched, num_nodes, dim, stream)) return rc;
+        } else {
+            if (int rc = launch_zero_words(out, static_cast<size_t>(num_nodes) * dim, stream)) return rc;
+        }
+    }
+    if (in) {
+        KernelTimer timer(stream, phase_sink(1));
+        if (int rc = launch_scale_rows(workspace, in, scale, gathered_rows, num_nodes, dim, ld, kRowSwizzleMask, stream)) return rc;
+    }
+    KernelTimer timer(stream, sink, sink2);
+    return launch_aggregate_stream(out, workspace + static_cast<size_t>(swizzle_padded_rows(num_nodes)) * ld, workspace, scol, sv, info, scale,
+                                   num_nodes, dim, ld, stream);
+}
+
 template <class Groups>
 static int aggregate_dispatch(float* out, const float* in, const int* col, const float* scale, Groups g,
                               int num_nodes, int dim, int num_parts, int group_size, float* workspace,
@@ -746,6 +806,7 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
 {
     const bool prescaled = workspace != nullptr;
     int ld_in = dim;
+    g_last_used_stream = 0;
     // rows the kernel writes with one plain store (a plan knows them) need no clearing; with fewer
     // groups than half the rows most rows have no group at all and the plain fill is the faster clear
     {
@@ -757,12 +818,14 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
         }
     }
     if (num_parts == 0) return kOk;
+    // a separate table (not the input scaled in place) holds its rows in swizzled order
+    const unsigned swz_mask = (prescaled && workspace != in) ? kRowSwizzleMask : 0u;
     if (prescaled) {
         // in == nullptr: the caller (the dense update) already wrote the scaled, padded rows
         ld_in = workspace == in ? dim : workspace_pitch(dim);
         if (in) {
             KernelTimer timer(stream, phase_sink(1));
-            if (int rc = launch_scale_rows(workspace, in, scale, gathered_rows, num_nodes, dim, ld_in, stream)) return rc;
+            if (int rc = launch_scale_rows(workspace, in, scale, gathered_rows, num_nodes, dim, ld_in, swz_mask, stream)) return rc;
         }
         in = workspace;
     }
@@ -788,6 +851,7 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
         sh.ld_in = ld_in;
         sh.width_out = dim - c0 < slab ? dim - c0 : slab;
         sh.ld_out = dim;
+        sh.swz_mask = swz_mask;
         hipError_t e;
 #define EPPGCN_SLAB(VW_, OVW_) slab_either<VW_, OVW_>(prescaled, out + c0, in + c0, col, scale, g, num_parts, sh, stream)
         if (vw == 4 && ovw_eff == 4) e = EPPGCN_SLAB(4, 4);
@@ -805,11 +869,15 @@ static int aggregate_dispatch(float* out, const float* in, const int* col, const
 // plan: nullptr, or an execution plan built for exactly these groups.
 int aggregate_forward_groups(float* out, const float* in, const int* col, const float* scale,
                              const int* part_ptr, const int* part2node, const void* plan, int num_nodes, int dim,
-                             int num_parts, int group_size, float* workspace, hipStream_t stream, double* sink,
-                             double* sink2)
+                             int num_parts, int group_size, float* workspace, size_t workspace_floats,
+                             hipStream_t stream, double* sink, double* sink2)
 {
     if (plan && num_parts > 0) {
         const PlanView v = plan_view(const_cast<void*>(plan), num_parts, num_nodes);
+        StreamInfo info;
+        if (stream_usable(find_stream_info(plan, &info), in, workspace, workspace_floats, num_nodes, dim, num_parts))
+            return aggregate_stream_call(out, in, v.col, scale, info, plan, num_nodes, dim, workspace, stream, sink, sink2,
+                                         nullptr);
         return aggregate_dispatch(out, in, v.col, scale, PlanGroups{v.ptr, v.row, v.flags}, num_nodes, dim, num_parts,
                                   group_size, workspace, stream, sink, sink2, v.single);
     }
@@ -821,11 +889,15 @@ int aggregate_forward_groups(float* out, const float* in, const int* col, const 
 // pre-scaling pass then skips the rows no group reads.
 int aggregate_compacted_groups(float* out, const float* in, const int* ids, const int* part_ptr,
                                const int* edge_list, const float* scale, const void* plan, int num_nodes, int dim,
-                               int num_parts, int group_size, float* workspace, const uint32_t* gathered_rows,
-                               hipStream_t stream, double* sink, double* sink2)
+                               int num_parts, int group_size, float* workspace, size_t workspace_floats,
+                               const uint32_t* gathered_rows, hipStream_t stream, double* sink, double* sink2)
 {
     if (plan && num_parts > 0) {
         const PlanView v = plan_view(const_cast<void*>(plan), num_parts, num_nodes);
+        StreamInfo info;
+        if (stream_usable(find_stream_info(plan, &info), in, workspace, workspace_floats, num_nodes, dim, num_parts))
+            return aggregate_stream_call(out, in, v.col, scale, info, plan, num_nodes, dim, workspace, stream, sink, sink2,
+                                         gathered_rows);
         return aggregate_dispatch(out, in, v.col, scale, PlanGroups{v.ptr, v.row, v.flags}, num_nodes, dim, num_parts,
                                   group_size, workspace, stream, sink, sink2, v.single, gathered_rows);
     }

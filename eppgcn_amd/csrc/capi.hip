@@ -12,12 +12,13 @@ namespace eppgcn {
 
 // ---- implemented in aggregate.hip / prepare.hip
 int aggregate_forward_groups(float*, const float*, const int*, const float*, const int*, const int*, const void*, int,
-                             int, int, int, float*, hipStream_t, double*, double*);
+                             int, int, int, float*, size_t, hipStream_t, double*, double*);
 int aggregate_compacted_groups(float*, const float*, const int*, const int*, const int*, const float*, const void*,
-                               int, int, int, int, float*, const uint32_t*, hipStream_t, double*, double*);
-size_t plan_workspace_bytes(long long);
-size_t plan_scan_state_offset(long long);
-size_t plan_sort_state_offset(long long);
+                               int, int, int, int, float*, size_t, const uint32_t*, hipStream_t, double*, double*);
+size_t plan_workspace_bytes(long long, long long);
+int read_plan_status(const void*, long long, long long, long long, long long*, hipStream_t);
+void set_stream_mode(int);
+int last_call_used_stream();
 int schedule_shift(int);
 void set_schedule_shift(int);
 void set_plan_keep_rows(int);
@@ -29,7 +30,7 @@ void set_agg_force_rounds(int);
 size_t feature_workspace_floats(long long, int);
 int workspace_pitch(int);
 int launch_dense_rows(float*, int, int, const float*, int, const float*, long long, long long, const float*,
-                      const float*, int, int, long long, int, int, hipStream_t);
+                      const float*, int, int, long long, int, int, hipStream_t, unsigned);
 size_t update_workspace_bytes(long long, int, int);
 int launch_dense_weight(float*, const float*, int, const float*, int, int, long long, int, int, void*, hipStream_t);
 size_t compact_workspace_bytes(long long);
@@ -46,7 +47,6 @@ int launch_split(bool, const int*, int, int, int*, int*, long long, bool, void*,
 int launch_count_nonzero(const int*, long long, int*, hipStream_t);
 int launch_ginfo_hist(const int*, long long, int*, hipStream_t);
 int launch_mark_listed_rows(const int*, long long, long long, uint32_t*, int*, hipStream_t);
-
 // ---- errors
 static thread_local std::string g_last_error;
 void set_error(const std::string& msg) { g_last_error = msg; }
@@ -87,7 +87,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 12; }
+int eppgcn_abi_version(void) { return 13; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -107,7 +107,8 @@ int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers
     EPPGCN_REQUIRE(!workspace || workspace == in || workspace_floats >= feature_workspace_floats(num_nodes, dim),
                    "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
     return aggregate_forward_groups(out, in, column_index, degrees, part_pointers, part2node, plan, num_nodes, dim,
-                                    num_parts, part_size, workspace, static_cast<hipStream_t>(stream), &g_for_agg_ms, nullptr);
+                                    num_parts, part_size, workspace, workspace_floats, static_cast<hipStream_t>(stream),
+                                    &g_for_agg_ms, nullptr);
 }
 
 int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* row_pointers,
@@ -128,7 +129,8 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
     EPPGCN_REQUIRE(!workspace || workspace == d_output || workspace_floats >= feature_workspace_floats(num_nodes, dim),
                    "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
     return aggregate_forward_groups(d_input, d_output, column_index, degrees, part_pointers, part2node, plan,
-                                    num_nodes, dim, num_parts, part_size, workspace, static_cast<hipStream_t>(stream), &g_back_agg_ms, nullptr);
+                                    num_nodes, dim, num_parts, part_size, workspace, workspace_floats,
+                                    static_cast<hipStream_t>(stream), &g_back_agg_ms, nullptr);
 }
 
 int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
@@ -150,7 +152,7 @@ int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* i
     EPPGCN_REQUIRE(!workspace || workspace == d_output || workspace_floats >= feature_workspace_floats(num_nodes, dim),
                    "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
     return aggregate_compacted_groups(d_input, d_output, ids, part_pointer, edge_list, degrees, plan, num_nodes,
-                                      dim, num_parts, part_size > 0 ? part_size : 1, workspace, gathered_rows,
+                                      dim, num_parts, part_size > 0 ? part_size : 1, workspace, workspace_floats, gathered_rows,
                                       static_cast<hipStream_t>(stream), &g_back_agg_ms,
                                       layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr);
 }
@@ -183,7 +185,10 @@ size_t eppgcn_plan_bytes(int64_t num_parts, int64_t num_slots, int64_t num_nodes
 {
     return plan_bytes(num_parts, num_slots, num_nodes);
 }
-size_t eppgcn_plan_workspace_bytes(int64_t num_parts) { return plan_workspace_bytes(num_parts); }
+size_t eppgcn_plan_workspace_bytes(int64_t num_parts, int64_t num_slots)
+{
+    return plan_workspace_bytes(num_parts, num_slots);
+}
 
 int eppgcn_build_plan(const int32_t* part_pointers, const int32_t* column_index, const int32_t* part2node,
                       const int32_t* ids, int num_parts, int64_t num_slots, int num_nodes, int dim, int block_shift,
@@ -377,16 +382,29 @@ int eppgcn_scan_status(const void* workspace, void* stream)
     return kOk;
 }
 
-int eppgcn_build_plan_status(const void* workspace, int num_parts, void* stream)
+int eppgcn_plan_status(const void* plan, int num_parts, int64_t num_slots, int num_nodes, int64_t* partial_rows,
+                       void* stream)
 {
-    EPPGCN_REQUIRE(num_parts >= 0, "negative size");
+    EPPGCN_REQUIRE(num_parts >= 0 && num_slots >= 0 && num_nodes >= 0, "negative size");
+    if (partial_rows) *partial_rows = 0;
     if (num_parts == 0) return kOk;
-    EPPGCN_REQUIRE(workspace && aligned(workspace, 256), "workspace must be 256-byte aligned");
-    ScanState host;
-    char* base = static_cast<char*>(const_cast<void*>(workspace));
-    if (int rc = read_state(base + plan_sort_state_offset(num_parts), static_cast<hipStream_t>(stream), &host)) return rc;
-    return read_state(base + plan_scan_state_offset(num_parts), static_cast<hipStream_t>(stream), &host);
+    EPPGCN_REQUIRE(plan && aligned(plan, 256), "plan must be 256-byte aligned");
+    long long partial = 0;
+    const int rc = read_plan_status(plan, num_parts, num_slots, num_nodes, &partial, static_cast<hipStream_t>(stream));
+    if (partial_rows) *partial_rows = partial;
+    return rc;
 }
+
+size_t eppgcn_plan_workspace_floats(const void* plan, int64_t num_nodes, int dim)
+{
+    size_t rows = static_cast<size_t>(swizzle_padded_rows(num_nodes));
+    StreamInfo info;
+    if (plan && find_stream_info(plan, &info) && info.header.valid) rows += static_cast<size_t>(info.header.num_partials);
+    return rows * static_cast<size_t>(dim > 0 ? workspace_pitch(dim) : 0);
+}
+
+void eppgcn_set_stream_mode(int on) { set_stream_mode(on); }
+int eppgcn_last_call_used_stream(void) { return last_call_used_stream(); }
 
 static int finish_split(void* workspace, hipStream_t s, int32_t* d_counts, int64_t* h_a, int64_t* h_b)
 {
@@ -520,7 +538,29 @@ int eppgcn_update_forward(float* out, int ld_out, const float* x, const float* w
     EPPGCN_REQUIRE(aligned(out, 4) && aligned(x, 4) && aligned(w, 4), "matrix pointers must be 4-byte aligned");
     EPPGCN_REQUIRE(out != x, "the product cannot be written over its input");
     return launch_dense_rows(out, ld_out, ld_out, x, in_dim, w, out_dim, 1, scale, nullptr, 0, relu_input ? 1 : 0,
-                             num_nodes, in_dim, out_dim, static_cast<hipStream_t>(stream));
+                             num_nodes, in_dim, out_dim, static_cast<hipStream_t>(stream), 0u);
+}
+
+int eppgcn_update_forward_table(float* table, size_t table_floats, const float* x, const float* w, const float* scale,
+                                int relu_input, int64_t num_nodes, int in_dim, int out_dim, void* stream)
+{
+    EPPGCN_REQUIRE(num_nodes >= 0 && in_dim > 0 && out_dim > 0, "num_nodes >= 0, in_dim > 0, out_dim > 0 required");
+    if (num_nodes == 0) return kOk;
+    EPPGCN_REQUIRE(table && x && w && scale, "null pointer");
+    EPPGCN_REQUIRE(aligned(table, 16) && aligned(x, 4) && aligned(w, 4), "table must be 16-byte, matrices 4-byte aligned");
+    EPPGCN_REQUIRE(table != x, "the product cannot be written over its input");
+    EPPGCN_REQUIRE(num_nodes < (1ll << 31), "too many rows");
+    EPPGCN_REQUIRE(table_floats >= feature_workspace_floats(num_nodes, out_dim),
+                   "table smaller than eppgcn_feature_workspace_floats(num_nodes, out_dim)");
+    const int pitch = workspace_pitch(out_dim);
+    return launch_dense_rows(table, pitch, pitch, x, in_dim, w, out_dim, 1, scale, nullptr, 0, relu_input ? 1 : 0,
+                             num_nodes, in_dim, out_dim, static_cast<hipStream_t>(stream), kRowSwizzleMask);
+}
+
+int64_t eppgcn_feature_workspace_row(int64_t vertex)
+{
+    return vertex < 0 ? -1 : static_cast<int64_t>((static_cast<uint64_t>(vertex) & ~0xffffffffull) |
+                                                  swizzled_row(static_cast<unsigned>(vertex & 0xffffffffll)));
 }
 
 int eppgcn_update_backward_input(float* d_x, const float* g, const float* w, const float* relu_ref,
@@ -534,7 +574,7 @@ int eppgcn_update_backward_input(float* d_x, const float* g, const float* w, con
     EPPGCN_REQUIRE(d_x != g, "the product cannot be written over its input");
     // reduction over the out_dim columns of g; operand element (d, k) is w[k, d]
     return launch_dense_rows(d_x, in_dim, in_dim, g, out_dim, w, 1, out_dim, nullptr, relu_ref, in_dim, 0, num_nodes,
-                             out_dim, in_dim, static_cast<hipStream_t>(stream));
+                             out_dim, in_dim, static_cast<hipStream_t>(stream), 0u);
 }
 
 size_t eppgcn_update_workspace_bytes(int64_t num_nodes, int in_dim, int out_dim)

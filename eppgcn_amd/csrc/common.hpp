@@ -52,27 +52,68 @@ void set_force_wide_index(bool on);
 int launch_zero_rows_unless(float* out, const uint32_t* skip, long long num_rows, int dim, hipStream_t stream);
 
 // ---------------------------------------------------------------- execution plan layout
-// One caller-owned buffer: ptr[P+1] | row[P] | flags[P] | single[ceil(N/32)] | col[S], each part
-// 256-byte aligned (contents described in schedule.hip).  Offsets depend on the group count and the
-// vertex count alone.
+// One caller-owned buffer: ptr[P+1] | row[P] | flags[P] | single[ceil(N/32)] | col[S_pad] | stream form, each
+// part 256-byte aligned (contents described in schedule.hip).  Offsets depend on the group count, the
+// slot count and the vertex count alone.
 struct PlanView {
     int* ptr;
     int* row;
     uint8_t* flags;
     uint32_t* single;   // bit r: row r consists of exactly one non-empty group (it is written by one plain store)
-    int* col;
+    int* col;           // column ids in processing order; bit 31 marks the last slot of a piece (see below)
+};
+
+// Stream form of a plan (read by stream.hip, built by schedule.hip).  A "piece" is a maximal stretch of
+// plan entries that continue one another, i.e. consecutive slots of one row.
+constexpr int kStreamWave = 512;     // slots a wave of the stream kernel takes
+constexpr int kStreamChunk = 32;     // piece ends are counted per chunk of this many slots
+constexpr unsigned kStreamFlag = 0x80000000u;
+constexpr int kStreamIdMask = 0x7fffffff;
+struct StreamHeader {
+    int valid;          // 1: the stream arrays describe the plan (0: groups were empty or a scan stalled)
+    int num_events;     // pieces
+    int num_partials;   // partial sums the stream kernel leaves for the fix-up kernel
+    int num_fix;        // rows the fix-up kernel writes
+    int empty_rows;     // rows without any slot (the output clear zeroes them)
+    int error;          // a look-back scan of the build stalled
+    int empty_groups;   // != 0: the plan holds empty groups (no stream form)
+    int pad[9];
+};
+static_assert(sizeof(StreamHeader) == 64, "header layout");
+struct StreamView {
+    StreamHeader* header;
+    int* erow;          // [P]  per piece: its row, or kStreamFlag | index of its partial sum
+    int* cev;           // [S_pad / 32 + 1]  pieces that end before slot 32 c; bit 31: slot 32 c continues a piece
+    int* wtail;         // [S_pad / 512]  index of the partial sum of what wave w holds at its end, or -1
+    uint32_t* touched;  // [ceil(N/32)]  bit r: row r has at least one slot
+    int* frow;          // [N]  rows with partial sums ...
+    int* fptr;          // [N+1] ... and where their partial sums start
 };
 inline size_t plan_align(size_t x) { return (x + 255) / 256 * 256; }
 inline size_t plan_single_words(long long num_nodes)
 {
     return (static_cast<size_t>(num_nodes > 0 ? num_nodes : 0) + 31) / 32;
 }
+inline long long stream_padded_slots(long long num_slots)
+{
+    const long long s = num_slots > 0 ? num_slots : 0;
+    return (s + kStreamWave - 1) / kStreamWave * kStreamWave;
+}
+inline size_t plan_groups_bytes(long long num_parts, long long num_slots, long long num_nodes)
+{
+    const size_t p = static_cast<size_t>(num_parts > 0 ? num_parts : 0);
+    const size_t s = static_cast<size_t>(stream_padded_slots(num_slots));
+    return plan_align(4 * (p + 1)) + plan_align(4 * p) + plan_align(p) + plan_align(4 * plan_single_words(num_nodes)) +
+           plan_align(4 * s);
+}
 inline size_t plan_bytes(long long num_parts, long long num_slots, long long num_nodes)
 {
     const size_t p = static_cast<size_t>(num_parts > 0 ? num_parts : 0);
-    const size_t s = static_cast<size_t>(num_slots > 0 ? num_slots : 0);
-    return plan_align(4 * (p + 1)) + plan_align(4 * p) + plan_align(p) + plan_align(4 * plan_single_words(num_nodes)) +
-           plan_align(4 * s);
+    const size_t s = static_cast<size_t>(stream_padded_slots(num_slots));
+    const size_t n = static_cast<size_t>(num_nodes > 0 ? num_nodes : 0);
+    return plan_groups_bytes(num_parts, num_slots, num_nodes) + plan_align(sizeof(StreamHeader)) + plan_align(4 * p) +
+           plan_align(4 * (s / kStreamChunk + 1)) + plan_align(4 * (s / kStreamWave)) +
+           plan_align(4 * plan_single_words(num_nodes)) + plan_align(4 * n) + plan_align(4 * (n + 1));
 }
 inline PlanView plan_view(void* plan, long long num_parts, long long num_nodes)
 {
@@ -90,6 +131,55 @@ inline PlanView plan_view(void* plan, long long num_parts, long long num_nodes)
     v.col = reinterpret_cast<int*>(b);
     return v;
 }
+inline StreamView stream_view(void* plan, long long num_parts, long long num_slots, long long num_nodes)
+{
+    const size_t p = static_cast<size_t>(num_parts > 0 ? num_parts : 0);
+    const size_t s = static_cast<size_t>(stream_padded_slots(num_slots));
+    const size_t n = static_cast<size_t>(num_nodes > 0 ? num_nodes : 0);
+    char* b = static_cast<char*>(plan) + plan_groups_bytes(num_parts, num_slots, num_nodes);
+    StreamView v;
+    v.header = reinterpret_cast<StreamHeader*>(b);
+    b += plan_align(sizeof(StreamHeader));
+    v.erow = reinterpret_cast<int*>(b);
+    b += plan_align(4 * p);
+    v.cev = reinterpret_cast<int*>(b);
+    b += plan_align(4 * (s / kStreamChunk + 1));
+    v.wtail = reinterpret_cast<int*>(b);
+    b += plan_align(4 * (s / kStreamWave));
+    v.touched = reinterpret_cast<uint32_t*>(b);
+    b += plan_align(4 * plan_single_words(num_nodes));
+    v.frow = reinterpret_cast<int*>(b);
+    b += plan_align(4 * n);
+    v.fptr = reinterpret_cast<int*>(b);
+    return v;
+}
+// Row order of a separate pre-scaled feature table.  Vertex ids of graphs with a recursive (Kronecker / R-MAT)
+// structure are biased towards few set bits, so the hot rows of a table laid out by id share their low address
+// bits and their gathers pile up on a few memory channels (measured at R-MAT scale 22: 8 % of the kernel time).
+// Row r therefore lives at index r ^ ((r >> 5) & 4095): a permutation inside every aligned block of 4096 rows,
+// which keeps a column block of the plan one contiguous range of the table.
+constexpr unsigned kRowSwizzleShift = 5;
+constexpr unsigned kRowSwizzleMask = 4095;
+__host__ __device__ inline unsigned swizzled_row(unsigned r, unsigned mask = kRowSwizzleMask)
+{
+    return r ^ ((r >> kRowSwizzleShift) & mask);
+}
+// rows a swizzled table of num_nodes vertices spans (whole blocks)
+__host__ __device__ inline long long swizzle_padded_rows(long long num_nodes)
+{
+    const long long n = num_nodes > 0 ? num_nodes : 0;
+    return (n + kRowSwizzleMask) / (kRowSwizzleMask + 1) * (kRowSwizzleMask + 1);
+}
+
+// What the host knows about a plan's stream form once eppgcn_plan_status has read its header.
+struct StreamInfo {
+    long long num_parts, num_slots, num_nodes;
+    StreamHeader header;
+};
+// nullptr when the plan at this address has no (known) stream form
+const StreamInfo* find_stream_info(const void* plan, StreamInfo* copy);
+void forget_stream_info(const void* plan);
+void remember_stream_info(const void* plan, const StreamInfo& info);
 
 // ---------------------------------------------------------------- kernel timers
 // Optional event timing of the kernels of one call (off by default: calls stay

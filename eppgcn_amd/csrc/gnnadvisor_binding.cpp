@@ -135,7 +135,7 @@ const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& ro
     void* base = nullptr;
     e.plan = aligned_bytes(bytes, part_ptr, &base);
     e.plan_ptr = base;
-    const size_t wbytes = eppgcn_plan_workspace_bytes(num_parts);
+    const size_t wbytes = eppgcn_plan_workspace_bytes(num_parts, num_slots);
     void* wbase = nullptr;
     auto ws = aligned_bytes(wbytes, part_ptr, &wbase);
     check(eppgcn_build_plan(part_ptr.data_ptr<int32_t>(), col.data_ptr<int32_t>(),
@@ -143,8 +143,10 @@ const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& ro
                             is_forward ? nullptr : rows.data_ptr<int32_t>(), static_cast<int>(num_parts), num_slots,
                             num_nodes, dim_of_class(dc), block_shift, base, bytes, wbase, wbytes, stream_of(part_ptr)),
           "build_plan");
-    // once per group array: wait for the build and refuse a plan whose look-back scan stalled
-    check(eppgcn_build_plan_status(wbase, static_cast<int>(num_parts), stream_of(part_ptr)), "build_plan");
+    // once per group array: wait for the build, refuse a plan whose look-back scan stalled and let the
+    // library read the counts of the plan's stream form
+    check(eppgcn_plan_status(base, static_cast<int>(num_parts), num_slots, num_nodes, nullptr, stream_of(part_ptr)),
+          "build_plan");
     g_plans.push_front(std::move(e));
     if (g_plans.size() > kMaxPlans) g_plans.pop_back();
     return g_plans.front().plan_ptr;
@@ -198,9 +200,10 @@ const PathChoice& path_choice(const Tensor& part_pointer, const Tensor& edge_lis
     return g_path_choices.front();
 }
 
-Tensor feature_scratch(const Tensor& feats)
+// room for the pre-scaled table and, behind it, the partial sums of a call through the plan's stream form
+Tensor feature_scratch(const Tensor& feats, const void* plan)
 {
-    const size_t n = eppgcn_feature_workspace_floats(feats.size(0), static_cast<int>(feats.size(1)));
+    const size_t n = eppgcn_plan_workspace_floats(plan, feats.size(0), static_cast<int>(feats.size(1)));
     return torch::empty({static_cast<int64_t>(n)}, feats.options());
 }
 
@@ -216,16 +219,16 @@ int dense_support(const Tensor& X, const Tensor& W)
 }
 
 // scale[r] * act(X) * W as the padded, pre-scaled feature table the aggregation gathers from
-Tensor scaled_product(const Tensor& X, const Tensor& W, const Tensor& degrees, bool relu_input, size_t* ws_floats)
+Tensor scaled_product(const Tensor& X, const Tensor& W, const Tensor& degrees, bool relu_input, const void* plan,
+                      size_t* ws_floats)
 {
     const int64_t n = X.size(0);
     const int dim = static_cast<int>(W.size(1));
-    const int pitch = eppgcn_feature_workspace_pitch(dim);
-    *ws_floats = eppgcn_feature_workspace_floats(n, dim);
+    *ws_floats = eppgcn_plan_workspace_floats(plan, n, dim);
     auto scaled = torch::empty({static_cast<int64_t>(*ws_floats)}, X.options());
-    check(eppgcn_update_forward(scaled.data_ptr<float>(), pitch, X.data_ptr<float>(), W.data_ptr<float>(),
-                                f32(degrees), relu_input ? 1 : 0, n, static_cast<int>(X.size(1)), dim, stream_of(X)),
-          "update_forward");
+    check(eppgcn_update_forward_table(scaled.data_ptr<float>(), *ws_floats, X.data_ptr<float>(), W.data_ptr<float>(), f32(degrees),
+                                      relu_input ? 1 : 0, n, static_cast<int>(X.size(1)), dim, stream_of(X)),
+          "update_forward_table");
     return scaled;
 }
 
@@ -279,7 +282,7 @@ std::vector<Tensor> forward(Tensor input, Tensor weight, Tensor row_pointers, Te
     if (n > 0 && (dense_support(input, weight) & 1)) {
         // the product is written scaled and padded, ready to be gathered: no separate scaling pass
         size_t ws_floats = 0;
-        auto scaled = scaled_product(input, weight, degrees, relu_input, &ws_floats);
+        auto scaled = scaled_product(input, weight, degrees, relu_input, plan, &ws_floats);
         check(eppgcn_spmm_forward(output.data_ptr<float>(), nullptr, i32(row_pointers), i32(column_index),
                                   f32(degrees), i32(part_pointers), i32(part2Node), static_cast<int>(n), dim,
                                   static_cast<int>(part2Node.numel()), partSize, dimWorker, warpPerBlock,
@@ -288,8 +291,9 @@ std::vector<Tensor> forward(Tensor input, Tensor weight, Tensor row_pointers, Te
         return {output};
     }
     auto tmp = torch::mm(relu_input ? torch::relu(input) : input, weight);
-    // tmp is ours: when its rows need no padding it is scaled in place, otherwise into scratch
-    const size_t ws_floats = eppgcn_feature_workspace_floats(tmp.size(0), dim);
+    // tmp is ours: when its rows need no padding and no partial sums follow the table it is scaled in place,
+    // otherwise into scratch
+    const size_t ws_floats = eppgcn_plan_workspace_floats(plan, tmp.size(0), dim);
     auto scaled = ws_floats == static_cast<size_t>(tmp.numel())
                       ? tmp
                       : torch::empty({static_cast<int64_t>(ws_floats)}, tmp.options());
@@ -313,16 +317,15 @@ std::vector<Tensor> backward(Tensor d_output, Tensor X, Tensor W, Tensor row_poi
     TORCH_CHECK(part_pointers.numel() >= part2Node.numel() + 1, "part_pointers needs num_parts + 1 entries");
     CHECK_COUNTS(column_index, d_output.size(0));
     auto d_input_prime = torch::empty_like(d_output);
-    auto scaled = feature_scratch(d_output);     // d_output belongs to autograd: scale into scratch
+    const void* plan = plan_for(part_pointers, column_index, part2Node, true, part2Node.numel(), column_index.numel(),
+                                static_cast<int>(d_output.size(0)), static_cast<int>(d_output.size(1)));
+    auto scaled = feature_scratch(d_output, plan);     // d_output belongs to autograd: scale into scratch
     check(eppgcn_spmm_backward(d_input_prime.data_ptr<float>(), f32(d_output), i32(row_pointers),
                                i32(column_index), f32(degrees), i32(part_pointers), i32(part2Node),
                                static_cast<int>(d_output.size(0)), static_cast<int>(d_output.size(1)),
                                static_cast<int>(part2Node.numel()), partSize, dimWorker, warpPerBlock,
                                scaled.numel() ? scaled.data_ptr<float>() : nullptr, static_cast<size_t>(scaled.numel()),
-                               plan_for(part_pointers, column_index, part2Node, true, part2Node.numel(),
-                                        column_index.numel(), static_cast<int>(d_output.size(0)),
-                                        static_cast<int>(d_output.size(1))),
-                               stream_of(d_output)),
+                               plan, stream_of(d_output)),
           "backward");
     return dense_backward(d_input_prime, X, W, need_dx, relu_input);
 }
@@ -360,7 +363,6 @@ std::vector<Tensor> ours_backward(Tensor d_output, Tensor X, Tensor W, Tensor id
                 "partPointer needs numParts + 1 entries");
     CHECK_COUNTS(edgeList, d_output.size(0));
     auto d_input_prime = torch::empty_like(d_output);
-    auto scaled = feature_scratch(d_output);     // d_output belongs to autograd: scale into scratch
     const int num_nodes = static_cast<int>(d_output.size(0));
     const void* plan = nullptr;
     const uint32_t* gathered = nullptr;
@@ -373,6 +375,7 @@ std::vector<Tensor> ours_backward(Tensor d_output, Tensor X, Tensor W, Tensor id
         plan = plan_for(partPointer, edgeList, id, false, numParts, valid_len, num_nodes,
                         static_cast<int>(d_output.size(1)), choice.use_plan ? 0 : 31);
     }
+    auto scaled = feature_scratch(d_output, plan);     // d_output belongs to autograd: scale into scratch
     check(eppgcn_ours_backward(d_input_prime.data_ptr<float>(), f32(d_output), i32(id), i32(partPointer),
                                i32(edgeList), f32(degrees), static_cast<int>(d_output.size(0)),
                                static_cast<int>(d_output.size(1)), numParts, partSize > 0 ? partSize : 1, layer, blockx,

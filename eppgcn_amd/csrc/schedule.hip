@@ -15,6 +15,18 @@
 //     single[ceil(N/32)]  bit r set: row r has exactly one group and the group is not empty; the
 //                kernel writes such a row with one plain store, so the output clear can skip it
 //
+// Stream form (for stream.hip).  Consecutive plan entries that continue one another form a piece (a stretch
+// of slots of one row); the last slot of every piece carries bit 31 in col[], col[] is padded to a multiple
+// of 512 slots with an id behind every table row (N rounded up to a multiple of 4096), and
+//     erow[e]    row of piece e when the stream kernel can write it with one store (the piece is all of its row
+//                and lies inside one wave's 512 slots), otherwise bit 31 | index of the partial sum it leaves
+//     cev[c]     pieces that end before slot 32 c; bit 31 when slot 32 c continues a piece
+//     wtail[w]   index of the partial sum for what wave w still holds at its last slot, or -1
+//     touched    one bit per vertex: the row has at least one slot
+//     frow/fptr  rows that have partial sums and the range of each; the partial sums are numbered row by row,
+//                in stream order inside a row, so that summing a range in order gives the same bits every run
+// and a header with the counts.  A plan with empty groups gets no stream form (header.valid = 0).
+//
 // The re-ordering changes no result, only which groups run together.  It depends on the graph
 // and the groups alone: a caller builds it once and passes it to every aggregation call.
 //
@@ -253,6 +265,164 @@ __global__ __launch_bounds__(256) void plan_fill_kernel(const int* __restrict__ 
     }
 }
 
+// ---------------------------------------------------------------- stream form
+__global__ void stream_init_kernel(StreamHeader* h, int num_nodes)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        StreamHeader z = {};
+        z.empty_rows = num_nodes;
+        *h = z;
+    }
+}
+
+// is_end[q]: plan entry q is the last of its piece
+__global__ __launch_bounds__(256) void stream_ends_kernel(PlanView plan, int num_parts, int* __restrict__ is_end,
+                                                         StreamHeader* h)
+{
+    const int q = blockIdx.x * blockDim.x + threadIdx.x;
+    if (q >= num_parts) return;
+    const bool nonempty = plan.ptr[q + 1] > plan.ptr[q];
+    is_end[q] = nonempty && (plan.flags[q] & 8) == 0;
+    if (!nonempty) h->empty_groups = 1;
+}
+
+// ends_before[q] = pieces that end before entry q (exclusive scan of is_end; [P] = number of pieces).  Piece e:
+// first[e] = its first slot | bit 31 when the row has groups before it, last[e] = its last slot,
+// erow[e] = its row | bit 31 when the row has groups after it; the last slot is flagged in col.
+__global__ __launch_bounds__(256) void stream_pieces_kernel(PlanView plan, int num_parts,
+                                                           const int* __restrict__ ends_before, int* __restrict__ first,
+                                                           int* __restrict__ last, int* __restrict__ erow, StreamHeader* h)
+{
+    const int q = blockIdx.x * blockDim.x + threadIdx.x;
+    if (q == 0) h->num_events = ends_before[num_parts];
+    if (q >= num_parts) return;
+    const int beg = plan.ptr[q], end = plan.ptr[q + 1];
+    if (end <= beg) return;
+    const int f = plan.flags[q];
+    const int e = ends_before[q];
+    if (e < 0 || e >= num_parts) return;          // only after a stalled scan (the plan is then refused)
+    if ((f & 4) == 0) first[e] = beg | ((f & 1) ? static_cast<int>(kStreamFlag) : 0);
+    if ((f & 8) == 0) {
+        last[e] = end - 1;
+        erow[e] = plan.row[q] | ((f & 2) ? static_cast<int>(kStreamFlag) : 0);
+        plan.col[end - 1] |= static_cast<int>(kStreamFlag);
+    }
+}
+
+// number of pieces whose last slot lies before `slot`
+__device__ __forceinline__ int pieces_before(const int* __restrict__ last, int num_events, int slot)
+{
+    int lo = 0, hi = num_events;
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (last[mid] < slot) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
+// Candidates for a partial sum: piece e at index e, the tail of wave w at index P + w.  key = the row for a real
+// candidate, num_nodes otherwise (sorts behind every row).  Also: plain pieces get their row in erow, every piece
+// marks its row as touched, wtail is preset to -1, the padding of col is written.
+__global__ __launch_bounds__(256) void stream_classify_kernel(PlanView plan, StreamView sv, int num_parts, int num_slots,
+                                                             int padded_slots, int num_nodes,
+                                                             const int* __restrict__ first, const int* __restrict__ last,
+                                                             unsigned* __restrict__ keys)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    const int num_waves = padded_slots / kStreamWave;
+    // "gathers nothing": an id whose row lies behind every table, in swizzled row order too
+    if (i < padded_slots - num_slots) plan.col[num_slots + i] = static_cast<int>(swizzle_padded_rows(num_nodes));
+    if (i >= num_parts + num_waves) return;
+    if (sv.header->empty_groups) { keys[i] = static_cast<unsigned>(num_nodes); if (i >= num_parts) sv.wtail[i - num_parts] = -1; return; }
+    const int num_events = sv.header->num_events;
+    unsigned key = static_cast<unsigned>(num_nodes);
+    if (i < num_parts) {
+        if (i < num_events) {
+            const int a = first[i], b = last[i], r = sv.erow[i];
+            const int row = r & kStreamIdMask;
+            const bool whole = a >= 0 && r >= 0;
+            const bool partial = !whole || (a & kStreamIdMask) < b / kStreamWave * kStreamWave;
+            if (row < num_nodes) atomicOr(sv.touched + (row >> 5), 1u << (row & 31));
+            if (partial) key = static_cast<unsigned>(row);
+            else sv.erow[i] = row;
+        }
+    } else {
+        const int w = i - num_parts;
+        sv.wtail[w] = -1;
+        const long long at = static_cast<long long>(w + 1) * kStreamWave - 1;
+        if (at < num_slots && plan.col[at] >= 0) {
+            const int e = pieces_before(last, num_events, static_cast<int>(at));
+            if (e < num_events) key = static_cast<unsigned>(sv.erow[e] & kStreamIdMask);
+        }
+    }
+    keys[i] = key;
+}
+
+__global__ __launch_bounds__(256) void stream_cev_kernel(StreamView sv, int num_slots, int padded_slots,
+                                                        const int* __restrict__ last)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c > padded_slots / kStreamChunk) return;
+    if (sv.header->empty_groups) { sv.cev[c] = 0; return; }
+    const int num_events = sv.header->num_events;
+    const long long pos = static_cast<long long>(c) * kStreamChunk;
+    const int e = pos >= num_slots ? num_events : pieces_before(last, num_events, static_cast<int>(pos));
+    const bool inside = pos > 0 && pos < num_slots && !(e > 0 && last[e - 1] == pos - 1);
+    sv.cev[c] = e | (inside ? static_cast<int>(kStreamFlag) : 0);
+}
+
+// sorted candidates: position k of a real one is the index of its partial sum
+__global__ __launch_bounds__(256) void stream_assign_kernel(StreamView sv, int num_parts, int total, int num_nodes,
+                                                           const unsigned* __restrict__ sorted_keys,
+                                                           const int* __restrict__ order, int* __restrict__ is_head)
+{
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= total) return;
+    const unsigned key = sorted_keys[k];
+    int head = 0;
+    if (key < static_cast<unsigned>(num_nodes) && !sv.header->empty_groups) {
+        const int src = order[k];
+        if (src >= 0 && src < num_parts) sv.erow[src] = static_cast<int>(kStreamFlag) | k;
+        else if (src >= num_parts && src < total) sv.wtail[src - num_parts] = k;
+        head = k == 0 || sorted_keys[k - 1] != key;
+        if (k + 1 == total || sorted_keys[k + 1] >= static_cast<unsigned>(num_nodes)) sv.header->num_partials = k + 1;
+    }
+    is_head[k] = head;
+}
+
+__global__ __launch_bounds__(256) void stream_fix_rows_kernel(StreamView sv, int total, int num_nodes,
+                                                             const unsigned* __restrict__ sorted_keys,
+                                                             const int* __restrict__ is_head, const int* __restrict__ heads_before)
+{
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= total || !is_head[k]) return;
+    const int j = heads_before[k];
+    if (j < 0 || j >= num_nodes) return;          // only after a stalled scan
+    sv.frow[j] = static_cast<int>(sorted_keys[k]);
+    sv.fptr[j] = k;
+}
+
+__global__ __launch_bounds__(256) void stream_count_rows_kernel(StreamView sv, int words)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    int c = i < words ? __popc(sv.touched[i]) : 0;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, kWave);
+    if ((threadIdx.x & (kWave - 1)) == 0 && c) atomicSub(&sv.header->empty_rows, c);
+}
+
+__global__ void stream_finish_kernel(StreamView sv, const int* __restrict__ heads_before, int total, int num_nodes,
+                                     const ScanState* a, const ScanState* b)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    StreamHeader* h = sv.header;
+    const int num_fix = h->empty_groups ? 0 : min(max(heads_before[total], 0), num_nodes);
+    h->num_fix = num_fix;
+    sv.fptr[num_fix] = h->num_partials;
+    h->error = (a->error || b->error) ? 1 : 0;
+    h->valid = (!h->empty_groups && !h->error) ? 1 : 0;
+}
+
 // ---------------------------------------------------------------- host
 static size_t scan_state_bytes(long long n)
 {
@@ -268,25 +438,35 @@ static size_t sort_temp_bytes(long long n)
     return 2 * align256(sizeof(int) * static_cast<size_t>(entries + 1)) + scan_state_bytes(entries);
 }
 
-// workspace layout: keys_in | keys_out | order (scratch) | order | sizes | scan state | sort temporaries
-size_t plan_workspace_bytes(long long num_parts)
+// The stream form sorts one candidate per plan entry and per wave of the stream kernel.
+static long long plan_sort_capacity(long long num_parts, long long num_slots)
+{
+    return (num_parts > 0 ? num_parts : 0) + stream_padded_slots(num_slots) / kStreamWave;
+}
+
+// workspace layout: six arrays of plan_sort_capacity + 1 ints (keys, sorted keys, two index arrays, sizes, one
+// more for the stream form) | scan state | sort temporaries
+constexpr int kPlanSlabs = 6;
+size_t plan_workspace_bytes(long long num_parts, long long num_slots)
 {
     if (num_parts <= 0) return 256;
-    return 5 * align256(sizeof(int) * (static_cast<size_t>(num_parts) + 1)) + scan_state_bytes(num_parts) +
-           sort_temp_bytes(num_parts) + 256;
+    const long long cap = plan_sort_capacity(num_parts, num_slots);
+    return kPlanSlabs * align256(sizeof(int) * (static_cast<size_t>(cap) + 1)) + scan_state_bytes(cap + 1) +
+           sort_temp_bytes(cap) + 256;
 }
 
-// where launch_build_plan keeps the state of its look-back scan inside the workspace
-size_t plan_scan_state_offset(long long num_parts)
+// where launch_build_plan keeps the state of its look-back scans inside the workspace
+static size_t plan_scan_state_offset(long long num_parts, long long num_slots)
 {
-    return 5 * align256(sizeof(int) * (static_cast<size_t>(num_parts > 0 ? num_parts : 0) + 1));
+    return kPlanSlabs * align256(sizeof(int) * (static_cast<size_t>(plan_sort_capacity(num_parts, num_slots)) + 1));
 }
 
-// ... and the state of the scans inside its radix sort (one state for all passes; the stall flag survives them)
-size_t plan_sort_state_offset(long long num_parts)
+// ... and the state of the scans inside its radix sorts (one state for all passes; the stall flag survives them)
+static size_t plan_sort_state_offset(long long num_parts, long long num_slots)
 {
-    const long long entries = sort_tiles(num_parts > 0 ? num_parts : 0) * kDigits;
-    return plan_scan_state_offset(num_parts) + scan_state_bytes(num_parts) +
+    const long long cap = plan_sort_capacity(num_parts, num_slots);
+    const long long entries = sort_tiles(cap) * kDigits;
+    return plan_scan_state_offset(num_parts, num_slots) + scan_state_bytes(cap + 1) +
            2 * align256(sizeof(int) * static_cast<size_t>(entries + 1));
 }
 
@@ -343,14 +523,13 @@ static int launch_exclusive_scan(const int* in, int* out, long long n, void* sta
 // Sorts the pairs (keys[i], i) by the low `bits` bits of the key, stably; the sorted indices end up in
 // `order`.  keys_a is overwritten; keys_b, vals_tmp and temp are scratch.
 static int stable_sort_by_key(unsigned* keys_a, unsigned* keys_b, int* vals_tmp, int* order, int n, int bits, void* temp,
-                              hipStream_t stream)
+                              void* state, hipStream_t stream, unsigned** sorted_keys = nullptr, bool keep_error = false)
 {
     const int tiles = static_cast<int>(sort_tiles(n));
     const long long entries = static_cast<long long>(tiles) * kDigits;
     char* t = static_cast<char*>(temp);
     int* hist = reinterpret_cast<int*>(t);
     int* offsets = reinterpret_cast<int*>(t + align256(sizeof(int) * static_cast<size_t>(entries + 1)));
-    void* state = t + 2 * align256(sizeof(int) * static_cast<size_t>(entries + 1));
     const int passes = bits <= 8 ? 1 : (bits + 7) / 8;
     // the last pass must write `order`: with an even number of passes the first one writes the temporary
     unsigned* kin = keys_a;
@@ -361,13 +540,67 @@ static int stable_sort_by_key(unsigned* keys_a, unsigned* keys_b, int* vals_tmp,
         const int shift = pass * 8;
         hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(kSortBlock), 0, stream, kin, n, shift, tiles, hist);
         EPPGCN_HIP(hipGetLastError());
-        if (int rc = launch_exclusive_scan(hist, offsets, entries, state, stream, pass > 0)) return rc;
+        if (int rc = launch_exclusive_scan(hist, offsets, entries, state, stream, keep_error || pass > 0)) return rc;
         hipLaunchKernelGGL(radix_scatter_kernel, dim3(tiles), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, shift,
                            tiles, offsets);
         EPPGCN_HIP(hipGetLastError());
         unsigned* tk = kin; kin = kout; kout = tk;
         vin = vout;
     }
+    if (sorted_keys) *sorted_keys = kin;
+    return kOk;
+}
+
+static int launch_build_stream(PlanView v, StreamView sv, int num_parts, long long num_slots, int num_nodes, char* base,
+                               size_t slab, ScanState* st, ScanState* sort_st, void* temp, hipStream_t stream)
+{
+    const int padded = static_cast<int>(stream_padded_slots(num_slots));
+    const int num_waves = padded / kStreamWave;
+    const int total = num_parts + num_waves;
+    int* is_end = reinterpret_cast<int*>(base);                       // later: scratch of the sort
+    int* ends_before = reinterpret_cast<int*>(base + slab);           // later: second key array of the sort
+    int* first = reinterpret_cast<int*>(base + 2 * slab);             // later: is_head
+    int* last = reinterpret_cast<int*>(base + 3 * slab);              // later: heads_before
+    unsigned* keys = reinterpret_cast<unsigned*>(base + 4 * slab);
+    int* order = reinterpret_cast<int*>(base + 5 * slab);
+    const auto blocks = [](long long n) { return dim3(static_cast<unsigned>((n + 255) / 256 > 0 ? (n + 255) / 256 : 1)); };
+    hipLaunchKernelGGL(stream_init_kernel, dim3(1), dim3(64), 0, stream, sv.header, num_nodes);
+    EPPGCN_HIP(hipGetLastError());
+    if (int rc = launch_zero_words(sv.touched, plan_single_words(num_nodes), stream)) return rc;
+    hipLaunchKernelGGL(stream_ends_kernel, blocks(num_parts), dim3(256), 0, stream, v, num_parts, is_end, sv.header);
+    EPPGCN_HIP(hipGetLastError());
+    if (int rc = launch_exclusive_scan(is_end, ends_before, num_parts, st, stream, true)) return rc;
+    hipLaunchKernelGGL(stream_pieces_kernel, blocks(num_parts), dim3(256), 0, stream, v, num_parts, ends_before, first, last,
+                       sv.erow, sv.header);
+    EPPGCN_HIP(hipGetLastError());
+    const long long classify_threads = total > padded - num_slots ? total : padded - num_slots;
+    hipLaunchKernelGGL(stream_classify_kernel, blocks(classify_threads), dim3(256), 0, stream, v, sv, num_parts,
+                       static_cast<int>(num_slots), padded, num_nodes, first, last, keys);
+    EPPGCN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(stream_cev_kernel, blocks(padded / kStreamChunk + 1), dim3(256), 0, stream, sv,
+                       static_cast<int>(num_slots), padded, last);
+    EPPGCN_HIP(hipGetLastError());
+    int bits = 1;
+    while (bits < 31 && (1ll << bits) <= num_nodes) ++bits;           // the key num_nodes needs a digit too
+    unsigned* sorted_keys = nullptr;
+    if (int rc = stable_sort_by_key(keys, reinterpret_cast<unsigned*>(ends_before), is_end, order, total, bits, temp, sort_st,
+                                    stream, &sorted_keys, true))
+        return rc;
+    int* is_head = first;
+    int* heads_before = last;
+    hipLaunchKernelGGL(stream_assign_kernel, blocks(total), dim3(256), 0, stream, sv, num_parts, total, num_nodes, sorted_keys,
+                       order, is_head);
+    EPPGCN_HIP(hipGetLastError());
+    if (int rc = launch_exclusive_scan(is_head, heads_before, total, st, stream, true)) return rc;
+    hipLaunchKernelGGL(stream_fix_rows_kernel, blocks(total), dim3(256), 0, stream, sv, total, num_nodes, sorted_keys,
+                       is_head, heads_before);
+    EPPGCN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(stream_count_rows_kernel, blocks(static_cast<long long>(plan_single_words(num_nodes))), dim3(256), 0,
+                       stream, sv, static_cast<int>(plan_single_words(num_nodes)));
+    EPPGCN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(stream_finish_kernel, dim3(1), dim3(64), 0, stream, sv, heads_before, total, num_nodes, st,
+                       sort_st);
+    EPPGCN_HIP(hipGetLastError());
     return kOk;
 }
 
@@ -375,33 +608,39 @@ int launch_build_plan(const int* part_ptr, const int* col, const int* part2node,
                       long long num_slots, int num_nodes, int shift, void* plan, size_t plan_size, void* workspace,
                       size_t workspace_bytes, hipStream_t stream)
 {
+    forget_stream_info(plan);
     if (num_parts <= 0) return kOk;
     if (plan_size < plan_bytes(num_parts, num_slots, num_nodes)) {
         set_error("build_plan: plan buffer smaller than eppgcn_plan_bytes(num_parts, num_slots, num_nodes)");
         return kErrInvalidArgument;
     }
-    const size_t slab = align256(sizeof(int) * (static_cast<size_t>(num_parts) + 1));
+    if (num_slots >= (1ll << 31) - kStreamWave) {
+        set_error("build_plan: slot count beyond 32-bit offsets");
+        return kErrInvalidArgument;
+    }
+    const long long cap = plan_sort_capacity(num_parts, num_slots);
+    const size_t slab = align256(sizeof(int) * (static_cast<size_t>(cap) + 1));
     char* base = static_cast<char*>(workspace);
     unsigned* keys_in = reinterpret_cast<unsigned*>(base);
     unsigned* keys_out = reinterpret_cast<unsigned*>(base + slab);
     int* order_tmp = reinterpret_cast<int*>(base + 2 * slab);
     int* order = reinterpret_cast<int*>(base + 3 * slab);
     int* sizes = reinterpret_cast<int*>(base + 4 * slab);
-    ScanState* st = reinterpret_cast<ScanState*>(base + plan_scan_state_offset(num_parts));
-    void* temp = base + 5 * slab + scan_state_bytes(num_parts);
+    ScanState* st = reinterpret_cast<ScanState*>(base + plan_scan_state_offset(num_parts, num_slots));
+    void* temp = base + kPlanSlabs * slab + scan_state_bytes(cap + 1);
+    ScanState* sort_st = reinterpret_cast<ScanState*>(base + plan_sort_state_offset(num_parts, num_slots));
     int bits = 1;
     while (bits < 30 && (static_cast<long long>(num_nodes) >> shift) >= (1ll << bits)) ++bits;
     if (g_length_classes) bits += 2;
-    const size_t temp_bytes = sort_temp_bytes(num_parts);
-    if (5 * slab + scan_state_bytes(num_parts) + temp_bytes > workspace_bytes) {
-        set_error("build_plan: workspace smaller than eppgcn_plan_workspace_bytes(num_parts)");
+    if (plan_workspace_bytes(num_parts, num_slots) > workspace_bytes) {
+        set_error("build_plan: workspace smaller than eppgcn_plan_workspace_bytes(num_parts, num_slots)");
         return kErrInvalidArgument;
     }
     const unsigned blocks = static_cast<unsigned>((num_parts + 255) / 256);
     hipLaunchKernelGGL(plan_keys_kernel, dim3(blocks), dim3(256), 0, stream, part_ptr, col, part2node, ids, num_parts,
                        shift, g_keep_rows * 32, g_length_classes, keys_in);
     EPPGCN_HIP(hipGetLastError());
-    if (int rc = stable_sort_by_key(keys_in, keys_out, order_tmp, order, num_parts, bits, temp, stream)) return rc;
+    if (int rc = stable_sort_by_key(keys_in, keys_out, order_tmp, order, num_parts, bits, temp, sort_st, stream)) return rc;
     hipLaunchKernelGGL(plan_sizes_kernel, dim3(blocks), dim3(256), 0, stream, part_ptr, order, num_parts, sizes);
     EPPGCN_HIP(hipGetLastError());
     PlanView v = plan_view(plan, num_parts, num_nodes);
@@ -411,6 +650,59 @@ int launch_build_plan(const int* part_ptr, const int* col, const int* part2node,
     hipLaunchKernelGGL(plan_fill_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream,
                        part_ptr, col, part2node, ids, order, num_parts, v);
     EPPGCN_HIP(hipGetLastError());
+    return launch_build_stream(v, stream_view(plan, num_parts, num_slots, num_nodes), num_parts, num_slots, num_nodes, base,
+                               slab, st, sort_st, temp, stream);
+}
+
+// ---------------------------------------------------------------- what the host knows about built plans
+}  // namespace eppgcn
+
+#include <map>
+#include <mutex>
+
+namespace eppgcn {
+
+static std::mutex g_info_mutex;
+static std::map<const void*, StreamInfo> g_infos;
+
+const StreamInfo* find_stream_info(const void* plan, StreamInfo* copy)
+{
+    std::lock_guard<std::mutex> lock(g_info_mutex);
+    auto it = g_infos.find(plan);
+    if (it == g_infos.end()) return nullptr;
+    *copy = it->second;
+    return copy;
+}
+void forget_stream_info(const void* plan)
+{
+    std::lock_guard<std::mutex> lock(g_info_mutex);
+    g_infos.erase(plan);
+}
+void remember_stream_info(const void* plan, const StreamInfo& info)
+{
+    std::lock_guard<std::mutex> lock(g_info_mutex);
+    g_infos[plan] = info;
+}
+
+// Synchronises the stream, reads the plan's header and records it; the return code tells whether a look-back scan
+// of the build stalled.
+int read_plan_status(const void* plan, long long num_parts, long long num_slots, long long num_nodes,
+                     long long* partial_rows, hipStream_t stream)
+{
+    if (partial_rows) *partial_rows = 0;
+    if (num_parts <= 0) return kOk;
+    StreamInfo info;
+    info.num_parts = num_parts; info.num_slots = num_slots; info.num_nodes = num_nodes;
+    const StreamView sv = stream_view(const_cast<void*>(plan), num_parts, num_slots, num_nodes);
+    EPPGCN_HIP(hipMemcpyAsync(&info.header, sv.header, sizeof(StreamHeader), hipMemcpyDeviceToHost, stream));
+    EPPGCN_HIP(hipStreamSynchronize(stream));
+    if (info.header.error) {
+        forget_stream_info(plan);
+        set_error("look-back scan stalled: a tile waited past its spin limit; the plan is invalid");
+        return kErrScanStalled;
+    }
+    remember_stream_info(plan, info);
+    if (partial_rows && info.header.valid) *partial_rows = info.header.num_partials;
     return kOk;
 }
 

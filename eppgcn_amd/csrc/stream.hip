@@ -1,0 +1,383 @@
+// Slot-stream aggregation for gfx950 (wave64): the aggregation of a planned launch as a segmented sum
+// over one stream of slots, every wave taking the same number of slots.
+//
+// Same contract as aggregate_kernel (EPPGCN/GCNConv/EPPGCN_kernel.cu:204-295, :626-670):
+//
+//   out[r, :] = s[r] * sum over the slots e of row r of  table[col[e], :]       (table[c, :] = s[c] * in[c, :])
+//
+// A plan lists the groups in processing order; consecutive groups that continue one another form a
+// "piece" (a stretch of slots of one row).  The stream form of the plan (schedule.hip) is
+//
+//   scol[S_pad]   column id of every slot in processing order; bit 31 set on the last slot of a piece;
+//                 padded to a multiple of kStreamWave slots with an id behind the table ("gathers nothing")
+//   erow[NE]      one entry per piece, in stream order: its row when one store writes it (the piece is all of
+//                 its row and lies inside one wave's slots), else bit 31 | the index of its partial sum
+//   cev[S_pad / 32 + 1]   number of pieces that end before slot 32 c; bit 31 set when slot 32 c lies inside
+//                 a piece that started earlier
+//   wtail[S_pad / 512]    index of the partial sum of what wave w holds after its last slot, or -1
+//   frow, fptr    the rows that have partial sums and the range of each (numbered row by row)
+//
+// Mapping.  A wave takes kStreamWave = 512 consecutive slots with two 16-byte loads per lane: lane l
+// holds slots 8l .. 8l+7.  A team of TS lanes (TS * 16 bytes = one table row) owns the 8 * TS slots its
+// own lanes hold and walks them in TS steps of 8 row gathers; the ids of step s are broadcast from lane
+// s of the team, so no id goes through LDS or is loaded twice.  Every gather instruction of the wave is
+// full (64 / TS rows) whatever the lengths of the rows.  A team adds rows into its partial sum and, at a
+// slot that ends a piece, writes the sum to that piece's row (s[r] and r come from a per-wave list in LDS,
+// staged once with coalesced loads).  What a team holds at the ends of its slot range - the tail of a piece
+// that goes on in the next team, the head of one that began in an earlier team - is combined across the
+// teams of the wave once, at the end, with a segmented scan in registers.  Pieces that cross waves and rows cut
+// into several pieces leave unscaled partial sums in a scratch area, which a second small kernel adds up row by
+// row in a fixed order: no float atomics, no output clear for rows that have slots, and the same bits every run.
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace eppgcn {
+
+constexpr int kStreamBlock = 256;
+constexpr int kStreamWaves = kStreamBlock / kWave;
+constexpr int kStreamEvents = kStreamWave;       // pieces that can end in a wave's slots
+constexpr unsigned kNoRowOffset = 0xffffffffu;
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+template <int OVW> __device__ __forceinline__ void stream_store(float* p, const float* v);
+template <> __device__ __forceinline__ void stream_store<4>(float* p, const float* v)
+{
+    const f32x4 t = {v[0], v[1], v[2], v[3]};
+    __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(p));
+}
+template <> __device__ __forceinline__ void stream_store<2>(float* p, const float* v)
+{
+    const f32x2 t = {v[0], v[1]};
+    __builtin_nontemporal_store(t, reinterpret_cast<f32x2*>(p));
+}
+template <> __device__ __forceinline__ void stream_store<1>(float* p, const float* v) { __builtin_nontemporal_store(v[0], p); }
+
+// table rows: pitch ld_bytes (a multiple of 16), `chunks` 16-byte vectors of a row are read (chunks <= TS);
+// out rows: pitch ld_out floats, columns < width_out written in pieces of OVW floats;
+// partial rows: pitch ld_bytes, written whole (unscaled sums).
+// U: row gathers per batch (4 or 8); two batches are in flight.
+template <int U> struct StreamBatch {
+    u32x4 v[U];
+    unsigned c[U];
+};
+
+template <int OVW, int TS, int U>
+__global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
+    float* __restrict__ out, float* __restrict__ partial, const float* __restrict__ table,
+    const int* __restrict__ scol, const int* __restrict__ erow, const int* __restrict__ cev,
+    const int* __restrict__ wtail, const float* __restrict__ scale, int num_wave_chunks, int num_events,
+    int num_nodes, int num_partials, int chunks, unsigned ld_bytes, int width_out, int ld_out, unsigned table_bytes)
+{
+    constexpr int TPW = kWave / TS;
+    constexpr int kParts = 8 / U;                  // batches per step
+    constexpr int kCevPerTeam = TS / 4;            // cev counts chunks of 32 slots; a team owns 8 * TS slots
+    __shared__ int ev_row[kStreamWaves][kStreamEvents + 3];
+    __shared__ float ev_scale[kStreamWaves][kStreamEvents + 3];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int team = lane / TS;
+    const int tl = lane % TS;
+    const int w = blockIdx.x * kStreamWaves + wave;
+    if (w >= num_wave_chunks) return;                       // wave-uniform; the LDS rows are wave-private
+    int* my_row = ev_row[wave];
+    float* my_scale = ev_scale[wave];
+
+    // the wave's 512 slot ids, 8 per lane (streamed once: non-temporal)
+    const u32x4* idp = reinterpret_cast<const u32x4*>(scol + static_cast<size_t>(w) * kStreamWave) + lane * 2;
+    const u32x4 id_lo = __builtin_nontemporal_load(idp);
+    const u32x4 id_hi = __builtin_nontemporal_load(idp + 1);
+    const unsigned ids[8] = {id_lo.x, id_lo.y, id_lo.z, id_lo.w, id_hi.x, id_hi.y, id_hi.z, id_hi.w};
+    const int c0 = w * (kStreamWave / 32);
+    const int ce_team = cev[c0 + team * kCevPerTeam];
+    const int ce_first = cev[c0];
+    const int ce_last = cev[c0 + kStreamWave / 32];
+    const int tail_at = wtail[w];
+
+    const __amdgpu_buffer_rsrc_t rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(table), 0,
+                                                                          static_cast<int>(table_bytes), 0x00020000);
+    const unsigned lane_off = tl < chunks ? static_cast<unsigned>(tl) * 16u : kNoRowOffset;
+
+    // batch (s, part): the ids come from lane s of the team, registers part * U ...
+    auto issue = [&](StreamBatch<U>& b, int s, auto part) {
+        constexpr int kPart = decltype(part)::value;
+        const int src = team * TS + s;
+#pragma unroll
+        for (int u = 0; u < U; ++u) b.c[u] = static_cast<unsigned>(__shfl(static_cast<int>(ids[kPart * U + u]), src, kWave));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const unsigned id = swizzled_row(b.c[u] & 0x7fffffffu);      // the table's row order (common.hpp)
+            const unsigned off = lane_off == kNoRowOffset ? kNoRowOffset : __umul24(id, ld_bytes) + lane_off;
+            b.v[u] = __builtin_amdgcn_raw_buffer_load_b128(rows, off, 0, 0);
+        }
+    };
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, kParts - 1>;
+
+    StreamBatch<U> ba, bb;
+    issue(ba, 0, P0{});            // the first gathers are under way while the piece list is staged
+
+    // pieces that end in the wave's slots: [ev0, ev1)
+    const int ev0 = ce_first & 0x7fffffff;
+    const int ev1 = ce_last & 0x7fffffff;
+    {
+        const int staged = min(min(ev1, num_events) - ev0, kStreamEvents);
+        for (int j = lane; j < staged; j += kWave) {
+            const int r = erow[ev0 + j];
+            my_row[j] = r;
+            my_scale[j] = r < 0 ? 1.f : scale[min(r, num_nodes - 1)];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+
+    // a complete piece goes to its row, scaled; anything else to its place among the partial sums
+    auto flush = [&](const float (&a)[4], int target, float s) {
+        if (target < 0) {
+            const int at = target & 0x7fffffff;
+            if (at >= num_partials || tl >= chunks) return;       // the first never happens with a well-formed stream
+            float* dst = reinterpret_cast<float*>(reinterpret_cast<char*>(partial) + static_cast<size_t>(at) * ld_bytes) + tl * 4;
+            const f32x4 t = {a[0], a[1], a[2], a[3]};
+            __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(dst));
+        } else {
+            if (target >= num_nodes) return;
+            float* dst = out + static_cast<size_t>(target) * ld_out + tl * 4;
+            const float v[4] = {a[0] * s, a[1] * s, a[2] * s, a[3] * s};
+#pragma unroll
+            for (int piece = 0; piece < 4 / OVW; ++piece)
+                if (tl * 4 + piece * OVW < width_out) stream_store<OVW>(dst + piece * OVW, v + piece * OVW);
+        }
+    };
+
+    int ev = min(max((ce_team & 0x7fffffff) - ev0, 0), kStreamEvents);   // the team's next piece end in the staged list
+    bool head_pending = ce_team < 0;             // the first piece end of the team closes a piece from an earlier team
+    bool had_event = false;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    float head[4] = {0.f, 0.f, 0.f, 0.f};
+    int head_row = 0;
+    float head_scale = 0.f;
+    int next_row = my_row[ev];
+    float next_scale = my_scale[ev];
+
+    auto consume = [&](const StreamBatch<U>& b) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            acc[0] += __uint_as_float(b.v[u].x);
+            acc[1] += __uint_as_float(b.v[u].y);
+            acc[2] += __uint_as_float(b.v[u].z);
+            acc[3] += __uint_as_float(b.v[u].w);
+            if (static_cast<int>(b.c[u]) < 0) {            // the slot ends a piece
+                if (head_pending) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) head[j] = acc[j];
+                    head_row = next_row;
+                    head_scale = next_scale;
+                    head_pending = false;
+                } else {
+                    flush(acc, next_row, next_scale);
+                }
+                had_event = true;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = 0.f;
+                ev = min(ev + 1, kStreamEvents);
+                next_row = my_row[ev];
+                next_scale = my_scale[ev];
+            }
+        }
+    };
+
+    // two batches in flight; the loop bodies issue unconditionally so that the waits can count on the younger batch
+    if constexpr (kParts == 2) {
+        for (int s = 0; s + 1 < TS; ++s) {
+            issue(bb, s, P1{});
+            consume(ba);
+            issue(ba, s + 1, P0{});
+            consume(bb);
+        }
+        issue(bb, TS - 1, P1{});
+        consume(ba);
+        consume(bb);
+    } else {
+        for (int s = 0; s + 2 < TS; s += 2) {
+            issue(bb, s + 1, P0{});
+            consume(ba);
+            issue(ba, s + 2, P0{});
+            consume(bb);
+        }
+        issue(bb, TS - 1, P0{});
+        consume(ba);
+        consume(bb);
+    }
+
+    // ---- combine across the teams of the wave.  Inclusive segmented scan of the tails: a team in which a piece
+    // ended starts a new segment (what came before it does not pass through it).
+    float run[4] = {acc[0], acc[1], acc[2], acc[3]};
+    bool stop = had_event;
+    if constexpr (TPW > 1) {
+#pragma unroll
+        for (int d = 1; d < TPW; d <<= 1) {
+            const bool take = team >= d && !stop;
+            const int other_stop = __shfl_up(static_cast<int>(stop), d * TS, kWave);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float o = __shfl_up(run[j], d * TS, kWave);
+                if (take) run[j] += o;
+            }
+            if (team >= d) stop = stop || other_stop != 0;
+        }
+    }
+    // what flows into a team is the scan value of the team before it
+    float carry[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float o = TPW > 1 ? __shfl_up(run[j], TS, kWave) : 0.f;
+        carry[j] = team > 0 ? o : 0.f;
+    }
+    if (ce_team < 0 && had_event) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) head[j] += carry[j];
+        flush(head, head_row, head_scale);
+    }
+    // the wave's last tail belongs to a piece that ends in a later wave: one more partial sum
+    if (team == TPW - 1 && tail_at >= 0) flush(run, tail_at | static_cast<int>(kStreamFlag), 1.f);
+}
+
+// Rows with partial sums: out[frow[i], :] = s[frow[i]] * (sum of the partial rows fptr[i] .. fptr[i+1]), summed in
+// a fixed order, so the result does not depend on the order in which the waves of the stream kernel ran.  A wave
+// takes 64 / TS rows.  Short lists: a team of TS lanes per row walks its list.  When a row of the wave has more
+// than kFixTeamMax partial sums (a hub row cut into column blocks and waves) the whole wave works on one row at a
+// time: team t adds the partial sums t, t + TPW, ..., and the teams are summed with cross-lane operations.
+constexpr int kFixTeamMax = 32;
+template <int OVW, int TS>
+__global__ __launch_bounds__(256) void stream_fixup_kernel(float* __restrict__ out, const float* __restrict__ partial,
+                                                           const int* __restrict__ frow, const int* __restrict__ fptr,
+                                                           const float* __restrict__ scale, const StreamHeader* header,
+                                                           int chunks, unsigned ld_bytes, int width_out, int ld_out)
+{
+    constexpr int TPW = kWave / TS;
+    const int num_fix = header->num_fix;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int team = lane / TS;
+    const int tl = lane % TS;
+    const long long wave0 = static_cast<long long>(blockIdx.x) * (256 / kWave) + threadIdx.x / kWave;
+    const long long waves = static_cast<long long>(gridDim.x) * (256 / kWave);
+    const char* base = reinterpret_cast<const char*>(partial) + tl * 16;
+    auto add_range = [&](float (&acc)[4], int beg, int end, int step) {
+        for (int k = beg; k < end; k += 4 * step) {
+            f32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                v[u] = (k + u * step < end && tl < chunks)
+                           ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(base + static_cast<size_t>(k + u * step) * ld_bytes))
+                           : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < 4; ++u) { acc[0] += v[u].x; acc[1] += v[u].y; acc[2] += v[u].z; acc[3] += v[u].w; }
+        }
+    };
+    auto write_row = [&](const float (&acc)[4], int r) {
+        const float s = scale[r];
+        const float v[4] = {acc[0] * s, acc[1] * s, acc[2] * s, acc[3] * s};
+        float* dst = out + static_cast<size_t>(r) * ld_out + tl * 4;
+#pragma unroll
+        for (int piece = 0; piece < 4 / OVW; ++piece)
+            if (tl * 4 + piece * OVW < width_out) stream_store<OVW>(dst + piece * OVW, v + piece * OVW);
+    };
+    for (long long wv = wave0; wv * TPW < num_fix; wv += waves) {
+        const long long i = wv * TPW + team;
+        const bool have = i < num_fix;
+        const int r = have ? frow[i] : 0;
+        const int beg = have ? fptr[i] : 0, end = have ? fptr[i + 1] : 0;
+        if (!__any(end - beg > kFixTeamMax)) {
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+            add_range(acc, beg, end, 1);
+            if (have) write_row(acc, r);
+        } else {
+#pragma unroll 1
+            for (int t = 0; t < TPW; ++t) {
+                const int rb = __shfl(beg, t * TS, kWave), re = __shfl(end, t * TS, kWave), rr = __shfl(r, t * TS, kWave);
+                if (re <= rb) continue;                  // wave-uniform
+                float acc[4] = {0.f, 0.f, 0.f, 0.f};
+                add_range(acc, rb + team, re, TPW);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = cross_team_sum<TS>(acc[j]);
+                if (team == 0) write_row(acc, rr);
+            }
+        }
+    }
+}
+
+static int g_stream_mode = 1;
+void set_stream_mode(int on) { g_stream_mode = on ? 1 : 0; }
+
+// Team size for rows of `chunks` 16-byte vectors, 0 when the stream kernel does not cover the shape.
+static int stream_team(int chunks)
+{
+    int ts = 4;
+    while (ts < 64 && ts < chunks) ts <<= 1;
+    return chunks <= 64 ? ts : 0;
+}
+
+// Can a launch over a pre-scaled table with rows of ld_in floats run through the stream kernel?
+bool stream_covers(int num_nodes, int dim, int ld_in, const float* table)
+{
+    if (!g_stream_mode || force_wide_index()) return false;
+    if (ld_in % 4 != 0 || reinterpret_cast<uintptr_t>(table) % 16 != 0) return false;
+    if (stream_team((dim + 3) / 4) == 0 || (dim + 3) / 4 * 4 > ld_in) return false;
+    const unsigned long long bytes = static_cast<unsigned long long>(swizzle_padded_rows(num_nodes)) * ld_in * 4ull;
+    return bytes + 16 < (1ull << 32) && swizzle_padded_rows(num_nodes) < (1 << 24) && ld_in * 4 < (1 << 24);
+}
+
+// Stream kernel + fix-up kernel over a pre-scaled table in swizzled row order (stream_covers() holds).  `partial` holds
+// info.header.num_partials rows of ld_in floats.  Rows without slots are not written (the caller clears them).
+int launch_aggregate_stream(float* out, float* partial, const float* table, const int* scol, const StreamView& sv,
+                            const StreamInfo& info, const float* scale, int num_nodes, int dim, int ld_in,
+                            hipStream_t stream)
+{
+    const int chunks = (dim + 3) / 4;
+    const int ts = stream_team(chunks);
+    const long long padded = stream_padded_slots(info.num_slots);
+    const unsigned long long bytes = static_cast<unsigned long long>(swizzle_padded_rows(num_nodes)) * ld_in * 4ull;
+    const int num_wave_chunks = static_cast<int>(padded / kStreamWave);
+    if (num_wave_chunks == 0) return kOk;
+    const dim3 grid((num_wave_chunks + kStreamWaves - 1) / kStreamWaves), block(kStreamBlock);
+    const uintptr_t a = reinterpret_cast<uintptr_t>(out);
+    const int ovw = (dim % 4 == 0 && a % 16 == 0) ? 4 : (dim % 2 == 0 && a % 8 == 0) ? 2 : 1;
+    const int num_fix = info.header.num_fix;
+    long long fix_blocks = (static_cast<long long>(num_fix) * ts + 255) / 256;
+    if (fix_blocks > 256 * 64) fix_blocks = 256 * 64;
+    const dim3 fgrid(static_cast<unsigned>(fix_blocks < 1 ? 1 : fix_blocks));
+#define EPPGCN_STREAM(OVW_, TS_)                                                                                      \
+    do {                                                                                                              \
+        hipLaunchKernelGGL((aggregate_stream_kernel<OVW_, TS_, 8>), grid, block, 0, stream, out, partial, table,      \
+                           scol, sv.erow, sv.cev, sv.wtail, scale, num_wave_chunks, info.header.num_events,           \
+                           num_nodes, info.header.num_partials, chunks, static_cast<unsigned>(ld_in) * 4u, dim, dim,  \
+                           static_cast<unsigned>(bytes));                                                             \
+        if (num_fix > 0)                                                                                              \
+            hipLaunchKernelGGL((stream_fixup_kernel<OVW_, TS_>), fgrid, dim3(256), 0, stream, out, partial, sv.frow,  \
+                               sv.fptr, scale, sv.header, chunks, static_cast<unsigned>(ld_in) * 4u, dim, dim);       \
+    } while (0)
+#define EPPGCN_STREAM_TS(OVW_)                                                                                        \
+    do {                                                                                                              \
+        switch (ts) {                                                                                                 \
+            case 4: EPPGCN_STREAM(OVW_, 4); break;                                                                    \
+            case 8: EPPGCN_STREAM(OVW_, 8); break;                                                                    \
+            case 16: EPPGCN_STREAM(OVW_, 16); break;                                                                  \
+            case 32: EPPGCN_STREAM(OVW_, 32); break;                                                                  \
+            default: EPPGCN_STREAM(OVW_, 64); break;                                                                  \
+        }                                                                                                             \
+    } while (0)
+    if (ovw == 4) EPPGCN_STREAM_TS(4);
+    else if (ovw == 2) EPPGCN_STREAM_TS(2);
+    else EPPGCN_STREAM_TS(1);
+#undef EPPGCN_STREAM_TS
+#undef EPPGCN_STREAM
+    EPPGCN_HIP(hipGetLastError());
+    return kOk;
+}
+
+}  // namespace eppgcn

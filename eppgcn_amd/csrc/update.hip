@@ -75,6 +75,7 @@ struct RowsArgs {
     int K, M;
     int relu_in;             // apply max(x, 0) to X on load
     int vec_store;           // 0: scalar stores; 1: rows of out are 16-byte aligned; 2: the same, non-temporal
+    unsigned swz_mask;       // row r of out lives at swizzled_row(r, swz_mask): 0 = vertex order (common.hpp)
 };
 
 template <int VW, int MT, int CU>
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_rows_kernel(RowsArgs a)
 
         if (!row_ok) continue;
         const float s = a.scale ? a.scale[r] : 1.f;
-        float* __restrict__ orow = a.out + r * a.ld_out;
+        float* __restrict__ orow = a.out + static_cast<long long>(swizzled_row(static_cast<unsigned>(r), a.swz_mask)) * a.ld_out;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int m0 = mt * 16 + 4 * j;
@@ -191,7 +192,7 @@ static hipError_t launch_rows_mt(const RowsArgs& a, int mt, int cu, unsigned blo
 // operand to fit the LDS (the caller then has to use a general GEMM).
 int launch_dense_rows(float* out, int ld_out, int out_cols, const float* x, int ld_x, const float* w, long long sk,
                       long long sm, const float* scale, const float* relu_ref, int ld_ref, int relu_in,
-                      long long n, int K, int M, hipStream_t stream)
+                      long long n, int K, int M, hipStream_t stream, unsigned swz_mask)
 {
     if (n == 0 || out_cols == 0) return kOk;
     const uintptr_t xa = reinterpret_cast<uintptr_t>(x);
@@ -229,6 +230,7 @@ int launch_dense_rows(float* out, int ld_out, int out_cols, const float* x, int 
         a.K = K;
         a.M = M - c0 > 0 ? (M - c0 < cols ? M - c0 : cols) : 0;
         a.relu_in = relu_in;
+        a.swz_mask = swz_mask;
         a.vec_store = (ld_out % 4 == 0 && reinterpret_cast<uintptr_t>(a.out) % 16 == 0) ? 1 : 0;
         // measured at 4.2 M rows: a [N, 96] result 0.63 -> 0.47 ms with non-temporal stores, [N, 16] and
         // [N, 32] results unchanged or slower

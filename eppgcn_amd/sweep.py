@@ -84,11 +84,11 @@ def main():
             for width in args.widths:
                 dy = graphs.normal32(7, (n, width), dev) * mask[:, None]
                 out = torch.empty_like(dy)
-                ws = capi.feature_workspace(n, width, dev)
                 plan = None
                 if not args.no_plans and num_parts > 0 and capi.plan_recommended(n, width):
                     plan = capi.build_plan(part_pointer, edge_list, num_parts, valid_len, n, width, ids=ids,
                                            block_shift=0 if 2 * valid_len >= e else 31)
+                ws = capi.feature_workspace(n, width, dev, plan)
                 capi.set_timing(True)
                 capi.clear_time()
                 for _ in range(args.reps):

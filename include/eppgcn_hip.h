@@ -20,7 +20,7 @@
  *     first, as the reference's compactors do.  Device-side failures of the
  *     scan-based functions (a stalled look-back, a capacity overflow) are only
  *     reported by such a synchronising call, or by eppgcn_scan_status /
- *     eppgcn_build_plan_status.
+ *     eppgcn_plan_status.
  *   - Scan-based functions need a workspace of at least the number of bytes the
  *     matching *_workspace_bytes() call returns, 8-byte aligned.  The library
  *     itself allocates no device memory.
@@ -33,10 +33,14 @@
  *     request per edge; with NULL the kernel gathers the
  *     neighbour's scale per edge and needs no scratch.  The workspace may be the
  *     input pointer itself when the caller no longer needs the unscaled input
- *     (it is then overwritten with degrees[r]*in[r,:], unpadded).  With a NULL
+ *     (it is then overwritten with degrees[r]*in[r,:], unpadded).  A separate
+ *     workspace holds the row of vertex r at row eppgcn_feature_workspace_row(r)
+ *     (a permutation inside blocks of 4096 rows that spreads the gathers of graphs
+ *     with Kronecker-like vertex ids over the memory channels; the size above counts
+ *     whole blocks).  With a NULL
  *     input and a workspace, the workspace must already hold the scaled rows
- *     degrees[r]*in[r,:] at a pitch of eppgcn_feature_workspace_pitch(dim) floats
- *     with zeros in the padding (eppgcn_update_forward writes exactly that) and
+ *     degrees[r]*in[r,:] in that row order at a pitch of eppgcn_feature_workspace_pitch(dim) floats
+ *     with zeros in the padding (eppgcn_update_forward_table writes exactly that) and
  *     the scaling pass is skipped.  Results of the modes agree to rounding (a few
  *     ulp per term).
  *   - Limits: vertices and slots (CSR entries, kept edges) are int32 as in the
@@ -75,14 +79,17 @@ int eppgcn_abi_version(void);
 size_t eppgcn_feature_workspace_floats(int64_t num_nodes, int dim);
 /* Row pitch (floats) of that workspace. */
 int eppgcn_feature_workspace_pitch(int dim);
+/* Row of that workspace which holds the features of `vertex`: vertex ^ ((vertex >> 5) & 4095). */
+int64_t eppgcn_feature_workspace_row(int64_t vertex);
 
 /* Execution plan for the aggregation kernels: a copy of the groups (pointers, rows, adjacency
  * flags, column ids) re-ordered by the column block (2^shift vertices, shift chosen from `dim`;
  * pass the widest feature width the plan will be used with) of each group's first slot, original
  * order inside a block.  The aggregation functions accept it as an optional argument (NULL = the
- * groups as given): it changes no result, only which groups run together, so that the rows
- * gathered at any moment come from one window of the table and are served from L2.  It is used
- * when a feature workspace is given as well.  Build it once per graph and group array:
+ * groups as given): it changes no result beyond the order of the float additions, only which groups
+ * run together, so that the rows gathered at any moment come from one window of the table and are
+ * served from L2.  It is used when a feature workspace is given as well.  Build it once per graph and
+ * group array:
  *   forward groups : part_pointers + column_index + part2node (ids = NULL)
  *   backward path  : part_pointer + edge_list + ids (part2node = NULL)
  * num_slots = number of slots the groups cover (num_edges, or the kept length).  The plan must
@@ -92,26 +99,52 @@ int eppgcn_feature_workspace_pitch(int dim);
  * writes those with one plain store, so the output clear of a planned call skips them.
  * block_shift: 0 = column blocks sized for `dim`-wide rows; n > 0 = blocks of 2^n vertices.  31 keeps
  * the groups in one block (original order apart from the length classes): the right choice for a
- * heavily pruned path, whose few gathered rows stay cached anyway and which then still gets the
- * precomputed group descriptions and the selective clear (cfg 4, last layer: 0.244 -> 0.227 ms).
- * No counterpart in the reference. */
+ * heavily pruned path, whose few gathered rows stay cached anyway.
+ *
+ * Stream form.  The plan also holds its slots as one stream with the ends of the rows' pieces marked
+ * (a piece = consecutive plan entries that continue one another), for a second kernel in which every
+ * wave takes the same number of slots, every gather instruction is full whatever the row lengths,
+ * and no float atomics are used: pieces that are all of their row and lie inside one wave's 512 slots
+ * are stored directly, the others leave partial sums in a scratch area behind the feature table,
+ * which a small second kernel adds up row by row in a fixed order.  Results are then the same bits
+ * on every run.  An aggregation call takes this path when
+ *   - eppgcn_plan_status has been called for the plan (it reads the counts the host needs),
+ *   - a separate feature workspace is given (not NULL, not the input itself) that holds at least
+ *     eppgcn_plan_workspace_floats(plan, num_nodes, dim) floats (the table plus the partial sums),
+ *   - rows are at most 1024 bytes, the table is below 4 GB and there are fewer than 2^24 vertices,
+ * and otherwise runs the group kernel over the same plan.  A plan that contains empty groups has no
+ * stream form.  No counterpart in the reference. */
 /* 1 when a plan is expected to pay off: the [num_nodes, dim] feature table has 4 MB or more.  Large
- * tables (hundreds of MB) gain from the column-blocked order (at 268 MB the width-16 forward goes
- * from 2.03 to 1.25 ms); small ones still gain 6-8 % from the length-sorted groups, the precomputed
- * group flags and the selective output clear (R-MAT scale 16 ... 20); below that the calls are
- * launch-bound and a plan changes nothing. */
+ * tables (hundreds of MB) gain from the column-blocked order; small ones still gain from the
+ * length-sorted groups, the precomputed group flags and the selective output clear; below that the
+ * calls are launch-bound and a plan changes nothing. */
 int eppgcn_plan_recommended(int64_t num_nodes, int dim);
 size_t eppgcn_plan_bytes(int64_t num_parts, int64_t num_slots, int64_t num_nodes);
-size_t eppgcn_plan_workspace_bytes(int64_t num_parts);
+size_t eppgcn_plan_workspace_bytes(int64_t num_parts, int64_t num_slots);
 int eppgcn_build_plan(const int32_t* part_pointers, const int32_t* column_index,
                       const int32_t* part2node, const int32_t* ids, int num_parts, int64_t num_slots,
                       int num_nodes, int dim, int block_shift, void* plan, size_t plan_bytes,
                       void* workspace, size_t workspace_bytes, void* stream);
-/* eppgcn_build_plan is asynchronous and contains a look-back scan.  This call synchronises `stream`
- * and returns 0 or EPPGCN_ERR_SCAN_STALLED for the build that last used `workspace` with this
- * num_parts (a stalled scan leaves a corrupt plan, which must not be used).  Call it once after the
- * build, before the workspace is released. */
-int eppgcn_build_plan_status(const void* workspace, int num_parts, void* stream);
+/* eppgcn_build_plan is asynchronous and contains look-back scans.  This call synchronises `stream`,
+ * reads the plan's header and returns 0 or EPPGCN_ERR_SCAN_STALLED (a stalled scan leaves a corrupt
+ * plan, which must not be used).  Pass the sizes the plan was built with.  *partial_rows (may be
+ * NULL) receives the number of partial sums a call through the stream form needs room for (0 when
+ * the plan has no stream form).  The library remembers the header by the plan's address until the
+ * next eppgcn_build_plan into that address, and the aggregation calls use the stream form only for
+ * plans it knows this way: call it once after the build (the build's workspace may be released
+ * afterwards); a plan copied to another address runs through the group kernel until this has been
+ * called for the copy. */
+int eppgcn_plan_status(const void* plan, int num_parts, int64_t num_slots, int num_nodes,
+                       int64_t* partial_rows, void* stream);
+/* Floats of the feature workspace that lets a [num_nodes, dim] aggregation over `plan` take the
+ * stream form: eppgcn_feature_workspace_floats(num_nodes, dim) plus one row per partial sum (what
+ * eppgcn_plan_status reported).  Equal to eppgcn_feature_workspace_floats for NULL or a plan
+ * without (known) stream form. */
+size_t eppgcn_plan_workspace_floats(const void* plan, int64_t num_nodes, int dim);
+/* 0 keeps every planned call on the group kernel (for comparisons); 1 (default) allows the stream form. */
+void eppgcn_set_stream_mode(int on);
+/* 1 when the calling thread's last aggregation call ran the stream form, 0 when it ran the group kernel. */
+int eppgcn_last_call_used_stream(void);
 
 /* Forward neighbour-group aggregation:
  *   out[r,:] = sum_{e in groups of r} fl32(degrees[r]*degrees[col[e]]) * in[col[e],:]
@@ -307,12 +340,18 @@ int eppgcn_update_supported(int in_dim, int out_dim);
 
 /* out[r, 0:out_dim] = scale[r] * act(x[r, :]) * w, columns out_dim..ld_out-1 = 0.
  * x [num_nodes, in_dim], w [in_dim, out_dim], out rows ld_out floats apart; scale may be NULL
- * (factor 1); relu_input != 0 applies max(x, 0) on load.  With scale = degrees and
- * ld_out = eppgcn_feature_workspace_pitch(out_dim) the result is the pre-scaled feature
- * workspace the aggregation functions accept with a NULL input.
+ * (factor 1); relu_input != 0 applies max(x, 0) on load.
  * Replaces `tmp = torch::mm(input, weight)`, EPPGCN_kernel.cu:142 (spmm_forward_cuda). */
 int eppgcn_update_forward(float* out, int ld_out, const float* x, const float* w, const float* scale,
                           int relu_input, int64_t num_nodes, int in_dim, int out_dim, void* stream);
+/* The same product written as the pre-scaled feature workspace the aggregation functions accept with a
+ * NULL input: table[eppgcn_feature_workspace_row(r), :] = scale[r] * act(x[r, :]) * w, rows
+ * eppgcn_feature_workspace_pitch(out_dim) floats apart with zeros in the padding; `table` holds
+ * table_floats >= eppgcn_feature_workspace_floats(num_nodes, out_dim) floats (more when partial sums follow
+ * it, see eppgcn_plan_workspace_floats), 16-byte aligned.  No separate scaling pass is then needed. */
+int eppgcn_update_forward_table(float* table, size_t table_floats, const float* x, const float* w,
+                                const float* scale, int relu_input, int64_t num_nodes, int in_dim,
+                                int out_dim, void* stream);
 
 /* d_x[num_nodes, in_dim] = g[num_nodes, out_dim] * w^T, w [in_dim, out_dim]; with relu_ref
  * ([num_nodes, in_dim], may be NULL) entries where relu_ref <= 0 are zeroed (gradient of a

@@ -78,13 +78,16 @@ def test_argument_errors_are_reported_before_any_device_work():
         (lib.eppgcn_spmm_forward(one, p0, p0, one, one, one, one, 8, 4, 2, 1, 1, 1, p0, 0, p0, p0), "null feature"),
         (lib.eppgcn_spmm_forward(one, one, p0, one, one, one, one, 8, 0, 2, 1, 1, 1, p0, 0, p0, p0), "dim > 0"),
     ]
-    cases += [(lib.eppgcn_scan_status(p0, p0), "workspace"), (lib.eppgcn_build_plan_status(p0, 5, p0), "workspace"),
-              (lib.eppgcn_build_plan_status(one, -1, p0), "negative")]
+    cases += [(lib.eppgcn_scan_status(p0, p0), "workspace"), (lib.eppgcn_plan_status(p0, 5, 9, 4, None, p0), "plan"),
+              (lib.eppgcn_plan_status(one, -1, 0, 4, None, p0), "negative")]
     for rc, needle in cases:
         assert rc == -1
     # the message belongs to the last failing call
     assert b"negative" in lib.eppgcn_last_error()
-    assert lib.eppgcn_build_plan_status(p0, 0, p0) == 0
+    assert lib.eppgcn_plan_status(p0, 0, 0, 4, None, p0) == 0
+    # a plan the library has not seen is sized like the plain feature workspace
+    assert lib.eppgcn_plan_workspace_floats(one, 10, 22) == lib.eppgcn_feature_workspace_floats(10, 22) == 4096 * 32
+    assert [lib.eppgcn_feature_workspace_row(r) for r in (0, 31, 32, 4095, 4096, 131072 + 64)] == [0, 31, 33, 4095 ^ 127, 4096 ^ 128, (131072 + 64) ^ 2]
     assert lib.eppgcn_update_supported(96, 16) == 7 and lib.eppgcn_update_supported(2000, 16) == 6
     assert lib.eppgcn_update_supported(16, 100) == 3 and lib.eppgcn_update_supported(0, 4) == 0
     assert lib.eppgcn_feature_workspace_pitch(16) == 16 and lib.eppgcn_feature_workspace_pitch(22) == 32
@@ -123,5 +126,5 @@ def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
     env = dict(os.environ, LD_LIBRARY_PATH="/opt/rocm/lib:" + os.environ.get("LD_LIBRARY_PATH", ""))
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True, env=env).stdout.split("\n")
     from oracle import c_oracle as co
-    assert out[0].split() == [str(capi.ABI_VERSION), "32", "320", str(max(1, co.map_back_part_size(1000, 5000))), "0", "-1"]
+    assert out[0].split() == [str(capi.ABI_VERSION), "32", str(4096 * 32), str(max(1, co.map_back_part_size(1000, 5000))), "0", "-1"]
     assert "dim > 0" in out[1]

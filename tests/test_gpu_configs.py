@@ -220,8 +220,8 @@ def test_headline_size_benched_numeric_path_within_tolerance(api):
         worst[f"fwd{dim}"] = _assert_within(got, want, bound, f"planned forward, width {dim}")
         # the same launch fed by a table that is already scaled and padded (what the dense update leaves)
         pitch = api.feature_workspace_pitch(dim)
-        table = torch.zeros(n, pitch, device="cuda")
-        table[:, :dim] = x * g.degrees[:, None]
+        table = torch.zeros(api.feature_workspace(n, dim, "cuda", wl.plans[dim]).numel() // pitch, pitch, device="cuda")
+        table[api.feature_workspace_rows(n, "cuda"), :dim] = x * g.degrees[:, None]
         out.fill_(float("nan"))
         got = api.spmm_forward(None, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 32, 8,
                                g.row_pointers, out, workspace=table.view(-1), plan=wl.plans[dim], prescaled_dim=dim)

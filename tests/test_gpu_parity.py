@@ -571,13 +571,15 @@ def test_gathered_rows_bitmap_and_restricted_prescaling(api, name, ratio):
         poisoned[~want_rows] = np.nan
         for alias in (False, True):
             d_in = dev(poisoned)
-            ws = d_in if alias else torch.full((n * api.feature_workspace_pitch(dim),), float("nan"), device="cuda")
+            ws = d_in if alias else torch.full((api.feature_workspace(n, dim, "cuda").numel(),), float("nan"), device="cuda")
             got = api.ours_backward(d_in, oid, bpp, oedge, dev(s), p, part_size=8, workspace=ws,
                                     gathered_rows=bitmap)
             assert_close(got.cpu().numpy(), want, bound, f"{name} r={ratio} D={dim} alias={alias}")
             if not alias:     # rows outside the set were not written
                 pitch = api.feature_workspace_pitch(dim)
-                assert torch.isnan(ws.view(n, pitch)[dev(~want_rows)]).all()
+                rows = api.feature_workspace_rows(n, "cuda")       # where the workspace keeps each vertex
+                assert torch.isnan(ws.view(-1, pitch)[rows[dev(~want_rows)]]).all()
+                assert not torch.isnan(ws.view(-1, pitch)[rows[dev(want_rows)]][:, :dim]).any()
         plan = api.build_plan(bpp, oedge, p, v, n, dim, ids=oid)
         got = api.ours_backward(dev(poisoned), oid, bpp, oedge, dev(s), p, part_size=8, plan=plan,
                                 gathered_rows=bitmap, out=torch.full((n, dim), float("nan"), device="cuda"))

@@ -111,15 +111,19 @@ def test_update_rejects_unsupported_shapes(api):
 
 @pytest.mark.parametrize("dim", [16, 22, 7, 40])
 def test_aggregation_accepts_the_prescaled_product(api, dim):
-    """update_forward(scale=degrees, pitch of the workspace) followed by the aggregation with a
-    NULL input equals the aggregation of the unscaled product."""
+    """update_forward_table (scaled rows at the workspace's pitch and in its row order) followed by the
+    aggregation with a NULL input equals the aggregation of the unscaled product."""
     indptr, col = random_symmetric_csr(5000, 30000, 21)
     n = indptr.size - 1
     s = scale_inv_sqrt(indptr)
     x, w, _, _ = data(n, 24, dim, 6)
     pp, p2n = api.build_part(8, dev(indptr), col.size)
-    ws = api.update_forward(dev(x), dev(w), scale=dev(s), ld_out=api.feature_workspace_pitch(dim))
-    got = api.spmm_forward(None, dev(col), dev(s), pp, p2n, part_size=8, workspace=ws.view(-1), prescaled_dim=dim)
+    ws = api.update_forward_table(dev(x), dev(w), dev(s))
+    # the table is the plain scaled product, row r at row feature_workspace_rows()[r], zeros in the padding
+    pitch = api.feature_workspace_pitch(dim)
+    plain = api.update_forward(dev(x), dev(w), scale=dev(s), ld_out=pitch)
+    assert torch.equal(ws.view(-1, pitch)[api.feature_workspace_rows(n, "cuda")], plain)
+    got = api.spmm_forward(None, dev(col), dev(s), pp, p2n, part_size=8, workspace=ws, prescaled_dim=dim)
     t = co.update_forward(x, w)
     want = co.spmm_f64(t, indptr, col, s)
     bound = co.spmm_f64(np.abs(t), indptr, col, s) + 1e-30
