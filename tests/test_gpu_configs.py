@@ -160,7 +160,8 @@ def test_backward_stress_cell(api, rmat20, ratio, width, group_size):
     if num_parts > 0 and api.plan_recommended(n, width):
         plan = api.build_plan(part_pointer, edge_list, num_parts, v, n, width, ids=ids,
                               block_shift=0 if 2 * v >= e else 31)
-    ws = api.feature_workspace(n, width, "cuda")
+    # room for the partial sums of either plan: the calls run the plans' stream form
+    ws = api.feature_workspace(n, width, "cuda", (plan, st.forward_plan(width)))
 
     def pruned(dy, scale, out=None):
         return api.ours_backward(dy, ids, part_pointer, edge_list, scale, num_parts, group_size, 1, 4, 16, out, ws,
@@ -190,6 +191,13 @@ def test_backward_stress_cell(api, rmat20, ratio, width, group_size):
     dy, want, bound = st.reference(ratio, width)
     what = f"ratio {ratio} width {width} group size {group_size}"
     _assert_within(pruned(dy, g.degrees), want, bound, "pruned, " + what)
+    assert api.last_call_used_stream() == (plan is not None)
+    api.set_stream_mode(False)               # the group kernel over the same plan
+    try:
+        _assert_within(pruned(dy, g.degrees), want, bound, "pruned, group kernel, " + what)
+        assert not api.last_call_used_stream()
+    finally:
+        api.set_stream_mode(True)
     if group_size == GROUP_SIZES[0]:
         _assert_within(unpruned(dy, g.degrees), want, bound, "unpruned, " + what)
         plain = api.ours_backward(dy, ids, part_pointer, edge_list, g.degrees, num_parts, group_size, workspace=None)
@@ -211,13 +219,27 @@ def test_headline_size_benched_numeric_path_within_tolerance(api):
     w = (g.degrees[row] * g.degrees[col]).double()
     worst = {}
     for dim, path, src in ((16, wl.paths[0], wl.ngh_masks[0]), (22, wl.paths[1], wl.train_mask)):
-        ws = api.feature_workspace(n, dim, "cuda")
+        ws = api.feature_workspace(n, dim, "cuda", (wl.plans[dim], path.plan))     # as bench.py sizes it
         x = graphs.normal32(1, (n, dim), "cuda", dim)
         want, bound = _weighted_sums(g.row_pointers, col, w, x)
         out = torch.full((n, dim), float("nan"), device="cuda")
         got = api.spmm_forward(x, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 32, 8,
                                g.row_pointers, out, workspace=ws, plan=wl.plans[dim])
+        assert api.last_call_used_stream(), "the benchmark's calls run the plans' stream form"
         worst[f"fwd{dim}"] = _assert_within(got, want, bound, f"planned forward, width {dim}")
+        again = api.spmm_forward(x, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 32, 8,
+                                 g.row_pointers, None, workspace=ws, plan=wl.plans[dim])
+        assert torch.equal(got, again), "the stream form sums in a fixed order"
+        del again
+        api.set_stream_mode(False)           # the group kernel over the same plan and workspace
+        try:
+            out.fill_(float("nan"))
+            got = api.spmm_forward(x, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 32, 8,
+                                   g.row_pointers, out, workspace=ws, plan=wl.plans[dim])
+            assert not api.last_call_used_stream()
+            worst[f"fwd{dim}_groups"] = _assert_within(got, want, bound, f"planned forward, group kernel, width {dim}")
+        finally:
+            api.set_stream_mode(True)
         # the same launch fed by a table that is already scaled and padded (what the dense update leaves)
         pitch = api.feature_workspace_pitch(dim)
         table = torch.zeros(api.feature_workspace(n, dim, "cuda", wl.plans[dim]).numel() // pitch, pitch, device="cuda")
@@ -235,6 +257,7 @@ def test_headline_size_benched_numeric_path_within_tolerance(api):
         got = api.ours_backward(dy, path.ids, path.part_pointer, path.edge_list, g.degrees, path.num_parts,
                                 path.part_size, path.layer, 4, 16, out, workspace=ws, plan=path.plan,
                                 gathered_rows=path.gathered_rows)
+        assert api.last_call_used_stream()
         worst[f"bwd{dim}"] = _assert_within(got, want, bound, f"planned pruned backward, width {dim}")
         un = api.spmm_forward(dy, g.column_index, g.degrees, wl.part_ptr, wl.part2node, wl.part_size, 32, 8, None,
                               None, True, ws, plan=wl.plans[dim])
