@@ -53,7 +53,8 @@ def parse():
     ap.add_argument("--plan_shift", type=int, default=0, help="force log2 of the plan's column block")
     ap.add_argument("--plan_keep", type=int, default=-1, help="rows with at most this many groups stay together")
     ap.add_argument("--force_plan", action="store_true", help="use execution plans even for small feature tables")
-    ap.add_argument("--no_length_classes", action="store_true", help="plans without the length-class key")
+    ap.add_argument("--length_classes", action="store_true",
+                    help="plans with the length-class key (the group kernel's optimum; off by default)")
     ap.add_argument("--fused_prep", action="store_true",
                     help="prepare the backward paths with the one-pass marking + compaction instead of the "
                          "reference's separate steps (same results, same time, no edge masks)")
@@ -158,8 +159,8 @@ def main():
     log(args, "graph", g.stats(), f"{time.perf_counter() - t0:.1f}s")
     if args.plan_shift:
         capi.set_plan_shift(args.plan_shift)
-    if args.no_length_classes:
-        capi.set_plan_length_classes(False)
+    if args.length_classes:
+        capi.set_plan_length_classes(True)
     if args.plan_keep >= 0:
         capi.set_plan_keep_rows(args.plan_keep)
     t0 = time.perf_counter()
@@ -332,7 +333,7 @@ def main():
     print(json.dumps(result), flush=True)
 
 
-PROFILED_SOURCES = ("aggregate.hip", "common.hpp", "schedule.hip", "prepare.hip")
+PROFILED_SOURCES = ("aggregate.hip", "stream.hip", "common.hpp", "schedule.hip", "prepare.hip")
 
 
 def kernel_source_hash():

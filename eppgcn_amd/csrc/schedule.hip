@@ -473,8 +473,16 @@ static size_t plan_sort_state_offset(long long num_parts, long long num_slots)
 int workspace_pitch(int dim);   // aggregate.hip
 
 static int g_force_shift = 0;
-static int g_keep_rows = 8;      // in units of 32 slots: rows of up to 256 slots stay together
-static int g_length_classes = 1;
+// Defaults chosen for the stream form (R-MAT 22, ms per epoch of aggregation): rows of up to 32 / 64 / 96 / 128 /
+// 256 slots kept together -> 4.11 / 4.04 / 4.05 / 4.08 / 4.08 without length classes, 4.15 with classes and 256.
+// Length classes only help the group kernel (equal gather steps per round); under the stream form every gather
+// instruction is full anyway and the classes cost locality of the output rows (one-block plan of the last-layer
+// path: 0.227 -> 0.178 ms without them).  The group kernel, which only runs over a plan when the stream form cannot
+// (no room for the partial sums, rows beyond 1024 bytes), is 10 % slower over such a plan than over its own optimum
+// (256 slots, classes: 5.11 against 4.66 ms); eppgcn_set_plan_keep_rows(8) + eppgcn_set_plan_length_classes(1)
+// before the build give that one.
+static int g_keep_rows = 2;      // in units of 32 slots: rows of up to 64 slots stay together
+static int g_length_classes = 0;
 void set_plan_length_classes(int on) { g_length_classes = on ? 1 : 0; }
 void set_schedule_shift(int shift) { g_force_shift = shift; }
 void set_plan_keep_rows(int keep) { g_keep_rows = keep < 0 ? 0 : keep; }

@@ -249,9 +249,9 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
 
 // Rows with partial sums: out[frow[i], :] = s[frow[i]] * (sum of the partial rows fptr[i] .. fptr[i+1]), summed in
 // a fixed order, so the result does not depend on the order in which the waves of the stream kernel ran.  A wave
-// takes 64 / TS rows.  Short lists: a team of TS lanes per row walks its list.  When a row of the wave has more
-// than kFixTeamMax partial sums (a hub row cut into column blocks and waves) the whole wave works on one row at a
-// time: team t adds the partial sums t, t + TPW, ..., and the teams are summed with cross-lane operations.
+// takes 64 / TS rows.  Short lists: a team of TS lanes per row walks its list.  Rows with more than kFixTeamMax
+// partial sums (hub rows cut into column blocks and waves) are then taken one at a time by the whole wave: team t
+// adds the partial sums t, t + TPW, ..., and the teams are summed with cross-lane operations.
 constexpr int kFixTeamMax = 32;
 template <int OVW, int TS>
 __global__ __launch_bounds__(256) void stream_fixup_kernel(float* __restrict__ out, const float* __restrict__ partial,
@@ -267,20 +267,24 @@ __global__ __launch_bounds__(256) void stream_fixup_kernel(float* __restrict__ o
     const long long wave0 = static_cast<long long>(blockIdx.x) * (256 / kWave) + threadIdx.x / kWave;
     const long long waves = static_cast<long long>(gridDim.x) * (256 / kWave);
     const char* base = reinterpret_cast<const char*>(partial) + tl * 16;
+    // sixteen row loads in flight (most rows have fewer partial sums: one round trip), none of them behind a
+    // branch of its own (an index past the end is replaced by a valid one and its row by zeros)
+    constexpr int kFixLoads = 16;
     auto add_range = [&](float (&acc)[4], int beg, int end, int step) {
-        for (int k = beg; k < end; k += 4 * step) {
-            f32x4 v[4];
+        if (tl >= chunks) return;
+        for (int k = beg; k < end; k += kFixLoads * step) {
+            f32x4 v[kFixLoads];
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
-                v[u] = (k + u * step < end && tl < chunks)
-                           ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(base + static_cast<size_t>(k + u * step) * ld_bytes))
-                           : f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int u = 0; u < kFixLoads; ++u) {
+                const bool ok = k + u * step < end;
+                v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(base + static_cast<size_t>(ok ? k + u * step : k) * ld_bytes));
+                if (!ok) v[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) { acc[0] += v[u].x; acc[1] += v[u].y; acc[2] += v[u].z; acc[3] += v[u].w; }
+            for (int u = 0; u < kFixLoads; ++u) { acc[0] += v[u].x; acc[1] += v[u].y; acc[2] += v[u].z; acc[3] += v[u].w; }
         }
     };
-    auto write_row = [&](const float (&acc)[4], int r) {
-        const float s = scale[r];
+    auto write_row = [&](const float (&acc)[4], int r, float s) {
         const float v[4] = {acc[0] * s, acc[1] * s, acc[2] * s, acc[3] * s};
         float* dst = out + static_cast<size_t>(r) * ld_out + tl * 4;
 #pragma unroll
@@ -292,21 +296,25 @@ __global__ __launch_bounds__(256) void stream_fixup_kernel(float* __restrict__ o
         const bool have = i < num_fix;
         const int r = have ? frow[i] : 0;
         const int beg = have ? fptr[i] : 0, end = have ? fptr[i + 1] : 0;
-        if (!__any(end - beg > kFixTeamMax)) {
+        // short lists: every team its own row; then the long ones, one at a time, by the whole wave
+        const bool is_long = end - beg > kFixTeamMax;
+        const float s_row = have ? scale[r] : 0.f;      // under way while the partial sums are read
+        if (!is_long) {
             float acc[4] = {0.f, 0.f, 0.f, 0.f};
             add_range(acc, beg, end, 1);
-            if (have) write_row(acc, r);
-        } else {
-#pragma unroll 1
-            for (int t = 0; t < TPW; ++t) {
-                const int rb = __shfl(beg, t * TS, kWave), re = __shfl(end, t * TS, kWave), rr = __shfl(r, t * TS, kWave);
-                if (re <= rb) continue;                  // wave-uniform
-                float acc[4] = {0.f, 0.f, 0.f, 0.f};
-                add_range(acc, rb + team, re, TPW);
+            if (have) write_row(acc, r, s_row);
+        }
+        uint64_t longs = __ballot(is_long && tl == 0);
+        while (longs) {                                 // wave-uniform
+            const int lead = __builtin_ctzll(longs);
+            longs &= longs - 1;
+            const int rb = __shfl(beg, lead, kWave), re = __shfl(end, lead, kWave), rr = __shfl(r, lead, kWave);
+            const float rs = __shfl(s_row, lead, kWave);
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+            add_range(acc, rb + team, re, TPW);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[j] = cross_team_sum<TS>(acc[j]);
-                if (team == 0) write_row(acc, rr);
-            }
+            for (int j = 0; j < 4; ++j) acc[j] = cross_team_sum<TS>(acc[j]);
+            if (team == 0) write_row(acc, rr, rs);
         }
     }
 }

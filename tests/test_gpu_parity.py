@@ -327,6 +327,19 @@ def test_plan_sort_with_three_radix_passes(api):
 
 
 def _check_plan_order(api, indptr, col, ps, cases):
+    # the defaults (rows of up to 64 slots together, no length classes: the stream form's optimum) and the
+    # group kernel's optimum (256 slots, length classes)
+    for keep, classes in ((2, False), (8, True)):
+        api.set_plan_keep_rows(keep)
+        api.set_plan_length_classes(classes)
+        try:
+            _check_plan_order_with(api, indptr, col, ps, cases, 32 * keep, classes)
+        finally:
+            api.set_plan_keep_rows(2)
+            api.set_plan_length_classes(False)
+
+
+def _check_plan_order_with(api, indptr, col, ps, cases, keep_slots, classes):
     n = indptr.size - 1
     pp, p2n = co.build_part(ps, indptr)
     P = p2n.size
@@ -348,14 +361,16 @@ def _check_plan_order(api, indptr, col, ps, cases):
             assert np.array_equal(pcol[ptr[q]:ptr[q + 1]], col[pp[p]:pp[p + 1]])
         sizes = np.diff(pp)[order]
         assert np.array_equal(np.diff(ptr), sizes)
-        # sort key: column block of the group's first slot; rows of at most 256 slots (in at most 64
+        # sort key: column block of the group's first slot; rows of at most keep_slots slots (in at most 64
         # groups) use the key of their first group so that they stay together
         groups_per_row = np.bincount(p2n, minlength=n)
         row_first_group = np.concatenate([[0], np.cumsum(groups_per_row)[:-1]])
-        short = (groups_per_row <= 64) & (np.diff(indptr) <= 256)
+        short = (groups_per_row <= 64) & (np.diff(indptr) <= keep_slots)
         key_col = np.where(short[p2n], col[pp[row_first_group[p2n]]], col[pp[:-1]])[order]
-        # second key: length class (steps of 8 slots) of rows that are a single group, 3 for the rest
-        cls = np.where(groups_per_row[p2n] == 1, np.minimum(3, (np.diff(pp) - 1) >> 3), 3)[order]
+        # second key (optional): length class (steps of 8 slots) of short rows that are a single group, 3 for the rest
+        cls = np.where((groups_per_row[p2n] == 1) & short[p2n], np.minimum(3, (np.diff(pp) - 1) >> 3), 3)[order]
+        if not classes:
+            cls = np.zeros_like(cls)
         ok = False
         for shift in ([forced] if forced else range(8, 18)):
             keys = ((key_col >> shift) << 2) | cls
@@ -374,7 +389,7 @@ def _check_plan_order(api, indptr, col, ps, cases):
 
 def test_plan_block_shift_argument(api):
     """The per-call block size equals the tuning knob's, and 31 leaves one block: the groups keep
-    their order apart from the length classes of single-group rows."""
+    their order (apart from the length classes of single-group rows when those are switched on)."""
     indptr, col = GRAPHS["hub"]()
     n = indptr.size - 1
     pp, p2n = co.build_part(5, indptr)
@@ -388,6 +403,13 @@ def test_plan_block_shift_argument(api):
     for a, b in zip(knob.view(), call.view()):
         assert torch.equal(a, b)
     one = api.build_plan(*args, part2node=dev(p2n), block_shift=31)
+    ptr, row, flags, pcol = [t.cpu().numpy() for t in one.view()]
+    assert np.array_equal(row, p2n) and np.array_equal(ptr, pp) and np.array_equal(pcol, col)
+    api.set_plan_length_classes(True)
+    try:
+        one = api.build_plan(*args, part2node=dev(p2n), block_shift=31)
+    finally:
+        api.set_plan_length_classes(False)
     ptr, row, flags, pcol = [t.cpu().numpy() for t in one.view()]
     groups_per_row = np.bincount(p2n, minlength=n)
     cls = np.where(groups_per_row[p2n] == 1, np.minimum(3, (np.diff(pp) - 1) >> 3), 3)
