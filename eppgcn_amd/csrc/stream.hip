@@ -69,7 +69,8 @@ template <int OVW, int TS, int U>
 __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     float* __restrict__ out, float* __restrict__ partial, const float* __restrict__ table,
     const int* __restrict__ scol, const int* __restrict__ erow, const int* __restrict__ cev,
-    const int* __restrict__ wtail, const float* __restrict__ scale, int num_wave_chunks, int num_events,
+    const int* __restrict__ wtail, const float* __restrict__ scale, const StreamHeader* __restrict__ header,
+    int num_wave_chunks, int num_events,
     int num_nodes, int num_partials, int chunks, unsigned ld_bytes, int width_out, int ld_out, unsigned table_bytes)
 {
     constexpr int TPW = kWave / TS;
@@ -84,6 +85,9 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     const int tl = lane % TS;
     const int w = blockIdx.x * kStreamWaves + wave;
     if (w >= num_wave_chunks) return;                       // wave-uniform; the LDS rows are wave-private
+    // the counts the host remembers must be those of the plan in memory (they are unless the plan's bytes were
+    // replaced behind the library's back): a mismatch ends the kernel instead of indexing with the wrong sizes
+    if (header->num_events != num_events || header->num_partials != num_partials || header->valid != 1) return;
     int* my_row = ev_row[wave];
     float* my_scale = ev_scale[wave];
 
@@ -257,9 +261,11 @@ template <int OVW, int TS>
 __global__ __launch_bounds__(256) void stream_fixup_kernel(float* __restrict__ out, const float* __restrict__ partial,
                                                            const int* __restrict__ frow, const int* __restrict__ fptr,
                                                            const float* __restrict__ scale, const StreamHeader* header,
-                                                           int chunks, unsigned ld_bytes, int width_out, int ld_out)
+                                                           int num_partials, int chunks, unsigned ld_bytes,
+                                                           int width_out, int ld_out)
 {
     constexpr int TPW = kWave / TS;
+    if (header->num_partials != num_partials || header->valid != 1) return;   // same rule as the stream kernel
     const int num_fix = header->num_fix;
     const int lane = threadIdx.x & (kWave - 1);
     const int team = lane / TS;
@@ -362,12 +368,14 @@ int launch_aggregate_stream(float* out, float* partial, const float* table, cons
 #define EPPGCN_STREAM(OVW_, TS_)                                                                                      \
     do {                                                                                                              \
         hipLaunchKernelGGL((aggregate_stream_kernel<OVW_, TS_, 8>), grid, block, 0, stream, out, partial, table,      \
-                           scol, sv.erow, sv.cev, sv.wtail, scale, num_wave_chunks, info.header.num_events,           \
+                           scol, sv.erow, sv.cev, sv.wtail, scale, sv.header, num_wave_chunks,                        \
+                           info.header.num_events,                                                                    \
                            num_nodes, info.header.num_partials, chunks, static_cast<unsigned>(ld_in) * 4u, dim, dim,  \
                            static_cast<unsigned>(bytes));                                                             \
         if (num_fix > 0)                                                                                              \
             hipLaunchKernelGGL((stream_fixup_kernel<OVW_, TS_>), fgrid, dim3(256), 0, stream, out, partial, sv.frow,  \
-                               sv.fptr, scale, sv.header, chunks, static_cast<unsigned>(ld_in) * 4u, dim, dim);       \
+                               sv.fptr, scale, sv.header, info.header.num_partials, chunks,                           \
+                               static_cast<unsigned>(ld_in) * 4u, dim, dim);                                          \
     } while (0)
 #define EPPGCN_STREAM_TS(OVW_)                                                                                        \
     do {                                                                                                              \
