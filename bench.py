@@ -157,6 +157,8 @@ def main():
     g = graphs.make_graph(args.config, device=dev)
     torch.cuda.synchronize()
     log(args, "graph", g.stats(), f"{time.perf_counter() - t0:.1f}s")
+    if args.no_stream:
+        capi.set_stream_mode(False)      # before the plans are built: their order follows the kernel that will run
     if args.plan_shift:
         capi.set_plan_shift(args.plan_shift)
     if args.length_classes:
@@ -185,8 +187,6 @@ def main():
     ws16, ws22 = ((capi.feature_workspace(n, 16, dev, (wl.plans.get(16), p_first.plan)),
                    capi.feature_workspace(n, 22, dev, (wl.plans.get(22), p_last.plan)))
                   if not args.no_workspace else (None, None))
-    if args.no_stream:
-        capi.set_stream_mode(False)
     if args.team:
         capi.set_team_size(args.team)
     if args.rounds:

@@ -673,13 +673,15 @@ def set_scan_test_mode(spin_limit: int = 0, mute_first_tile: bool = False):
     load().eppgcn_set_scan_test_mode(int(spin_limit), int(bool(mute_first_tile)))
 
 
-def set_plan_length_classes(on: bool):
-    load().eppgcn_set_plan_length_classes(int(bool(on)))
+def set_plan_length_classes(on):
+    """True / False, or None: chosen per build from the kernel that will run over the plan (the default)."""
+    load().eppgcn_set_plan_length_classes(-1 if on is None else int(bool(on)))
 
 
 def set_plan_shift(shift: int):
     load().eppgcn_set_plan_shift(int(shift))
 
 
-def set_plan_keep_rows(groups: int):
-    load().eppgcn_set_plan_keep_rows(int(groups))
+def set_plan_keep_rows(groups):
+    """Rows of up to 32 * groups slots stay together; None: chosen per build (the default)."""
+    load().eppgcn_set_plan_keep_rows(-1 if groups is None else int(groups))

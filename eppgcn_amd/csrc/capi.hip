@@ -23,8 +23,8 @@ int schedule_shift(int);
 void set_schedule_shift(int);
 void set_plan_keep_rows(int);
 void set_plan_length_classes(int);
-int launch_build_plan(const int*, const int*, const int*, const int*, int, long long, int, int, void*, size_t, void*,
-                      size_t, hipStream_t);
+int launch_build_plan(const int*, const int*, const int*, const int*, int, long long, int, int, int, void*, size_t,
+                      void*, size_t, hipStream_t);
 void set_agg_force_team(int);
 void set_agg_force_rounds(int);
 size_t feature_workspace_floats(long long, int);
@@ -201,9 +201,8 @@ int eppgcn_build_plan(const int32_t* part_pointers, const int32_t* column_index,
     EPPGCN_REQUIRE((part2node != nullptr) != (ids != nullptr), "give exactly one of part2node (forward) and ids (backward)");
     EPPGCN_REQUIRE(aligned(plan, 256) && workspace && aligned(workspace, 256), "plan and workspace must be 256-byte aligned");
     return launch_build_plan(part_pointers, column_index, part2node, ids, num_parts, num_slots, num_nodes,
-                             block_shift > 0 ? block_shift : schedule_shift(dim), plan, plan_size, workspace,
-                             workspace_bytes,
-                             static_cast<hipStream_t>(stream));
+                             block_shift > 0 ? block_shift : schedule_shift(dim), dim, plan, plan_size, workspace,
+                             workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 size_t eppgcn_compact_workspace_bytes(int64_t length) { return compact_workspace_bytes(length < 0 ? 0 : length); }

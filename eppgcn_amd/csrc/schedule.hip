@@ -473,19 +473,28 @@ static size_t plan_sort_state_offset(long long num_parts, long long num_slots)
 int workspace_pitch(int dim);   // aggregate.hip
 
 static int g_force_shift = 0;
-// Defaults chosen for the stream form (R-MAT 22, ms per epoch of aggregation): rows of up to 32 / 64 / 96 / 128 /
-// 256 slots kept together -> 4.11 / 4.04 / 4.05 / 4.08 / 4.08 without length classes, 4.15 with classes and 256.
-// Length classes only help the group kernel (equal gather steps per round); under the stream form every gather
-// instruction is full anyway and the classes cost locality of the output rows (one-block plan of the last-layer
-// path: 0.227 -> 0.178 ms without them).  The group kernel, which only runs over a plan when the stream form cannot
-// (no room for the partial sums, rows beyond 1024 bytes), is 10 % slower over such a plan than over its own optimum
-// (256 slots, classes: 5.11 against 4.66 ms); eppgcn_set_plan_keep_rows(8) + eppgcn_set_plan_length_classes(1)
-// before the build give that one.
-static int g_keep_rows = 2;      // in units of 32 slots: rows of up to 64 slots stay together
-static int g_length_classes = 0;
-void set_plan_length_classes(int on) { g_length_classes = on ? 1 : 0; }
+// Plan policy.  Rows of up to 32 * keep slots are kept together instead of being cut at column-block borders, and
+// single-group rows may be ordered by length class inside a block.  Negative = chosen per build from the kernel that
+// will run over the plan:
+//  * stream form (R-MAT 22, ms per epoch of aggregation): rows of up to 32 / 64 / 96 / 128 / 256 slots kept together
+//    -> 4.11 / 4.04 / 4.05 / 4.08 / 4.08 without length classes, 4.15 with classes and 256.  Every gather instruction
+//    is full whatever the lengths, so the classes only cost locality of the output rows (one-block plan of the
+//    last-layer path: 0.227 -> 0.178 ms without them): keep 2, no classes.
+//  * group kernel (runs over a plan when the shape is outside the stream kernel's: table of 4 GB or more, rows beyond
+//    1024 bytes, stream mode off): equal gather steps per round matter, 256 slots with classes is its optimum and the
+//    stream policy costs it 10 % (5.11 against 4.66 ms at R-MAT 22; 22.6 against 20.6 ms at R-MAT 24): keep 8, classes.
+static int g_keep_rows = -1;         // in units of 32 slots
+static int g_length_classes = -1;
+void set_plan_length_classes(int on) { g_length_classes = on < 0 ? -1 : on ? 1 : 0; }
+void set_plan_keep_rows(int keep) { g_keep_rows = keep < 0 ? -1 : keep; }
+bool stream_covers(int num_nodes, int dim, int ld_in, const float* table);   // stream.hip
+static void plan_policy(int num_nodes, int dim, int* keep_rows, int* length_classes)
+{
+    const bool stream = stream_covers(num_nodes, dim, workspace_pitch(dim), nullptr);
+    *keep_rows = g_keep_rows >= 0 ? g_keep_rows : stream ? 2 : 8;
+    *length_classes = g_length_classes >= 0 ? g_length_classes : stream ? 0 : 1;
+}
 void set_schedule_shift(int shift) { g_force_shift = shift; }
-void set_plan_keep_rows(int keep) { g_keep_rows = keep < 0 ? 0 : keep; }
 
 int schedule_shift(int dim)
 {
@@ -613,10 +622,12 @@ static int launch_build_stream(PlanView v, StreamView sv, int num_parts, long lo
 }
 
 int launch_build_plan(const int* part_ptr, const int* col, const int* part2node, const int* ids, int num_parts,
-                      long long num_slots, int num_nodes, int shift, void* plan, size_t plan_size, void* workspace,
-                      size_t workspace_bytes, hipStream_t stream)
+                      long long num_slots, int num_nodes, int shift, int dim, void* plan, size_t plan_size,
+                      void* workspace, size_t workspace_bytes, hipStream_t stream)
 {
     forget_stream_info(plan);
+    int keep_rows, length_classes;
+    plan_policy(num_nodes, dim, &keep_rows, &length_classes);
     if (num_parts <= 0) return kOk;
     if (plan_size < plan_bytes(num_parts, num_slots, num_nodes)) {
         set_error("build_plan: plan buffer smaller than eppgcn_plan_bytes(num_parts, num_slots, num_nodes)");
@@ -639,14 +650,14 @@ int launch_build_plan(const int* part_ptr, const int* col, const int* part2node,
     ScanState* sort_st = reinterpret_cast<ScanState*>(base + plan_sort_state_offset(num_parts, num_slots));
     int bits = 1;
     while (bits < 30 && (static_cast<long long>(num_nodes) >> shift) >= (1ll << bits)) ++bits;
-    if (g_length_classes) bits += 2;
+    if (length_classes) bits += 2;
     if (plan_workspace_bytes(num_parts, num_slots) > workspace_bytes) {
         set_error("build_plan: workspace smaller than eppgcn_plan_workspace_bytes(num_parts, num_slots)");
         return kErrInvalidArgument;
     }
     const unsigned blocks = static_cast<unsigned>((num_parts + 255) / 256);
     hipLaunchKernelGGL(plan_keys_kernel, dim3(blocks), dim3(256), 0, stream, part_ptr, col, part2node, ids, num_parts,
-                       shift, g_keep_rows * 32, g_length_classes, keys_in);
+                       shift, keep_rows * 32, length_classes, keys_in);
     EPPGCN_HIP(hipGetLastError());
     if (int rc = stable_sort_by_key(keys_in, keys_out, order_tmp, order, num_parts, bits, temp, sort_st, stream)) return rc;
     hipLaunchKernelGGL(plan_sizes_kernel, dim3(blocks), dim3(256), 0, stream, part_ptr, order, num_parts, sizes);

@@ -36,6 +36,7 @@ namespace eppgcn {
 
 constexpr int kStreamBlock = 256;
 constexpr int kStreamWaves = kStreamBlock / kWave;
+constexpr int kStreamShiftTeams = 8;   // teams up to this size address rows with a shift (power-of-two row pitch)
 constexpr int kStreamEvents = kStreamWave;       // pieces that can end in a wave's slots
 constexpr unsigned kNoRowOffset = 0xffffffffu;
 
@@ -105,6 +106,7 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     const __amdgpu_buffer_rsrc_t rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(table), 0,
                                                                           static_cast<int>(table_bytes), 0x00020000);
     const unsigned lane_off = tl < chunks ? static_cast<unsigned>(tl) * 16u : kNoRowOffset;
+    const unsigned row_step = static_cast<unsigned>(__builtin_ctz(ld_bytes));       // wave-uniform
 
     // batch (s, part): the ids come from lane s of the team, registers part * U ...
     auto issue = [&](StreamBatch<U>& b, int s, auto part) {
@@ -115,7 +117,12 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const unsigned id = swizzled_row(b.c[u] & 0x7fffffffu);      // the table's row order (common.hpp)
-            const unsigned off = lane_off == kNoRowOffset ? kNoRowOffset : __umul24(id, ld_bytes) + lane_off;
+            // rows of a narrow team are a power of two bytes apart (row_step = log2): a shift serves any row count
+            // of a table below 4 GB; wider rows use the 24-bit multiply (the host checks the row count)
+            unsigned row_off;
+            if constexpr (TS <= kStreamShiftTeams) row_off = id << row_step;
+            else row_off = __umul24(id, ld_bytes);
+            const unsigned off = lane_off == kNoRowOffset ? kNoRowOffset : row_off + lane_off;
             b.v[u] = __builtin_amdgcn_raw_buffer_load_b128(rows, off, 0, 0);
         }
     };
@@ -343,7 +350,11 @@ bool stream_covers(int num_nodes, int dim, int ld_in, const float* table)
     if (ld_in % 4 != 0 || reinterpret_cast<uintptr_t>(table) % 16 != 0) return false;
     if (stream_team((dim + 3) / 4) == 0 || (dim + 3) / 4 * 4 > ld_in) return false;
     const unsigned long long bytes = static_cast<unsigned long long>(swizzle_padded_rows(num_nodes)) * ld_in * 4ull;
-    return bytes + 16 < (1ull << 32) && swizzle_padded_rows(num_nodes) < (1 << 24) && ld_in * 4 < (1 << 24);
+    if (bytes + 16 >= (1ull << 32)) return false;                      // 32-bit byte offsets into the table
+    // teams of up to kStreamShiftTeams lanes turn a row into a byte offset with a shift: rows a power of two bytes apart
+    // (the workspace's pitch for such widths), any row count; wider teams multiply 24-bit operands
+    if (stream_team((dim + 3) / 4) <= kStreamShiftTeams) return (ld_in & (ld_in - 1)) == 0;
+    return swizzle_padded_rows(num_nodes) < (1 << 24) && ld_in * 4 < (1 << 24);
 }
 
 // Stream kernel + fix-up kernel over a pre-scaled table in swizzled row order (stream_covers() holds).  `partial` holds

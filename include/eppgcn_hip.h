@@ -111,7 +111,9 @@ int64_t eppgcn_feature_workspace_row(int64_t vertex);
  *   - eppgcn_plan_status has been called for the plan (it reads the counts the host needs),
  *   - a separate feature workspace is given (not NULL, not the input itself) that holds at least
  *     eppgcn_plan_workspace_floats(plan, num_nodes, dim) floats (the table plus the partial sums),
- *   - rows are at most 1024 bytes, the table is below 4 GB and there are fewer than 2^24 vertices,
+ *   - rows are at most 1024 bytes and the table is below 4 GB; rows of more than 128 bytes also need
+ *     fewer than 2^24 vertices (narrower rows are a power of two bytes apart and are addressed with a
+ *     shift, wider ones with a 24-bit multiply),
  * and otherwise runs the group kernel over the same plan.  A plan that contains empty groups has no
  * stream form.  No counterpart in the reference. */
 /* 1 when a plan is expected to pay off: the [num_nodes, dim] feature table has 4 MB or more.  Large
@@ -401,11 +403,15 @@ void eppgcn_set_scan_test_mode(unsigned spin_limit, int mute_first_tile);
 /* Forces the column block size of eppgcn_build_plan to 2^shift vertices (0 = choose from the
  * feature width).  For tuning runs. */
 void eppgcn_set_plan_shift(int shift);
-/* Rows of at most 32 * groups slots (and at most 64 groups) stay together in a plan (default 8, i.e.
- * 256 slots; 0 = block every group). */
+/* Plan policy (tuning runs).  Rows of at most 32 * groups slots (and at most 64 groups) stay together in
+ * a plan instead of being cut at column-block borders (0 = block every group).  Negative (the default) =
+ * chosen per build: 2 when the launch shape (num_nodes, dim) is one the stream form runs, 8 when the
+ * group kernel will run over the plan. */
 void eppgcn_set_plan_keep_rows(int groups);
 /* Within a column block, order single-group rows by length class (1-8, 9-16, 17-24, 25+ slots) so
- * that the groups of one round take the same number of gather steps (default on). */
+ * that the groups of one round take the same number of gather steps.  1 on, 0 off, negative (the
+ * default) = per build: off for the stream form (its gather instructions are full whatever the
+ * lengths), on for the group kernel. */
 void eppgcn_set_plan_length_classes(int on);
 
 #ifdef __cplusplus

@@ -266,3 +266,35 @@ def test_headline_size_benched_numeric_path_within_tolerance(api):
         assert ((got - un).abs().double() <= 2 * RTOL * bound + 1e-30).all()
         del dy, want, bound, got, un, out, ws
     print("worst err / limit:", {k: round(v, 4) for k, v in worst.items()})
+
+
+# ----------------------------------------------------------------------------- more than 2^24 vertices
+def test_stream_form_with_25_bit_vertex_ids(api):
+    """R-MAT scale 25, one generated pair per vertex (33.5 M vertices, many of them isolated): vertex ids and the
+    padding id need 25 bits.  At width 16 (64-byte rows, a 2 GB table) the stream form addresses rows with a
+    shift and runs; at width 22 the table passes 4 GB and the group kernel takes the same plan.  Both against
+    the float64 sparse product."""
+    from eppgcn_amd import graphs
+    g = graphs.make_graph("rmat:25:1", device="cuda")
+    n, e = g.num_nodes, g.num_edges
+    assert n == 1 << 25 and int(g.column_index.max()) >= 1 << 24
+    ps = 4
+    part_ptr, part2node = api.build_part(ps, g.row_pointers, e)
+    col = g.column_index.long()
+    w = (g.degrees[g.row_index()] * g.degrees[col]).double()
+    for dim, streams in ((16, True), (22, False)):
+        plan = api.build_plan(part_ptr, g.column_index, part2node.numel(), e, n, dim, part2node=part2node)
+        ws = api.feature_workspace(n, dim, "cuda", plan)
+        x = graphs.normal32(3, (n, dim), "cuda", dim)
+        want, bound = _weighted_sums(g.row_pointers, col, w, x)
+        out = torch.full((n, dim), float("nan"), device="cuda")
+        got = api.spmm_forward(x, g.column_index, g.degrees, part_ptr, part2node, ps, 32, 8, g.row_pointers, out,
+                               workspace=ws, plan=plan)
+        assert api.last_call_used_stream() == streams
+        _assert_within(got, want, bound, f"planned forward at 2^25 vertices, width {dim}")
+        if streams:
+            again = api.spmm_forward(x, g.column_index, g.degrees, part_ptr, part2node, ps, 32, 8, g.row_pointers,
+                                     None, workspace=ws, plan=plan)
+            assert torch.equal(got, again), "the stream form sums in a fixed order"
+            del again
+        del plan, ws, x, want, bound, out, got

@@ -335,8 +335,8 @@ def _check_plan_order(api, indptr, col, ps, cases):
         try:
             _check_plan_order_with(api, indptr, col, ps, cases, 32 * keep, classes)
         finally:
-            api.set_plan_keep_rows(2)
-            api.set_plan_length_classes(False)
+            api.set_plan_keep_rows(None)
+            api.set_plan_length_classes(None)
 
 
 def _check_plan_order_with(api, indptr, col, ps, cases, keep_slots, classes):
@@ -409,7 +409,7 @@ def test_plan_block_shift_argument(api):
     try:
         one = api.build_plan(*args, part2node=dev(p2n), block_shift=31)
     finally:
-        api.set_plan_length_classes(False)
+        api.set_plan_length_classes(None)
     ptr, row, flags, pcol = [t.cpu().numpy() for t in one.view()]
     groups_per_row = np.bincount(p2n, minlength=n)
     cls = np.where(groups_per_row[p2n] == 1, np.minimum(3, (np.diff(pp) - 1) >> 3), 3)
