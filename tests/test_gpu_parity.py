@@ -419,6 +419,39 @@ def test_plan_block_shift_argument(api):
         api.build_plan(*args, part2node=dev(p2n), block_shift=32)
 
 
+def test_plan_policy_follows_the_kernel_that_will_run(api):
+    """With the policy left automatic a plan is ordered for the kernel that will run over it: the stream form's
+    order (rows of up to 64 slots together, no length classes) when the launch shape is one the stream kernel
+    covers, the group kernel's (256 slots, length classes) when the stream mode is off at build time or the rows
+    are wider than the stream kernel takes (more than 1024 bytes)."""
+    indptr, col = GRAPHS["medium"]()
+    n = indptr.size - 1
+    pp, p2n = co.build_part(31, indptr)       # single-group rows of 1 ... 31 slots: all four length classes
+
+    def build(dim, keep=None, classes=None):
+        api.set_plan_keep_rows(keep)
+        api.set_plan_length_classes(classes)
+        try:
+            return api.build_plan(dev(pp), dev(col), p2n.size, col.size, n, dim, part2node=dev(p2n), block_shift=8)
+        finally:
+            api.set_plan_keep_rows(None)
+            api.set_plan_length_classes(None)
+
+    def same(a, b):
+        return all(torch.equal(x, y) for x, y in zip(a.view(), b.view()))
+
+    stream_order, group_order = build(16, 2, False), build(16, 8, True)
+    assert not same(stream_order, group_order), "the two policies must differ on this graph for the test to mean anything"
+    assert same(build(16), stream_order)
+    api.set_stream_mode(False)
+    try:
+        assert same(build(16), group_order)
+    finally:
+        api.set_stream_mode(True)
+    assert same(build(260), build(260, 8, True))          # 1040-byte rows: group kernel
+    assert same(build(256), build(256, 2, False))         # 1024-byte rows: stream kernel
+
+
 @pytest.mark.parametrize("rounds", [0, 1, 3])
 @pytest.mark.parametrize("dim", [16, 22, 64, 256])
 @pytest.mark.parametrize("shift", [0, 3, 20])

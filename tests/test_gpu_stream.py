@@ -309,3 +309,70 @@ def test_stream_from_a_table_written_by_the_dense_update(api):
     want = co.spmm_f64(t, indptr, col, s)
     bound = co.spmm_f64(np.abs(x) @ np.abs(w), indptr, col, s) + 1e-30
     assert_close(got.cpu().numpy(), want, 2 * bound, "product then aggregation")
+
+
+def _ragged_csr(rng, n):
+    """Rows of very different lengths: a share of empty rows, mostly short ones, a few hubs of up to thousands of
+    slots (longer than a wave's 512 slots, cut into many column blocks)."""
+    deg = rng.geometric(rng.uniform(0.05, 0.6), n).astype(np.int64)
+    deg[rng.random(n) < rng.uniform(0.0, 0.5)] = 0
+    hubs = rng.integers(0, n, rng.integers(0, 4))
+    deg[hubs] = rng.integers(300, 4000, hubs.size)
+    deg = np.minimum(deg, n)
+    indptr = np.zeros(n + 1, np.int64)
+    np.cumsum(deg, out=indptr[1:])
+    col = np.concatenate([np.sort(rng.choice(n, d, replace=False)) for d in deg] or [np.zeros(0, np.int64)])
+    return indptr.astype(np.int32), col.astype(np.int32)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_stream_random_ragged_graphs_exact(api, seed):
+    """Random ragged graphs, group sizes, column-block sizes, keep-together bounds and widths: the stream arrays
+    against the host construction, and with integer features and unit scales the forward sums and the pruned
+    backward sums exactly (every partial sum and every order of adding them is exact in fp32)."""
+    rng = np.random.default_rng(1000 + seed)
+    n = int(rng.integers(1, 6000))
+    indptr, col = _ragged_csr(rng, n)
+    if col.size == 0:
+        indptr, col = np.array([0] * n + [1], np.int32), np.zeros(1, np.int32)
+    ps = int(rng.choice([1, 2, 3, 5, 8, 16, 31, 32, 64]))
+    shift = int(rng.choice([3, 5, 8, 11, 14, 31]))
+    dim = int(rng.choice([1, 2, 4, 6, 16, 22, 33, 64, 130]))
+    api.set_plan_keep_rows(int(rng.choice([0, 1, 2, 8])))
+    api.set_plan_length_classes(bool(rng.integers(0, 2)))
+    try:
+        ones = np.ones(n, np.float32)
+        x = rng.integers(-4, 5, (n, dim)).astype(np.float32)
+        pp, p2n = co.build_part(ps, indptr)
+        plan = api.build_plan(dev(pp), dev(col), p2n.size, col.size, n, dim, part2node=dev(p2n), block_shift=shift)
+        check_stream_form(api, plan, n)
+        out = torch.full((n, dim), float("nan"), device="cuda")
+        api.spmm_forward(dev(x), dev(col), dev(ones), dev(pp), dev(p2n), part_size=ps, plan=plan, out=out)
+        assert api.last_call_used_stream()
+        what = f"seed {seed}: n {n}, slots {col.size}, group size {ps}, shift {shift}, width {dim}"
+        assert np.array_equal(out.cpu().numpy(), co.spmm_f64(x, indptr, col, ones).astype(np.float32)), what
+
+        # the pruned backward over the path of a random source mask
+        src = rng.random(n) < rng.uniform(0.02, 0.9)
+        mask = torch.full((col.size,), -1, dtype=torch.int32, device="cuda")
+        degs = torch.zeros(n, dtype=torch.int32, device="cuda")
+        api.mask_forward(dev(p2n), dev(pp), dev(col), dev(src), None, mask, degs, True)
+        oid, oedge, v = api.compact_back_edge(mask, dev(col))
+        if v == 0:
+            return
+        bps = int(rng.choice([1, 4, 16, 32]))
+        bpp, p, _ = api.split_back_part(degs, col.size, bps)
+        bitmap, _ = api.mark_gathered_rows(oedge, v, n)
+        dy = x * src[:, None]
+        poisoned = dy.copy()
+        poisoned[~src] = np.nan
+        bplan = api.build_plan(bpp, oedge, p, v, n, dim, ids=oid, block_shift=shift)
+        check_stream_form(api, bplan, n)
+        out.fill_(float("nan"))
+        api.ours_backward(dev(poisoned), oid, bpp, oedge, dev(ones), p, part_size=bps, plan=bplan, gathered_rows=bitmap,
+                          out=out)
+        assert api.last_call_used_stream()
+        assert np.array_equal(out.cpu().numpy(), co.spmm_f64(dy, indptr, col, ones).astype(np.float32)), what + " (backward)"
+    finally:
+        api.set_plan_keep_rows(None)
+        api.set_plan_length_classes(None)
