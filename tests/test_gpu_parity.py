@@ -95,6 +95,21 @@ def test_compact_back_edge_bit_exact(api, length, density):
     assert np.array_equal(oedge.cpu().numpy(), want_edge)
 
 
+@pytest.mark.parametrize("shift", [1, 2, 3])
+@pytest.mark.parametrize("length", [1, 4095, 16384, 16385, 70001])
+def test_compact_back_edge_unaligned_arrays(api, length, shift):
+    """Arrays that start at any 4-byte boundary (views into larger buffers); lengths around the kernel's tile of
+    16384 items."""
+    rng = np.random.default_rng(length + shift)
+    em = np.where(rng.random(length + shift) < 0.4, rng.integers(0, 1 << 20, length + shift), -1).astype(np.int32)
+    col = rng.integers(0, 1 << 20, length + shift).astype(np.int32)
+    want_id, want_edge, want_v = cf.compact_mask(em[shift:], col[shift:])
+    for a, b in ((dev(em)[shift:], dev(col)[shift:]), (dev(em[shift:]), dev(col)[shift:]), (dev(em)[shift:], dev(col[shift:]))):
+        oid, oedge, v = api.compact_back_edge(a, b)
+        assert v == want_v
+        assert np.array_equal(oid.cpu().numpy(), want_id) and np.array_equal(oedge.cpu().numpy(), want_edge)
+
+
 def test_compact_is_deterministic_across_runs(api):
     rng = np.random.default_rng(5)
     length = 3_000_000
