@@ -502,3 +502,10 @@ def test_epoch_replayed_from_a_hip_graph_follows_the_eager_trajectory(GNNA):
     w_e = eager.model.convs[0].weights.detach()
     w_g = graphed.model.convs[0].weights.detach()
     assert torch.allclose(w_e, w_g, rtol=1e-4, atol=1e-6)
+
+
+def test_entry_point_smoke_runs():
+    """The repository's smoke entry point (one small pass of the whole path on cuda:0 against the checker) is part
+    of the suite, so that a change of the library's contracts cannot leave it behind."""
+    import __graft_entry__ as entry
+    entry.smoke()
