@@ -243,6 +243,7 @@ def main():
     reps = max(3, min(args.steps, 10))
     for name, fn, nbytes in kernels:
         call_ms = _event_ms(fn, reps)
+        streamed = capi.last_call_used_stream()       # which kernel family the call just ran
         which = 0 if name.startswith("fwd") else 1
         capi.set_timing(True)
         capi.clear_time()
@@ -252,7 +253,7 @@ def main():
         capi.set_timing(False)
         capi.clear_time()
         per_kernel[name] = {"call_ms": round(call_ms, 4), "kernel_ms": round(ms, 4), "clear_ms": round(clear_ms, 4),
-                            "prescale_ms": round(scale_ms, 4), "alg_bytes": nbytes,
+                            "prescale_ms": round(scale_ms, 4), "stream_form": streamed, "alg_bytes": nbytes,
                             "alg_GBps": round(nbytes / call_ms / 1e6, 1),
                             "pct_peak": round(nbytes / call_ms / 1e6 / PEAK_HBM_GBS * 100, 2),
                             "kernel_only_pct_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS * 100, 2)}
@@ -295,7 +296,11 @@ def main():
                    "backward_groups": [p.num_parts for p in wl.paths], "max_degree": g.stats()["max_degree"],
                    "feature_workspace": not args.no_workspace,
                    "column_blocked_plan": bool(wl.plans),
-                   "stream_form": bool(wl.plans) and not args.no_stream and not args.no_workspace},
+                   "stream_form": all(k["stream_form"] for k in per_kernel.values()),
+                   "partial_sum_rows": {"fwd_agg_d16": getattr(wl.plans.get(16), "partial_rows", 0),
+                                        "fwd_agg_d22": getattr(wl.plans.get(22), "partial_rows", 0),
+                                        "bwd_agg_d22_last": getattr(p_last.plan, "partial_rows", 0),
+                                        "bwd_agg_d16_first": getattr(p_first.plan, "partial_rows", 0)}},
         "agg_ms_per_epoch": round(ms_per_step, 4), "alg_bytes_per_epoch": bytes_epoch,
         "pct_of_peak_hbm": round(value / PEAK_HBM_GBS * 100, 2),
         "value_is": "algorithmic (gather-model) bytes of the epoch / wall time; not measured HBM traffic",
