@@ -791,10 +791,14 @@ def test_fused_and_stepwise_path_preparation_agree_at_scale(api):
 
 
 # ----------------------------------------------------------------------------- HIP graph capture
-def test_aggregation_calls_replay_from_a_hip_graph(api):
+@pytest.mark.parametrize("stream_form", [False, True])
+def test_aggregation_calls_replay_from_a_hip_graph(api, stream_form):
     """The library allocates nothing and clears its outputs with a fill kernel (no memset nodes),
     so a caller can capture the calls into a HIP graph.  Every replay, with eager work and
-    synchronisations in between and fresh inputs each time, must equal the eager result."""
+    synchronisations in between and fresh inputs each time, must equal the eager result - through the
+    group kernel (workspace without room for partial sums) and through the plans' stream form (pre-scaling
+    pass, stream kernel, fix-up kernel and the clear of rows without slots all recorded), where replay and
+    eager run must agree bit for bit."""
     indptr, col = random_symmetric_csr(6000, 40000, 77)
     n = indptr.size - 1
     s = scale_inv_sqrt(indptr)
@@ -808,17 +812,22 @@ def test_aggregation_calls_replay_from_a_hip_graph(api):
     part_pointer, num_parts, _ = api.split_back_part(degs, col.size, 8)
     x = torch.zeros((n, 22), device="cuda")
     y_fwd, y_bwd = torch.empty_like(x), torch.empty_like(x)
-    ws = api.feature_workspace(n, 22, "cuda")
     # with a plan (selective output clear) and the gathered-rows bitmap (restricted pre-scaling)
     plan = api.build_plan(pp, d_col, p2n.numel(), col.size, n, 22, part2node=p2n)
+    bplan = api.build_plan(part_pointer, edge_list, num_parts, v, n, 22, ids=ids) if stream_form else None
+    ws = api.feature_workspace(n, 22, "cuda", (plan, bplan) if stream_form else None)
     bitmap, _ = api.mark_gathered_rows(edge_list, v, n)
+    used = []
 
     def both():
         api.spmm_forward(x, d_col, d_s, pp, p2n, 8, out=y_fwd, workspace=ws, plan=plan)
+        used.append(api.last_call_used_stream())
         api.ours_backward(x, ids, part_pointer, edge_list, d_s, num_parts, 8, out=y_bwd, workspace=ws,
-                          gathered_rows=bitmap)
+                          plan=bplan, gathered_rows=bitmap)
+        used.append(api.last_call_used_stream())
 
     both()                                    # warm-up outside the capture
+    assert used == [stream_form, stream_form]
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
@@ -836,6 +845,8 @@ def test_aggregation_calls_replay_from_a_hip_graph(api):
         assert_close(got_f.cpu().numpy(), y_fwd.cpu().numpy().astype(np.float64), 2 * bound, f"forward replay {rep}")
         assert_close(got_b.cpu().numpy(), y_bwd.cpu().numpy().astype(np.float64), 2 * bound, f"backward replay {rep}")
         assert_close(got_f.cpu().numpy(), co.spmm_f64(xn, indptr, col, s), bound, f"forward replay {rep} vs checker")
+        if stream_form:
+            assert torch.equal(got_f, y_fwd) and torch.equal(got_b, y_bwd), "the stream form sums in a fixed order"
 
 
 # ----------------------------------------------------------------------------- headline size
