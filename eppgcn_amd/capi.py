@@ -23,7 +23,7 @@ EXPORTS = [
     "eppgcn_build_part", "eppgcn_get_ginfo", "eppgcn_set_timing", "eppgcn_print_time",
     "eppgcn_clear_time", "eppgcn_get_time_ms", "eppgcn_set_team_size", "eppgcn_set_rounds", "eppgcn_set_plan_shift", "eppgcn_set_plan_keep_rows",
     "eppgcn_feature_workspace_pitch", "eppgcn_update_forward", "eppgcn_update_backward_input",
-    "eppgcn_update_workspace_bytes", "eppgcn_update_backward_weight", "eppgcn_update_supported",
+    "eppgcn_update_workspace_bytes", "eppgcn_update_backward_weight", "eppgcn_update_supported", "eppgcn_update_backward",
     "eppgcn_mark_compact_workspace_bytes", "eppgcn_mark_compact", "eppgcn_set_plan_length_classes",
     "eppgcn_mark_gathered_rows", "eppgcn_set_wide_index", "eppgcn_wave64_back_part_size",
     "eppgcn_compact_back_edge_static", "eppgcn_compact_back_edge_static_max_length",
@@ -32,7 +32,7 @@ EXPORTS = [
     "eppgcn_update_forward_table", "eppgcn_feature_workspace_row",
 ]
 
-ABI_VERSION = 13      # what eppgcn_abi_version() of a matching library returns
+ABI_VERSION = 14      # what eppgcn_abi_version() of a matching library returns
 
 _lib = None
 
@@ -136,7 +136,9 @@ def load():
     lib.eppgcn_update_workspace_bytes.argtypes = [i64, i, i]
     lib.eppgcn_update_workspace_bytes.restype = sz
     lib.eppgcn_update_backward_weight.argtypes = [p, p, p, i, i64, i, i, p, sz, p]
-    for name in ("eppgcn_update_forward", "eppgcn_update_backward_input", "eppgcn_update_backward_weight"):
+    lib.eppgcn_update_backward.argtypes = [p, p, p, p, p, i, i64, i, i, p, sz, p]
+    for name in ("eppgcn_update_forward", "eppgcn_update_backward_input", "eppgcn_update_backward_weight",
+                 "eppgcn_update_backward"):
         getattr(lib, name).restype = i
     for name in ("eppgcn_spmm_forward", "eppgcn_spmm_backward", "eppgcn_ours_backward", "eppgcn_mask_forward",
                  "eppgcn_compact_back_edge", "eppgcn_count_nonzero", "eppgcn_map_back_part_size",
@@ -266,6 +268,25 @@ def update_backward_weight(x, g, relu_input=False):
     _check(lib.eppgcn_update_backward_weight(_ptr(d_w), _ptr(x), _ptr(g), int(bool(relu_input)), n, k, m, _ptr(ws),
                                              nbytes, _stream()))
     return d_w
+
+
+def update_backward(x, w, g, relu_input=False):
+    """Both gradients of a layer ``act(x) @ w`` from the gradient ``g`` of the product, in one call:
+    -> (d_x [N, in_dim], d_w [in_dim, out_dim]); the same bits as update_backward_input (with
+    ``relu_ref=x`` when ``relu_input``) and update_backward_weight."""
+    lib = load()
+    _dev(x, torch.float32, "x"); _dev(w, torch.float32, "w"); _dev(g, torch.float32, "g")
+    n, k = x.shape
+    m = g.shape[1]
+    if g.shape[0] != n or tuple(w.shape) != (k, m):
+        raise EppgcnError("x [N, in_dim], w [in_dim, out_dim] and g [N, out_dim] are expected")
+    d_x = torch.empty((n, k), dtype=torch.float32, device=x.device)
+    d_w = torch.empty((k, m), dtype=torch.float32, device=x.device)
+    nbytes = lib.eppgcn_update_workspace_bytes(n, k, m)
+    ws = torch.empty(max(1, (nbytes + 3) // 4), dtype=torch.float32, device=x.device)
+    _check(lib.eppgcn_update_backward(_ptr(d_x), _ptr(d_w), _ptr(x), _ptr(g), _ptr(w), int(bool(relu_input)), n, k, m,
+                                      _ptr(ws), nbytes, _stream()))
+    return d_x, d_w
 
 
 def _feature_workspace(workspace, feats, plan=None):

@@ -33,6 +33,9 @@ int launch_dense_rows(float*, int, int, const float*, int, const float*, long lo
                       const float*, int, int, long long, int, int, hipStream_t, unsigned);
 size_t update_workspace_bytes(long long, int, int);
 int launch_dense_weight(float*, const float*, int, const float*, int, int, long long, int, int, void*, hipStream_t);
+bool dense_backward_fused_covers(int, int, const float*, const float*);
+int launch_dense_backward(float*, float*, const float*, const float*, const float*, int, long long, int, int, void*,
+                          hipStream_t);
 size_t compact_workspace_bytes(long long);
 size_t split_workspace_bytes(long long);
 int launch_mask_forward(const int*, const int*, const int*, const uint8_t*, uint8_t*, int*, int*, int, long long, int,
@@ -87,7 +90,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 13; }
+int eppgcn_abi_version(void) { return 14; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -593,6 +596,30 @@ int eppgcn_update_backward_weight(float* d_w, const float* x, const float* g, in
                    "workspace smaller than eppgcn_update_workspace_bytes(num_nodes, in_dim, out_dim)");
     return launch_dense_weight(d_w, x, in_dim, g, out_dim, relu_input ? 1 : 0, num_nodes, in_dim, out_dim, workspace,
                                static_cast<hipStream_t>(stream));
+}
+
+int eppgcn_update_backward(float* d_x, float* d_w, const float* x, const float* g, const float* w, int relu_input,
+                           int64_t num_nodes, int in_dim, int out_dim, void* workspace, size_t workspace_bytes,
+                           void* stream)
+{
+    EPPGCN_REQUIRE(num_nodes >= 0 && in_dim > 0 && out_dim > 0, "num_nodes >= 0, in_dim > 0, out_dim > 0 required");
+    EPPGCN_REQUIRE(d_w, "null output pointer");
+    EPPGCN_REQUIRE(num_nodes == 0 || (d_x && x && g && w), "null matrix pointer");
+    EPPGCN_REQUIRE(aligned(d_x, 4) && aligned(d_w, 4) && aligned(x, 4) && aligned(g, 4) && aligned(w, 4),
+                   "matrix pointers must be 4-byte aligned");
+    EPPGCN_REQUIRE(d_x != g && d_x != x, "the input gradient cannot be written over an input");
+    EPPGCN_REQUIRE(num_nodes == 0 || (workspace && aligned(workspace, 4) &&
+                                      workspace_bytes >= update_workspace_bytes(num_nodes, in_dim, out_dim)),
+                   "workspace smaller than eppgcn_update_workspace_bytes(num_nodes, in_dim, out_dim)");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (num_nodes == 0 || dense_backward_fused_covers(in_dim, out_dim, x, g))
+        return launch_dense_backward(d_x, d_w, x, g, w, relu_input ? 1 : 0, num_nodes, in_dim, out_dim, workspace, s);
+    if (int rc = launch_dense_weight(d_w, x, in_dim, g, out_dim, relu_input ? 1 : 0, num_nodes, in_dim, out_dim,
+                                     workspace, s))
+        return rc;
+    if (num_nodes == 0) return kOk;
+    return launch_dense_rows(d_x, in_dim, in_dim, g, out_dim, w, 1, out_dim, nullptr, relu_input ? x : nullptr, in_dim,
+                             0, num_nodes, out_dim, in_dim, s, 0u);
 }
 
 }  // extern "C"

@@ -239,6 +239,17 @@ std::vector<Tensor> dense_backward(const Tensor& G, const Tensor& X, const Tenso
     const int in_dim = static_cast<int>(X.size(1)), out_dim = static_cast<int>(W.size(1));
     const int sup = dense_support(X, W);
     Tensor d_weight, d_input;
+    if (need_dx && (sup & 6) == 6) {
+        // both gradients from one call: narrow layers read X and G once for the two products
+        d_weight = torch::empty({in_dim, out_dim}, X.options());
+        d_input = torch::empty({n, in_dim}, X.options());
+        const size_t nbytes = eppgcn_update_workspace_bytes(n, in_dim, out_dim);
+        auto ws = torch::empty({static_cast<int64_t>((nbytes + 3) / 4) + 1}, X.options());
+        check(eppgcn_update_backward(d_input.data_ptr<float>(), d_weight.data_ptr<float>(), f32(X), f32(G), f32(W),
+                                     relu_input ? 1 : 0, n, in_dim, out_dim, ws.data_ptr<float>(), nbytes, stream_of(X)),
+              "update_backward");
+        return {d_input, d_weight};
+    }
     if (sup & 4) {
         d_weight = torch::empty({in_dim, out_dim}, X.options());
         const size_t nbytes = eppgcn_update_workspace_bytes(n, in_dim, out_dim);

@@ -399,4 +399,201 @@ int launch_dense_weight(float* dw, const float* x, int ld_x, const float* g, int
     return kOk;
 }
 
+// ---------------------------------------------------------------- input and weight gradient in one pass
+// dX[r, k] = [act'(X[r, k])] * sum_d G[r, d] * W[k, d]   and   dW[k, d] = sum_r act(X[r, k]) * G[r, d]
+// for a narrow layer (K <= 16 inputs, D <= 32 gradient columns): both products read G and X, so a wave that owns a
+// contiguous range of rows does both for every 16 rows it loads - G and X come from HBM once instead of twice.
+// The 16 rows of G and of X are contiguous in memory (64 D and 64 K bytes): the wave copies them into its own LDS
+// area with full 16-byte loads (three load instructions per step at K = 16, D = 22, where the operand layouts of
+// the two products would take twenty narrow ones) and both products read their operands from there; the next
+// step's rows are requested before the current step's products start.  Each product is accumulated exactly as
+// dense_rows_kernel / dense_weight_kernel accumulate it (same tiles, same order of additions, same block sums), so
+// the results equal those of the two separate launches bit for bit.
+struct BackwardArgs {
+    float* dx;               // [N, K]
+    float* partial;          // [gridDim.x][K * D] block sums of dW
+    const float* x;          // [N, K] layer input, 16-byte aligned
+    const float* g;          // [N, D] gradient of the layer's product, 16-byte aligned
+    const float* w;          // [K, D]
+    long long n, rows_per_wave;
+    int K, D;
+    int relu_in;             // the layer applied max(x, 0) to its input
+    int vec_store;           // rows of dx are 16-byte aligned
+};
+
+constexpr int kBackMaxK = 16, kBackMaxD = 32;
+
+template <int VW, int DT>
+__global__ __launch_bounds__(kUpdateThreads) void dense_backward_kernel(BackwardArgs a)
+{
+    constexpr int CH = 4 * DT / VW;                          // steps of 4 * VW gradient columns that cover 16 * DT
+    constexpr int kGVecs = 16 * 16 * DT / 4 / kWave;         // 16-byte vectors per lane that cover 16 rows of G
+    __shared__ __align__(16) float w_lds[CH * kWave * VW];   // operand of the dX product, element (d, k) = w[k, d]
+    __shared__ __align__(16) float g_lds[kUpdateWaves][16 * 16 * DT];
+    __shared__ __align__(16) float x_lds[kUpdateWaves][16 * kBackMaxK];
+    __shared__ float red[kUpdateWaves][DT * 4 * kWave];
+    for (int idx = threadIdx.x; idx < CH * kWave * VW; idx += kUpdateThreads) {
+        const int v = idx % VW;
+        const int l = (idx / VW) % kWave;
+        const int t = idx / (VW * kWave);
+        const int d = (4 * t + l / 16) * VW + v;
+        const int k = l % 16;
+        w_lds[idx] = (d < a.D && k < a.K) ? a.w[k * a.D + d] : 0.f;
+    }
+    __syncthreads();
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x / kWave;
+    const int i = lane % 16, j = lane / 16;
+    float* __restrict__ gt = g_lds[wave];
+    float* __restrict__ xt = x_lds[wave];
+    floatx4 accw[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) accw[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const long long wave_id = static_cast<long long>(blockIdx.x) * kUpdateWaves + wave;
+    const long long r_begin = wave_id * a.rows_per_wave;
+    long long r_end = r_begin + a.rows_per_wave;
+    if (r_end > a.n) r_end = a.n;
+
+    // 16 rows from row r0 on (fewer at the end of the matrix; what lies past the wave's own range is loaded but
+    // never used): G as kGVecs vectors per lane, X as one
+    floatx4 gv[kGVecs], xv;
+    auto request = [&](long long r0) {
+        const long long rows = a.n - r0 < 16 ? a.n - r0 : 16;
+        const float* __restrict__ gsrc = a.g + r0 * a.D;
+        const float* __restrict__ xsrc = a.x + r0 * a.K;
+        const int gcount = static_cast<int>(rows) * a.D, xcount = static_cast<int>(rows) * a.K;
+#pragma unroll
+        for (int q = 0; q < kGVecs; ++q) {
+            const int off = (q * kWave + lane) * 4;
+            if (off + 4 <= gcount) gv[q] = *reinterpret_cast<const floatx4*>(gsrc + off);
+            else
+#pragma unroll
+                for (int c = 0; c < 4; ++c) gv[q][c] = off + c < gcount ? gsrc[off + c] : 0.f;
+        }
+        const int off = lane * 4;
+        if (off + 4 <= xcount) xv = *reinterpret_cast<const floatx4*>(xsrc + off);
+        else
+#pragma unroll
+            for (int c = 0; c < 4; ++c) xv[c] = off + c < xcount ? xsrc[off + c] : 0.f;
+    };
+    if (r_begin < r_end) request(r_begin);
+
+    for (long long r0 = r_begin; r0 < r_end; r0 += 16) {
+        // the wave's LDS area is its own: its LDS operations execute in order, so the stores below come after the
+        // previous step's reads without a barrier
+#pragma unroll
+        for (int q = 0; q < kGVecs; ++q) *reinterpret_cast<floatx4*>(gt + (q * kWave + lane) * 4) = gv[q];
+        *reinterpret_cast<floatx4*>(xt + lane * 4) = xv;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (r0 + 16 < r_end) request(r0 + 16);               // under way during this step's products
+
+        // ---- dX for rows r0 .. r0 + 15: lane (i, j) takes VW consecutive gradient columns of row r0 + i per step
+        const long long r = r0 + i;
+        const bool row_ok = r < r_end;
+        floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < CH; ++t) {
+            const float* wp = w_lds + (t * kWave + lane) * VW;
+#pragma unroll
+            for (int v = 0; v < VW; ++v) {
+                const int d = (4 * t + j) * VW + v;
+                acc = mfma16(wp[v], d < a.D ? gt[i * a.D + d] : 0.f, acc);
+            }
+        }
+        const int m0 = 4 * j;
+        if (row_ok && m0 < a.K) {
+            float y[4] = {acc[0], acc[1], acc[2], acc[3]};
+            if (a.relu_in) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (m0 + v < a.K && !(xt[i * a.K + m0 + v] > 0.f)) y[v] = 0.f;
+            }
+            float* __restrict__ orow = a.dx + r * a.K;
+            if (a.vec_store && m0 + 4 <= a.K) {
+                *reinterpret_cast<float4*>(orow + m0) = make_float4(y[0], y[1], y[2], y[3]);
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (m0 + v < a.K) orow[m0 + v] = y[v];
+            }
+        }
+        // ---- dW: lane (i, j) supplies column i of X and columns i, 16 + i of G for rows r0 + 4 s + j
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int lr = 4 * s + j;
+            const bool ok = r0 + lr < r_end;
+            const float t = (ok && i < a.K) ? xt[lr * a.K + i] : 0.f;
+            const float av = a.relu_in ? fmaxf(t, 0.f) : t;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int d = dt * 16 + i;
+                accw[dt] = mfma16(av, (ok && d < a.D) ? gt[lr * a.D + d] : 0.f, accw[dt]);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][(dt * 4 + v) * kWave + lane] = accw[dt][v];
+    __syncthreads();
+    float* __restrict__ mine = a.partial + static_cast<size_t>(blockIdx.x) * a.K * a.D;
+    for (int e = threadIdx.x; e < DT * 4 * kWave; e += kUpdateThreads) {
+        float sum = red[0][e];
+#pragma unroll
+        for (int w = 1; w < kUpdateWaves; ++w) sum += red[w][e];
+        const int l = e % kWave;
+        const int v = (e / kWave) % 4;
+        const int dt = e / (4 * kWave);
+        const int k = 4 * (l / 16) + v;
+        const int d = dt * 16 + l % 16;
+        if (k < a.K && d < a.D) mine[static_cast<size_t>(k) * a.D + d] = sum;
+    }
+}
+
+// Shapes the one-pass kernel covers.
+bool dense_backward_fused_covers(int K, int D, const float* x, const float* g)
+{
+    return K >= 1 && K <= kBackMaxK && D >= 1 && D <= kBackMaxD &&
+           (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(g)) % 16 == 0;
+}
+
+// dx[N, K] and dw[K, D] of a layer out = act(X) * W from the gradient G[N, D] of the product, in one pass over X
+// and G (dense_backward_fused_covers(K, D) holds; `workspace` as for launch_dense_weight).
+int launch_dense_backward(float* dx, float* dw, const float* x, const float* g, const float* w, int relu_in,
+                          long long n, int K, int D, void* workspace, hipStream_t stream)
+{
+    if (n == 0) return launch_zero_words(dw, static_cast<size_t>(K) * D, stream);
+    const int blocks = weight_blocks(n);
+    const long long waves = static_cast<long long>(blocks) * kUpdateWaves;
+    BackwardArgs a;
+    a.dx = dx;
+    a.partial = static_cast<float*>(workspace);
+    a.x = x;
+    a.g = g;
+    a.w = w;
+    a.n = n;
+    a.rows_per_wave = ((n + waves - 1) / waves + 15) / 16 * 16;
+    a.K = K;
+    a.D = D;
+    a.relu_in = relu_in;
+    a.vec_store = (K % 4 == 0 && reinterpret_cast<uintptr_t>(dx) % 16 == 0) ? 1 : 0;
+    const int vw = D % 4 == 0 ? 4 : D % 2 == 0 ? 2 : 1;        // the order of additions of dense_rows_kernel for aligned g
+    const int dt = D <= 16 ? 1 : 2;
+#define EPPGCN_B(VW_, DT_) hipLaunchKernelGGL((dense_backward_kernel<VW_, DT_>), dim3(blocks), dim3(kUpdateThreads), 0, stream, a)
+    if (vw == 4) { if (dt == 1) EPPGCN_B(4, 1); else EPPGCN_B(4, 2); }
+    else if (vw == 2) { if (dt == 1) EPPGCN_B(2, 1); else EPPGCN_B(2, 2); }
+    else { if (dt == 1) EPPGCN_B(1, 1); else EPPGCN_B(1, 2); }
+#undef EPPGCN_B
+    EPPGCN_HIP(hipGetLastError());
+    const int count = K * D;
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3((count + 63) / 64), dim3(256), 0, stream, dw, a.partial, blocks, count);
+    EPPGCN_HIP(hipGetLastError());
+    return kOk;
+}
+
 }  // namespace eppgcn

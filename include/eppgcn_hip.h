@@ -370,6 +370,17 @@ size_t eppgcn_update_workspace_bytes(int64_t num_nodes, int in_dim, int out_dim)
 int eppgcn_update_backward_weight(float* d_w, const float* x, const float* g, int relu_input, int64_t num_nodes,
                                   int in_dim, int out_dim, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Both gradients of a layer out = act(x) * w in one call: d_x as eppgcn_update_backward_input gives it with
+ * relu_ref = x when relu_input != 0 (NULL otherwise), d_w as eppgcn_update_backward_weight gives it - the same
+ * bits.  For narrow layers (in_dim <= 16, out_dim <= 32) one kernel forms both products from one pass over x
+ * and g (they come from memory once instead of twice); other shapes run the two kernels one after the other
+ * and are subject to their limits (out_dim <= 64).  workspace as for eppgcn_update_backward_weight.
+ * Replaces the pair `d_input = torch::mm(d_input_prime, W.transpose(0,1))`, `d_weight =
+ * torch::mm(X.transpose(0,1), d_input_prime)`, EPPGCN_kernel.cu:461-462,614-615. */
+int eppgcn_update_backward(float* d_x, float* d_w, const float* x, const float* g, const float* w, int relu_input,
+                           int64_t num_nodes, int in_dim, int out_dim, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
 /* ---------------------------------------------------------------------------
  * Timers (print_time / clear_time, EPPGCN_kernel.cu:89-116; EPPGCN.cpp:394-395).
  * Timing is off by default so that calls stay asynchronous; when enabled every

@@ -85,6 +85,51 @@ def test_update_backward_weight_matches_checker(api, n, k, m, relu):
     assert_close(a.cpu().numpy(), co.update_backward_weight(x, g, relu_input=relu), bound, "weight gradient")
 
 
+# rows x layer inputs x gradient columns: the benchmark's hidden layer (16 -> 22), a 16 -> 16 hidden layer of the
+# deeper models, tile edges and odd widths (every load width of the one-pass kernel), row counts around the 16-row
+# steps and the waves' row ranges, and shapes outside the one-pass kernel (in_dim > 16, out_dim > 32)
+@pytest.mark.parametrize("n,k,m", [(1, 1, 1), (5, 3, 2), (16, 16, 16), (17, 16, 22), (1000, 16, 22), (4097, 16, 16),
+                                   (300, 13, 17), (123, 16, 32), (999, 8, 7), (65536, 16, 22), (300007, 16, 22),
+                                   (1000, 96, 16), (500, 16, 40), (200, 33, 33)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_update_backward_pair_equals_the_two_products(api, n, k, m, relu):
+    """eppgcn_update_backward gives both gradients of a layer; for narrow layers from one pass over x and g.  Each
+    product is formed exactly as the separate calls form it, so the results are the same bits, and they are held
+    against the checker like those."""
+    x, w, g, _ = data(n, k, m, 6)
+    dx, dw = api.update_backward(dev(x), dev(w), dev(g), relu_input=relu)
+    assert torch.equal(dx, api.update_backward_input(dev(g), dev(w), relu_ref=dev(x) if relu else None))
+    assert torch.equal(dw, api.update_backward_weight(dev(x), dev(g), relu_input=relu))
+    again = api.update_backward(dev(x), dev(w), dev(g), relu_input=relu)
+    assert torch.equal(again[0], dx) and torch.equal(again[1], dw), "bitwise reproducible"
+    xa = np.maximum(x, 0) if relu else x
+    assert_close(dw.cpu().numpy(), co.update_backward_weight(x, g, relu_input=relu),
+                 np.abs(xa).astype(np.float64).T @ np.abs(g).astype(np.float64), "weight gradient")
+    assert_close(dx.cpu().numpy(), co.update_backward_input(g, w, relu_ref=x if relu else None),
+                 np.abs(g).astype(np.float64) @ np.abs(w).astype(np.float64).T, "input gradient")
+    if relu:
+        assert not dx.cpu().numpy()[x <= 0].any()
+
+
+def test_update_backward_pair_on_unaligned_views(api):
+    """Gradient and input that start 4 or 8 bytes into an allocation: the one-pass kernel's narrower loads and
+    scalar stores."""
+    n, k, m = 777, 16, 22
+    x, w, g, _ = data(n, k, m, 7)
+    for shift in (1, 2):
+        gflat = torch.empty(n * m + shift, dtype=torch.float32, device="cuda")
+        gv = gflat[shift:].view(n, m)
+        gv.copy_(dev(g))
+        xflat = torch.empty(n * k + shift, dtype=torch.float32, device="cuda")
+        xv = xflat[shift:].view(n, k)
+        xv.copy_(dev(x))
+        dx, dw = api.update_backward(xv, dev(w), gv, relu_input=True)
+        assert torch.equal(dx, api.update_backward_input(gv, dev(w), relu_ref=xv))     # same views: same load widths
+        assert torch.equal(dw, api.update_backward_weight(xv, gv, relu_input=True))
+        bound = np.abs(g).astype(np.float64) @ np.abs(w).astype(np.float64).T
+        assert_close(dx.cpu().numpy(), co.update_backward_input(g, w, relu_ref=x), bound, f"input gradient, shift {shift}")
+
+
 def test_update_handles_unaligned_views(api):
     """Operands that start 4 bytes into an allocation take the narrower load paths."""
     n, k, m = 777, 22, 16
