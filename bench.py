@@ -128,6 +128,9 @@ def pipeline_figures(g, wl, kernels, x16, x22, out16, out22, args):
         ("g1_w1t_relu_masked", lambda: capi.update_backward_input(x22, w1, relu_ref=x16), n * (22 + 16 + 16) * f32),
         ("x96t_g0_weight_grad", lambda: capi.update_backward_weight(x96, x16), n * (96 + 16) * f32),
         ("relu_y1t_g1_weight_grad", lambda: capi.update_backward_weight(x16, x22, relu_input=True), n * (16 + 22) * f32),
+        # the two products above in one pass over G1 and Y1 (what the extension module's backward calls)
+        ("hidden_layer_backward_pair", lambda: capi.update_backward(x16, w1, x22, relu_input=True),
+         n * (22 + 16 + 16) * f32),
     ]
     fig["dense_update"] = {}
     for name, fn, nbytes in dense:
