@@ -5,8 +5,8 @@
 //
 // All three run on the fp32 matrix cores with v_mfma_f32_16x16x4_f32 (one wave computes a
 // 16x16 tile of C += A[16x4] * B[4x16]; lane l supplies A[l%16][l/16] and B[l/16][l%16] and
-// holds C[4*(l/16) + v][l%16] in accumulator register v).  The tall operand is read straight
-// from global memory in the operand layout, so no staging through LDS is needed:
+// holds C[4*(l/16) + v][l%16] in accumulator register v).  The rows and weight kernels read the tall
+// operand straight from global memory in the operand layout, without staging through LDS:
 //
 //   rows kernel    out[r, m] = f(r, m) * sum_k act(X[r, k]) * Wop(k, m)      (X*W and G*W^T)
 //                  tile: 16 output columns (MFMA rows) x 16 matrix rows (MFMA columns); a lane
@@ -18,6 +18,9 @@
 //                  tile: 16 k x 16 d, reduction over 4 rows per instruction; every wave owns a
 //                  contiguous range of rows, block partial sums go to a workspace and a second
 //                  kernel adds them in a fixed order (deterministic, no float atomics).
+//   backward kernel  both gradients of a narrow layer (<= 16 inputs, <= 32 gradient columns) in one pass:
+//                  the 16 rows of a step are copied to LDS with full 16-byte loads and both products take
+//                  their operands from there, accumulated exactly as the two kernels above do it.
 #include "common.hpp"
 
 namespace eppgcn {
