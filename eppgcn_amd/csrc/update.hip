@@ -78,6 +78,8 @@ struct RowsArgs {
     int K, M;
     int relu_in;             // apply max(x, 0) to X on load
     int vec_store;           // 0: scalar stores; 1: rows of out are 16-byte aligned; 2: the same, non-temporal
+    int tile_store;          // the 16 rows of a tile are 16 * out_cols contiguous floats (ld_out == out_cols == 32,
+                             // 16-byte aligned): they go through LDS and out as two 1 KB stores per wave
     unsigned swz_mask;       // row r of out lives at swizzled_row(r, swz_mask): 0 = vertex order (common.hpp)
 };
 
@@ -137,6 +139,49 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_rows_kernel(RowsArgs a)
             }
         }
 
+        if constexpr (MT == 2) {
+            // Rows of 32 floats: a lane holds 4 columns of one row per 16-column tile, so a store instruction would
+            // write one half of each of 16 lines.  The tile goes through the wave's LDS area instead and leaves as
+            // 2 KB of consecutive 16-byte stores.  In the table's row order the 16 rows of a tile stay one aligned
+            // block of 16 rows, permuted by the low bits of the XOR term (the same for all rows of the tile).
+            if (a.tile_store) {
+                __shared__ __align__(16) float o_lds[kUpdateWaves][16 * 32];
+                float* __restrict__ ot = o_lds[wave];
+                const long long r0 = tile * kTileRows;
+                const unsigned x = (static_cast<unsigned>(r0) >> kRowSwizzleShift) & a.swz_mask;
+                const float s = (row_ok && a.scale) ? a.scale[r] : 1.f;
+                const int p = i ^ static_cast<int>(x & 15u);              // place of row r0 + i in the block
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt) {
+                    const int m0 = mt * 16 + 4 * j;
+                    float y[4] = {acc[mt][0] * s, acc[mt][1] * s, acc[mt][2] * s, acc[mt][3] * s};
+                    if (a.relu_ref && row_ok) {
+                        const float* __restrict__ ref = a.relu_ref + r * a.ld_ref;
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            if (m0 + v < a.M && !(ref[m0 + v] > 0.f)) y[v] = 0.f;
+                    }
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (m0 + v >= a.M) y[v] = 0.f;
+                    *reinterpret_cast<float4*>(ot + p * 32 + m0) = make_float4(y[0], y[1], y[2], y[3]);
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                const long long b0 = static_cast<long long>((static_cast<unsigned>(r0) ^ (x & ~15u)));   // first row of the block
+                float* __restrict__ obase = a.out + b0 * 32;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int q = h * kWave + lane;                        // 16-byte vector of the 2 KB block
+                    const int prow = q >> 3;                               // its row inside the block
+                    if (r0 + (prow ^ static_cast<int>(x & 15u)) < a.n)
+                        *reinterpret_cast<float4*>(obase + q * 4) = *reinterpret_cast<const float4*>(ot + q * 4);
+                }
+                __builtin_amdgcn_wave_barrier();                           // the area is rewritten by the next tile
+                continue;
+            }
+        }
         if (!row_ok) continue;
         const float s = a.scale ? a.scale[r] : 1.f;
         float* __restrict__ orow = a.out + static_cast<long long>(swizzled_row(static_cast<unsigned>(r), a.swz_mask)) * a.ld_out;
@@ -238,6 +283,7 @@ int launch_dense_rows(float* out, int ld_out, int out_cols, const float* x, int 
         // measured at 4.2 M rows: a [N, 96] result 0.63 -> 0.47 ms with non-temporal stores, [N, 16] and
         // [N, 32] results unchanged or slower
         if (a.vec_store && out_cols >= 64) a.vec_store = 2;
+        a.tile_store = (a.vec_store && ld_out == 32 && cols == 32 && c0 == 0 && n < (1ll << 32)) ? 1 : 0;
         const size_t lds = lds_per_tile * mt;
         hipError_t e;
         if (vw == 4) e = launch_rows_mt<4>(a, mt, cu, static_cast<unsigned>(blocks), lds, stream);
