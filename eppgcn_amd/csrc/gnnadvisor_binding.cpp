@@ -188,17 +188,13 @@ const PathChoice& path_choice(const Tensor& part_pointer, const Tensor& edge_lis
     PathChoice c{part_pointer.data_ptr(), edge_list.data_ptr(), num_parts, num_nodes,
                  static_cast<int64_t>(part_pointer._version()), static_cast<int64_t>(edge_list._version()),
                  g_plan_policy > 0 || 2 * valid_len >= edge_list.numel(), part_pointer, edge_list, Tensor()};
-    // a path that keeps half of the edges or more reads most rows: its bitmap would not be used, and marking it
-    // (one random bitmap access per kept edge) is the slowest step of the preparation
-    if (2 * valid_len < edge_list.numel()) {
-        auto bitmap = torch::empty({(static_cast<int64_t>(num_nodes) + 31) / 32 + 1}, edge_list.options());
-        int64_t distinct = 0;
-        check(eppgcn_mark_gathered_rows(i32(edge_list), valid_len, num_nodes,
-                                        reinterpret_cast<uint32_t*>(bitmap.data_ptr<int32_t>()),
-                                        bitmap.data_ptr<int32_t>() + bitmap.numel() - 1, &distinct, stream_of(edge_list)),
-              "mark_gathered_rows");
-        if (2 * distinct < num_nodes) c.gathered = bitmap;
-    }
+    auto bitmap = torch::empty({(static_cast<int64_t>(num_nodes) + 31) / 32 + 1}, edge_list.options());
+    int64_t distinct = 0;
+    check(eppgcn_mark_gathered_rows(i32(edge_list), valid_len, num_nodes,
+                                    reinterpret_cast<uint32_t*>(bitmap.data_ptr<int32_t>()),
+                                    bitmap.data_ptr<int32_t>() + bitmap.numel() - 1, &distinct, stream_of(edge_list)),
+          "mark_gathered_rows");
+    if (2 * distinct < num_nodes) c.gathered = bitmap;
     g_path_choices.push_front(std::move(c));
     if (g_path_choices.size() > 8) g_path_choices.pop_back();
     return g_path_choices.front();

@@ -113,16 +113,10 @@ def prepare(graph: graphs.Graph, num_layers: int = 2, train_ratio: float = 0.1, 
         path_plan = (capi.build_plan(part_pointer, edge_list, num_parts, valid_len, n, width, ids=ids,
                                      block_shift=0 if 2 * valid_len >= e else 31)
                      if plan and num_parts > 0 else None)
-        # the pre-scaling pass of the gradient only has to cover the rows the path reads.  A path that keeps half of
-        # the edges or more reads most rows: its bitmap would not be used, and marking it is the slowest step of the
-        # preparation (one random bitmap access per kept edge), so it is not made
-        bitmap = None
-        if 2 * valid_len < e:
-            bitmap, distinct = capi.mark_gathered_rows(edge_list, valid_len, n)
-            if 2 * distinct >= n:
-                bitmap = None
+        # the pre-scaling pass of the gradient only has to cover the rows the path reads
+        bitmap, distinct = capi.mark_gathered_rows(edge_list, valid_len, n)
         paths.append(BackwardPath(k + 1, ids, edge_list, part_pointer, node_degs[k], bps, num_parts,
-                                  valid_len, valid_node, path_plan, bitmap))
+                                  valid_len, valid_node, path_plan, bitmap if 2 * distinct < n else None))
     # one plan of the forward groups serves every width (the column block is sized for the widest)
     plans = {}
     if plan and part2node.numel() > 0:
