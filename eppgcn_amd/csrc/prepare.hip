@@ -407,7 +407,7 @@ __global__ __launch_bounds__(256) void mark_listed_rows_kernel(const int* __rest
     for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < length; i += stride) {
         const unsigned c = static_cast<unsigned>(list[i]);
         const uint32_t bit = 1u << (c & 31);
-        if ((__builtin_nontemporal_load(bitmap + (c >> 5)) & bit) == 0)
+        if ((bitmap[c >> 5] & bit) == 0)
             fresh += (atomicOr(bitmap + (c >> 5), bit) & bit) == 0;
     }
 #pragma unroll

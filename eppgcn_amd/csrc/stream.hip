@@ -281,7 +281,9 @@ __global__ __launch_bounds__(256) void stream_fixup_kernel(float* __restrict__ o
     const long long waves = static_cast<long long>(gridDim.x) * (256 / kWave);
     const char* base = reinterpret_cast<const char*>(partial) + tl * 16;
     // sixteen row loads in flight (most rows have fewer partial sums: one round trip), none of them behind a
-    // branch of its own (an index past the end is replaced by a valid one and its row by zeros)
+    // branch of its own (an index past the end is replaced by a valid one and its row by zeros).  Plain loads: the
+    // replaced indices re-read one row and the two halves of a 128-byte line are read by different instructions, both
+    // of which the caches serve (non-temporal loads here cost 20 us per launch at R-MAT 22)
     constexpr int kFixLoads = 16;
     auto add_range = [&](float (&acc)[4], int beg, int end, int step) {
         if (tl >= chunks) return;
@@ -290,7 +292,7 @@ __global__ __launch_bounds__(256) void stream_fixup_kernel(float* __restrict__ o
 #pragma unroll
             for (int u = 0; u < kFixLoads; ++u) {
                 const bool ok = k + u * step < end;
-                v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(base + static_cast<size_t>(ok ? k + u * step : k) * ld_bytes));
+                v[u] = *reinterpret_cast<const f32x4*>(base + static_cast<size_t>(ok ? k + u * step : k) * ld_bytes);
                 if (!ok) v[u] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
 #pragma unroll
