@@ -44,18 +44,24 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
-template <int OVW> __device__ __forceinline__ void stream_store(float* p, const float* v);
-template <> __device__ __forceinline__ void stream_store<4>(float* p, const float* v)
+// A piece of OVW floats of an output row.  16-byte pieces belong to rows of whole 16-byte units, for the benchmark's
+// widths whole 64-byte sectors, written once and never read here: non-temporal stores.  Narrower pieces belong to
+// rows that share their sectors with their neighbours, which other teams write at other times: plain stores let the
+// cache put a sector together before it goes to memory (width 22, 88-byte rows at R-MAT 22: forward call 1.589 ->
+// 1.566 ms, backward 0.266 -> 0.254 ms; plain stores for 64-byte rows: forward call 1.092 -> 1.137 ms).
+template <int OVW>
+__device__ __forceinline__ void stream_store(float* p, const float* v)
 {
-    const f32x4 t = {v[0], v[1], v[2], v[3]};
-    __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(p));
+    if constexpr (OVW == 4) {
+        const f32x4 t = {v[0], v[1], v[2], v[3]};
+        __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(p));
+    } else if constexpr (OVW == 2) {
+        const f32x2 t = {v[0], v[1]};
+        *reinterpret_cast<f32x2*>(p) = t;
+    } else {
+        p[0] = v[0];
+    }
 }
-template <> __device__ __forceinline__ void stream_store<2>(float* p, const float* v)
-{
-    const f32x2 t = {v[0], v[1]};
-    __builtin_nontemporal_store(t, reinterpret_cast<f32x2*>(p));
-}
-template <> __device__ __forceinline__ void stream_store<1>(float* p, const float* v) { __builtin_nontemporal_store(v[0], p); }
 
 // table rows: pitch ld_bytes (a multiple of 16), `chunks` 16-byte vectors of a row are read (chunks <= TS);
 // out rows: pitch ld_out floats, columns < width_out written in pieces of OVW floats;
