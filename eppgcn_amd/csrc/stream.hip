@@ -157,7 +157,9 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     auto flush = [&](const float (&a)[4], int target, float s) {
         if (target < 0) {
             const int at = target & 0x7fffffff;
-            if (at >= num_partials || tl >= chunks) return;       // the first never happens with a well-formed stream
+            // the whole pitch is written (lanes past the row's vectors hold zeros): a partial sum then fills its
+            // 64- or 128-byte line and goes to memory without a read-modify-write
+            if (at >= num_partials || tl * 16u >= ld_bytes) return;   // the first never happens with a well-formed stream
             float* dst = reinterpret_cast<float*>(reinterpret_cast<char*>(partial) + static_cast<size_t>(at) * ld_bytes) + tl * 4;
             const f32x4 t = {a[0], a[1], a[2], a[3]};
             __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(dst));
