@@ -65,13 +65,10 @@ template <> struct Vec<2> {
         float2 t = *reinterpret_cast<const float2*>(p);
         Vec r; r.v[0] = t.x; r.v[1] = t.y; return r;
     }
-    // output rows are written once and not read again by the kernel: non-temporal stores
-    __device__ void store(float* p) const
-    {
-        typedef float f2 __attribute__((ext_vector_type(2)));
-        const f2 t = {v[0], v[1]};
-        __builtin_nontemporal_store(t, reinterpret_cast<f2*>(p));
-    }
+    // 8-byte pieces belong to rows that share their 64-byte sectors with their neighbours (width 22: 88-byte rows),
+    // written by other teams at other times: plain stores, so that the cache puts the sectors together (rows of
+    // 16-byte pieces below are whole sectors for the usual widths, written once: non-temporal)
+    __device__ void store(float* p) const { *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]); }
 };
 template <> struct Vec<4> {
     float v[4];
