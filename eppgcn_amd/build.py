@@ -21,7 +21,8 @@ LIB_DIR = os.path.join(HERE, "lib")
 OBJ_DIR = os.path.join(HERE, "csrc", "_obj")
 HIP_LIB = os.path.join(LIB_DIR, "libeppgcn_hip.so")
 HIP_SOURCES = ["aggregate.hip", "stream.hip", "prepare.hip", "schedule.hip", "update.hip", "capi.hip"]
-HIP_HEADERS = ["common.hpp", os.path.join(ROOT, "include", "eppgcn_hip.h")]
+HIP_HEADERS = ["common.hpp", os.path.join(ROOT, "include", "eppgcn_hip.h"),
+               os.path.join(ROOT, "include", "eppgcn_hip_tuning.h")]
 ARCH = "gfx950"
 
 # packed fp32 instructions are switched off for every device compile

@@ -29,10 +29,10 @@ EXPORTS = [
     "eppgcn_compact_back_edge_static", "eppgcn_compact_back_edge_static_max_length",
     "eppgcn_auto_back_part_size", "eppgcn_scan_status", "eppgcn_plan_status", "eppgcn_set_scan_test_mode",
     "eppgcn_plan_workspace_floats", "eppgcn_set_stream_mode", "eppgcn_last_call_used_stream",
-    "eppgcn_update_forward_table", "eppgcn_feature_workspace_row",
+    "eppgcn_update_forward_table", "eppgcn_feature_workspace_row", "eppgcn_plan_release", "eppgcn_aggregation_status",
 ]
 
-ABI_VERSION = 14      # what eppgcn_abi_version() of a matching library returns
+ABI_VERSION = 15      # what eppgcn_abi_version() of a matching library returns
 
 _lib = None
 
@@ -91,6 +91,10 @@ def load():
     lib.eppgcn_scan_status.restype = i
     lib.eppgcn_plan_status.argtypes = [p, i, i64, i, C.POINTER(i64), p]
     lib.eppgcn_plan_status.restype = i
+    lib.eppgcn_plan_release.argtypes = [p]
+    lib.eppgcn_plan_release.restype = None
+    lib.eppgcn_aggregation_status.argtypes = [p]
+    lib.eppgcn_aggregation_status.restype = i
     lib.eppgcn_plan_workspace_floats.argtypes = [p, i64, i]
     lib.eppgcn_plan_workspace_floats.restype = sz
     lib.eppgcn_set_stream_mode.argtypes = [i]
@@ -333,6 +337,18 @@ class Plan:
         self.buffer, self.base_ptr, self.num_parts, self.num_slots = buffer, base_ptr, num_parts, num_slots
         self.num_nodes = num_nodes
         self.partial_rows = partial_rows      # partial sums of a call through the stream form (0: no stream form)
+
+    def release(self):
+        """Tells the library that this plan's memory is given up (it forgets the header it read there)."""
+        if self.base_ptr and _lib is not None:
+            _lib.eppgcn_plan_release(C.c_void_p(self.base_ptr))
+        self.base_ptr = 0
+
+    def __del__(self):
+        try:
+            self.release()
+        except Exception:      # interpreter shutdown
+            pass
 
     @property
     def padded_slots(self):
@@ -612,8 +628,15 @@ def auto_back_part_size(valid_node: int, valid_len: int):
 
 
 def scan_status(workspace) -> None:
-    """Raises if the last scan-based call over ``workspace`` stalled or overflowed (synchronises)."""
+    """Raises if the last scan-based call over ``workspace`` stalled or overflowed (synchronises).
+    ``None``: the static scratch of ``compact_back_edge_static`` on the current device."""
     _check(load().eppgcn_scan_status(_ptr(workspace), _stream()))
+
+
+def aggregation_status() -> None:
+    """Raises (once) if the stream or fix-up kernel of an aggregation call found a plan header in memory
+    that was not the one ``build_plan`` left there (synchronises)."""
+    _check(load().eppgcn_aggregation_status(_stream()))
 
 
 def split_back_part(node_deg, num_edges: int, part_size: int):

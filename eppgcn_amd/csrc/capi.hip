@@ -1,6 +1,6 @@
 // extern "C" entry points of libeppgcn_hip.so: argument checks, timers and the
 // host halves (count read-back, heuristics) of the aggregation path.
-#include "../../include/eppgcn_hip.h"
+#include "../../include/eppgcn_hip_tuning.h"
 
 #include <cmath>
 #include <cstdio>
@@ -43,6 +43,8 @@ int launch_mask_forward(const int*, const int*, const int*, const uint8_t*, uint
 int launch_compact_mask(const int*, int*, const int*, int*, long long, void*, hipStream_t);
 long long static_compact_max_length();
 int launch_compact_mask_static(const int*, int*, const int*, int*, long long, void**, hipStream_t);
+int static_compact_workspace(void**);
+int read_aggregation_status(hipStream_t);
 size_t mark_compact_workspace_bytes(long long);
 int launch_mark_compact(const int*, const int*, const int*, const uint8_t*, uint8_t*, int*, int*, int*, int, long long,
                         int, void*, hipStream_t);
@@ -90,7 +92,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 14; }
+int eppgcn_abi_version(void) { return 15; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -373,7 +375,12 @@ int eppgcn_auto_back_part_size(int64_t valid_node, int64_t valid_len, int* fell_
 
 int eppgcn_scan_status(const void* workspace, void* stream)
 {
-    EPPGCN_REQUIRE(workspace && aligned(workspace, 8), "workspace must be 8-byte aligned");
+    if (!workspace) {       // the static scratch of eppgcn_compact_back_edge_static on the current device
+        void* ws = nullptr;
+        if (int rc = static_compact_workspace(&ws)) return rc;
+        workspace = ws;
+    }
+    EPPGCN_REQUIRE(aligned(workspace, 8), "workspace must be 8-byte aligned");
     ScanState host;
     if (int rc = read_state(const_cast<void*>(workspace), static_cast<hipStream_t>(stream), &host)) return rc;
     if (host.overflow) {
@@ -396,6 +403,13 @@ int eppgcn_plan_status(const void* plan, int num_parts, int64_t num_slots, int n
     if (partial_rows) *partial_rows = partial;
     return rc;
 }
+
+void eppgcn_plan_release(const void* plan)
+{
+    if (plan) forget_stream_info(plan);
+}
+
+int eppgcn_aggregation_status(void* stream) { return read_aggregation_status(static_cast<hipStream_t>(stream)); }
 
 size_t eppgcn_plan_workspace_floats(const void* plan, int64_t num_nodes, int dim)
 {

@@ -21,6 +21,7 @@ enum : int {
     kErrHip = -2,
     kErrScanStalled = -3,   // a look-back wait exceeded its spin limit
     kErrCapacity = -4,      // an output buffer was too small for the result
+    kErrPlanMismatch = -5,  // the memory at a plan's address does not hold the plan the library knows there
 };
 
 void set_error(const std::string& msg);
@@ -69,6 +70,7 @@ constexpr int kStreamWave = 512;     // slots a wave of the stream kernel takes
 constexpr int kStreamChunk = 32;     // piece ends are counted per chunk of this many slots
 constexpr unsigned kStreamFlag = 0x80000000u;
 constexpr int kStreamIdMask = 0x7fffffff;
+constexpr int kPlanMagic = 0x45505047;   // "EPPG"
 struct StreamHeader {
     int valid;          // 1: the stream arrays describe the plan (0: groups were empty or a scan stalled)
     int num_events;     // pieces
@@ -77,7 +79,12 @@ struct StreamHeader {
     int empty_rows;     // rows without any slot (the output clear zeroes them)
     int error;          // a look-back scan of the build stalled
     int empty_groups;   // != 0: the plan holds empty groups (no stream form)
-    int pad[9];
+    int magic;          // kPlanMagic: the build got as far as writing the header
+    int generation;     // number of the build in this process (> 0); the host remembers it with the counts
+    int num_parts;      // the sizes the plan was built with (its layout depends on them)
+    int num_nodes;
+    int num_slots;
+    int pad[4];
 };
 static_assert(sizeof(StreamHeader) == 64, "header layout");
 struct StreamView {
@@ -180,6 +187,12 @@ struct StreamInfo {
 const StreamInfo* find_stream_info(const void* plan, StreamInfo* copy);
 void forget_stream_info(const void* plan);
 void remember_stream_info(const void* plan, const StreamInfo& info);
+// Device words (one set per GPU, inside the library) in which the stream and fix-up kernels leave a mark when
+// the plan header in memory is not the one the host remembers for that address: [0] != 0 says so, [1] which kernel
+// saw it (1 stream, 2 fix-up), [2] / [3] the build number the host expected / the one found.  The address on the
+// current device; looked up once per device (eppgcn_plan_status does it, so never under a graph capture).
+constexpr int kPlanFaultWords = 4;
+int plan_fault_address(int** words);
 
 // ---------------------------------------------------------------- kernel timers
 // Optional event timing of the kernels of one call (off by default: calls stay

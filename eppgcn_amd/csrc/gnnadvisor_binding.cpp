@@ -97,6 +97,18 @@ struct PlanEntry {
 };
 std::list<PlanEntry> g_plans;
 constexpr size_t kMaxPlans = 8;
+// An entry that leaves the cache gives its plan's memory back to torch: the library is told first, so that it
+// forgets the header it read at that address.
+void drop_oldest_plan()
+{
+    eppgcn_plan_release(g_plans.back().plan_ptr);
+    g_plans.pop_back();
+}
+void drop_all_plans()
+{
+    for (const PlanEntry& e : g_plans) eppgcn_plan_release(e.plan_ptr);
+    g_plans.clear();
+}
 int g_plan_policy = 0;   // 0: where eppgcn_plan_recommended says so, 1: always, -1: never
 
 int dim_class_of(int dim) { return dim <= 32 ? 0 : dim <= 128 ? 1 : 2; }
@@ -148,7 +160,7 @@ const void* plan_for(const Tensor& part_ptr, const Tensor& col, const Tensor& ro
     check(eppgcn_plan_status(base, static_cast<int>(num_parts), num_slots, num_nodes, nullptr, stream_of(part_ptr)),
           "build_plan");
     g_plans.push_front(std::move(e));
-    if (g_plans.size() > kMaxPlans) g_plans.pop_back();
+    if (g_plans.size() > kMaxPlans) drop_oldest_plan();
     return g_plans.front().plan_ptr;
 }
 
@@ -586,9 +598,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("print_time", &eppgcn_print_time, "print accumulated kernel times");
     m.def("clear_time", &eppgcn_clear_time, "reset accumulated kernel times");
     m.def("set_timing", [](bool on) { eppgcn_set_timing(on ? 1 : 0); }, "enable per-call kernel timing");
+    m.def("aggregation_status",
+          []() { check(eppgcn_aggregation_status(static_cast<void*>(c10::hip::getCurrentHIPStream().stream())), "aggregation_status"); },
+          "synchronise and raise if a planned aggregation call found its plan's memory replaced (see eppgcn_hip.h)");
     m.def("get_time_ms", &eppgcn_get_time_ms, "accumulated kernel time in ms");
-    m.def("clear_plans", []() { g_plans.clear(); g_path_choices.clear(); }, "drop the cached execution plans");
-    m.def("set_plan_policy", [](int policy) { g_plan_policy = policy; g_plans.clear(); g_path_choices.clear(); },
+    m.def("clear_plans", []() { drop_all_plans(); g_path_choices.clear(); }, "drop the cached execution plans");
+    m.def("set_plan_policy", [](int policy) { g_plan_policy = policy; drop_all_plans(); g_path_choices.clear(); },
           "execution plans: 0 = where the feature table outgrows the caches (default), 1 = always, -1 = never");
     m.def("cached_plans", []() { return static_cast<int>(g_plans.size()); }, "number of execution plans held");
 

@@ -18,11 +18,12 @@
 #include "common.hpp"
 
 // Scan scratch of the allocation-free compaction entry point: one ScanState and one 64-bit tile
-// descriptor per 4096-slot tile, for inputs of up to 2^30 slots (2 MiB + 32 bytes per GPU, held
-// until the process ends).  The name is a host-side stand-in; host code only ever uses the device
-// address hipGetSymbolAddress returns for it (static_compact_scratch below).
+// descriptor per tile of compact_mask_kernel (16384 slots), for inputs of up to 2^30 slots (512 KiB + 32
+// bytes per GPU, held until the process ends).  The name is a host-side stand-in; host code only ever uses
+// the device address hipGetSymbolAddress returns for it (static_compact_scratch below).
 constexpr long long kStaticCompactMaxLength = 1ll << 30;
-constexpr size_t kStaticCompactScratchBytes = 32 + 8 * static_cast<size_t>(kStaticCompactMaxLength / 4096);
+constexpr long long kStaticCompactTile = 16384;
+constexpr size_t kStaticCompactScratchBytes = 32 + 8 * static_cast<size_t>(kStaticCompactMaxLength / kStaticCompactTile);
 static __device__ __align__(256) unsigned char scratch[kStaticCompactScratchBytes];
 
 namespace eppgcn {
@@ -771,6 +772,9 @@ static int static_compact_scratch(void** out)
     return kOk;
 }
 
+// The scratch address for the status call (and the look-up of the address outside a graph capture).
+int static_compact_workspace(void** out) { return static_compact_scratch(out); }
+
 // compact_mask_kernel over the static scratch; *workspace_out receives the scratch address (its
 // ScanState holds the kept length once the stream has run).  The scan state and the descriptors of
 // the tiles this call uses are cleared by init_scan's fill kernel on every call: the array keeps
@@ -778,9 +782,9 @@ static int static_compact_scratch(void** out)
 int launch_compact_mask_static(const int* in_id, int* out_id, const int* in_edge, int* out_edge, long long length,
                                void** workspace_out, hipStream_t stream)
 {
-    static_assert(kStaticCompactMaxLength % kCompactTile == 0 &&
-                      kStaticCompactScratchBytes == sizeof(ScanState) + 8 * (kStaticCompactMaxLength / kCompactTile),
-                  "the static scratch holds the scan state and one descriptor per tile");
+    static_assert(kStaticCompactTile == kCompactMaskTile && kStaticCompactMaxLength % kCompactMaskTile == 0 &&
+                      kStaticCompactScratchBytes == sizeof(ScanState) + 8 * (kStaticCompactMaxLength / kCompactMaskTile),
+                  "the static scratch holds the scan state and one descriptor per tile of compact_mask_kernel");
     void* ws = nullptr;
     if (int rc = static_compact_scratch(&ws)) return rc;
     *workspace_out = ws;

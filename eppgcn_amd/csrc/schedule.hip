@@ -33,6 +33,7 @@
 // Everything is written here: the keys, a stable least-significant-digit radix sort of the
 // (key, group index) pairs (8 bits per pass: tile histograms, one look-back scan, stable scatter with
 // ballot-based ranks), the look-back scan of the group sizes, the flags and the column copy.
+#include <atomic>
 #include <cstring>
 
 #include "common.hpp"
@@ -266,11 +267,16 @@ __global__ __launch_bounds__(256) void plan_fill_kernel(const int* __restrict__ 
 }
 
 // ---------------------------------------------------------------- stream form
-__global__ void stream_init_kernel(StreamHeader* h, int num_nodes)
+__global__ void stream_init_kernel(StreamHeader* h, int num_parts, int num_slots, int num_nodes, int generation)
 {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         StreamHeader z = {};
         z.empty_rows = num_nodes;
+        z.magic = kPlanMagic;
+        z.generation = generation;
+        z.num_parts = num_parts;
+        z.num_nodes = num_nodes;
+        z.num_slots = num_slots;
         *h = z;
     }
 }
@@ -569,7 +575,8 @@ static int stable_sort_by_key(unsigned* keys_a, unsigned* keys_b, int* vals_tmp,
 }
 
 static int launch_build_stream(PlanView v, StreamView sv, int num_parts, long long num_slots, int num_nodes, char* base,
-                               size_t slab, ScanState* st, ScanState* sort_st, void* temp, hipStream_t stream)
+                               size_t slab, ScanState* st, ScanState* sort_st, void* temp, int generation,
+                               hipStream_t stream)
 {
     const int padded = static_cast<int>(stream_padded_slots(num_slots));
     const int num_waves = padded / kStreamWave;
@@ -581,7 +588,8 @@ static int launch_build_stream(PlanView v, StreamView sv, int num_parts, long lo
     unsigned* keys = reinterpret_cast<unsigned*>(base + 4 * slab);
     int* order = reinterpret_cast<int*>(base + 5 * slab);
     const auto blocks = [](long long n) { return dim3(static_cast<unsigned>((n + 255) / 256 > 0 ? (n + 255) / 256 : 1)); };
-    hipLaunchKernelGGL(stream_init_kernel, dim3(1), dim3(64), 0, stream, sv.header, num_nodes);
+    hipLaunchKernelGGL(stream_init_kernel, dim3(1), dim3(64), 0, stream, sv.header, num_parts,
+                       static_cast<int>(num_slots), num_nodes, generation);
     EPPGCN_HIP(hipGetLastError());
     if (int rc = launch_zero_words(sv.touched, plan_single_words(num_nodes), stream)) return rc;
     hipLaunchKernelGGL(stream_ends_kernel, blocks(num_parts), dim3(256), 0, stream, v, num_parts, is_end, sv.header);
@@ -620,6 +628,17 @@ static int launch_build_stream(PlanView v, StreamView sv, int num_parts, long lo
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }
+
+// Every build gets a number of its own (> 0): it is written into the plan's header and remembered by the host with the
+// header's counts, so that a kernel can tell the plan it was launched for from other bytes at the same address.
+static std::atomic<int> g_plan_generation{0};
+static int next_plan_generation()
+{
+    int g = g_plan_generation.fetch_add(1) + 1;
+    if (g <= 0) { g_plan_generation.store(1); g = 1; }      // wrapped after 2^31 builds
+    return g;
+}
+static int last_plan_generation() { return g_plan_generation.load(); }
 
 int launch_build_plan(const int* part_ptr, const int* col, const int* part2node, const int* ids, int num_parts,
                       long long num_slots, int num_nodes, int shift, int dim, void* plan, size_t plan_size,
@@ -670,7 +689,7 @@ int launch_build_plan(const int* part_ptr, const int* col, const int* part2node,
                        part_ptr, col, part2node, ids, order, num_parts, v);
     EPPGCN_HIP(hipGetLastError());
     return launch_build_stream(v, stream_view(plan, num_parts, num_slots, num_nodes), num_parts, num_slots, num_nodes, base,
-                               slab, st, sort_st, temp, stream);
+                               slab, st, sort_st, temp, next_plan_generation(), stream);
 }
 
 // ---------------------------------------------------------------- what the host knows about built plans
@@ -703,6 +722,25 @@ void remember_stream_info(const void* plan, const StreamInfo& info)
     g_infos[plan] = info;
 }
 
+// Synchronises the stream and reports (once) a header mismatch that a stream or fix-up kernel has seen on the current
+// device since the last report.
+int read_aggregation_status(hipStream_t stream)
+{
+    int* words = nullptr;
+    if (int rc = plan_fault_address(&words)) return rc;
+    int host[kPlanFaultWords] = {0, 0, 0, 0};
+    EPPGCN_HIP(hipMemcpyAsync(host, words, sizeof(host), hipMemcpyDeviceToHost, stream));
+    EPPGCN_HIP(hipStreamSynchronize(stream));
+    if (!host[0]) return kOk;
+    if (int rc = launch_zero_words(words, kPlanFaultWords, stream)) return rc;
+    set_error(std::string("an aggregation call was given a plan whose header in memory is not the one the library read at "
+                          "that address (seen by the ") + (host[1] == 2 ? "fix-up" : "stream") + " kernel: build " +
+              std::to_string(host[2]) + " expected, " + std::to_string(host[3]) +
+              " found); that call wrote no output.  The plan's memory was overwritten or replaced: rebuild the plan, or "
+              "call eppgcn_plan_release when a plan's memory is given up");
+    return kErrPlanMismatch;
+}
+
 // Synchronises the stream, reads the plan's header and records it; the return code tells whether a look-back scan
 // of the build stalled.
 int read_plan_status(const void* plan, long long num_parts, long long num_slots, long long num_nodes,
@@ -715,6 +753,24 @@ int read_plan_status(const void* plan, long long num_parts, long long num_slots,
     const StreamView sv = stream_view(const_cast<void*>(plan), num_parts, num_slots, num_nodes);
     EPPGCN_HIP(hipMemcpyAsync(&info.header, sv.header, sizeof(StreamHeader), hipMemcpyDeviceToHost, stream));
     EPPGCN_HIP(hipStreamSynchronize(stream));
+    {   // the address of the mismatch mark on this device is looked up here, outside any graph capture
+        int* words = nullptr;
+        if (int rc = plan_fault_address(&words)) return rc;
+    }
+    // only a header that a build of this process wrote for these sizes is taken on: its counts size the launches
+    const StreamHeader& h = info.header;
+    const long long waves = stream_padded_slots(num_slots) / kStreamWave;
+    const bool plausible = h.magic == kPlanMagic && h.generation > 0 && h.generation <= last_plan_generation() &&
+                           h.num_parts == num_parts && h.num_nodes == num_nodes && h.num_slots == num_slots &&
+                           h.num_events >= 0 && h.num_events <= num_parts && h.num_partials >= 0 &&
+                           h.num_partials <= num_parts + waves && h.num_fix >= 0 && h.num_fix <= num_nodes &&
+                           h.num_fix <= h.num_partials && h.empty_rows >= 0 && h.empty_rows <= num_nodes;
+    if (!plausible) {
+        forget_stream_info(plan);
+        set_error("plan_status: the memory at `plan` does not hold a plan built with these sizes (no build has "
+                  "finished there, or its bytes were overwritten); rebuild it with eppgcn_build_plan");
+        return kErrPlanMismatch;
+    }
     if (info.header.error) {
         forget_stream_info(plan);
         set_error("look-back scan stalled: a tile waited past its spin limit; the plan is invalid");

@@ -72,12 +72,29 @@ template <int U> struct StreamBatch {
     unsigned c[U];
 };
 
+// Is the header in memory the one the host remembers for this plan address?  (num_events < 0: not compared)
+__device__ __forceinline__ bool header_mismatch(const StreamHeader* __restrict__ h, int generation, int num_events,
+                                                int num_partials)
+{
+    return h->valid != 1 || h->magic != kPlanMagic || h->generation != generation || h->num_partials != num_partials ||
+           (num_events >= 0 && h->num_events != num_events);
+}
+// One lane leaves the mark in the library's own device words (ordinary vector stores; the plan's memory is not
+// written: whatever replaced the plan there belongs to somebody else).
+__device__ __forceinline__ void report_mismatch(int* __restrict__ fault, int which, int expected, int found)
+{
+    __hip_atomic_store(fault + 1, which, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(fault + 2, expected, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(fault + 3, found, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 template <int OVW, int TS, int U>
 __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     float* __restrict__ out, float* __restrict__ partial, const float* __restrict__ table,
     const int* __restrict__ scol, const int* __restrict__ erow, const int* __restrict__ cev,
     const int* __restrict__ wtail, const float* __restrict__ scale, const StreamHeader* __restrict__ header,
-    int num_wave_chunks, int num_events,
+    int* __restrict__ fault, int generation, int num_wave_chunks, int num_events,
     int num_nodes, int num_partials, int chunks, unsigned ld_bytes, int width_out, int ld_out, unsigned table_bytes)
 {
     constexpr int TPW = kWave / TS;
@@ -93,8 +110,12 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     const int w = blockIdx.x * kStreamWaves + wave;
     if (w >= num_wave_chunks) return;                       // wave-uniform; the LDS rows are wave-private
     // the counts the host remembers must be those of the plan in memory (they are unless the plan's bytes were
-    // replaced behind the library's back): a mismatch ends the kernel instead of indexing with the wrong sizes
-    if (header->num_events != num_events || header->num_partials != num_partials || header->valid != 1) return;
+    // replaced behind the library's back): a mismatch ends the kernel instead of indexing with the wrong sizes,
+    // and leaves a mark that eppgcn_aggregation_status reports (the output of this call is not written)
+    if (header_mismatch(header, generation, num_events, num_partials)) {
+        if (w == 0 && lane == 0) report_mismatch(fault, 1, generation, header->generation);
+        return;
+    }
     int* my_row = ev_row[wave];
     float* my_scale = ev_scale[wave];
 
@@ -276,11 +297,15 @@ template <int OVW, int TS>
 __global__ __launch_bounds__(256) void stream_fixup_kernel(float* __restrict__ out, const float* __restrict__ partial,
                                                            const int* __restrict__ frow, const int* __restrict__ fptr,
                                                            const float* __restrict__ scale, const StreamHeader* header,
+                                                           int* __restrict__ fault, int generation,
                                                            int num_partials, int chunks, unsigned ld_bytes,
                                                            int width_out, int ld_out)
 {
     constexpr int TPW = kWave / TS;
-    if (header->num_partials != num_partials || header->valid != 1) return;   // same rule as the stream kernel
+    if (header_mismatch(header, generation, -1, num_partials)) {              // same rule as the stream kernel
+        if (blockIdx.x == 0 && threadIdx.x == 0) report_mismatch(fault, 2, generation, header->generation);
+        return;
+    }
     const int num_fix = header->num_fix;
     const int lane = threadIdx.x & (kWave - 1);
     const int team = lane / TS;
@@ -342,6 +367,32 @@ __global__ __launch_bounds__(256) void stream_fixup_kernel(float* __restrict__ o
     }
 }
 
+// ---------------------------------------------------------------- the mark of a header mismatch
+static __device__ __align__(16) int plan_fault_words[kPlanFaultWords];
+}  // namespace eppgcn
+
+#include <map>
+#include <mutex>
+
+namespace eppgcn {
+static std::mutex g_fault_mutex;
+static std::map<int, int*> g_fault_address;     // per device: each GPU holds its own copy of the words
+
+int plan_fault_address(int** words)
+{
+    int device = 0;
+    EPPGCN_HIP(hipGetDevice(&device));
+    std::lock_guard<std::mutex> lock(g_fault_mutex);
+    auto it = g_fault_address.find(device);
+    if (it == g_fault_address.end()) {
+        void* p = nullptr;
+        EPPGCN_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(plan_fault_words)));
+        it = g_fault_address.emplace(device, static_cast<int*>(p)).first;
+    }
+    *words = it->second;
+    return kOk;
+}
+
 static int g_stream_mode = 1;
 void set_stream_mode(int on) { g_stream_mode = on ? 1 : 0; }
 
@@ -386,16 +437,19 @@ int launch_aggregate_stream(float* out, float* partial, const float* table, cons
     long long fix_blocks = (static_cast<long long>(num_fix) * ts + 255) / 256;
     if (fix_blocks > 256 * 64) fix_blocks = 256 * 64;
     const dim3 fgrid(static_cast<unsigned>(fix_blocks < 1 ? 1 : fix_blocks));
+    int* fault = nullptr;
+    if (int rc = plan_fault_address(&fault)) return rc;
 #define EPPGCN_STREAM(OVW_, TS_)                                                                                      \
     do {                                                                                                              \
         hipLaunchKernelGGL((aggregate_stream_kernel<OVW_, TS_, 8>), grid, block, 0, stream, out, partial, table,      \
-                           scol, sv.erow, sv.cev, sv.wtail, scale, sv.header, num_wave_chunks,                        \
-                           info.header.num_events,                                                                    \
+                           scol, sv.erow, sv.cev, sv.wtail, scale, sv.header, fault, info.header.generation,          \
+                           num_wave_chunks, info.header.num_events,                                                   \
                            num_nodes, info.header.num_partials, chunks, static_cast<unsigned>(ld_in) * 4u, dim, dim,  \
                            static_cast<unsigned>(bytes));                                                             \
         if (num_fix > 0)                                                                                              \
             hipLaunchKernelGGL((stream_fixup_kernel<OVW_, TS_>), fgrid, dim3(256), 0, stream, out, partial, sv.frow,  \
-                               sv.fptr, scale, sv.header, info.header.num_partials, chunks,                           \
+                               sv.fptr, scale, sv.header, fault, info.header.generation,                              \
+                               info.header.num_partials, chunks,                                                      \
                                static_cast<unsigned>(ld_in) * 4u, dim, dim);                                          \
     } while (0)
 #define EPPGCN_STREAM_TS(OVW_)                                                                                        \

@@ -65,6 +65,7 @@ extern "C" {
 #define EPPGCN_ERR_HIP (-2)
 #define EPPGCN_ERR_SCAN_STALLED (-3)
 #define EPPGCN_ERR_CAPACITY (-4)
+#define EPPGCN_ERR_PLAN_MISMATCH (-5)
 
 /* Message of the last failure on the calling thread ("" if none). */
 const char* eppgcn_last_error(void);
@@ -115,7 +116,15 @@ int64_t eppgcn_feature_workspace_row(int64_t vertex);
  *     fewer than 2^24 vertices (narrower rows are a power of two bytes apart and are addressed with a
  *     shift, wider ones with a 24-bit multiply),
  * and otherwise runs the group kernel over the same plan.  A plan that contains empty groups has no
- * stream form.  No counterpart in the reference. */
+ * stream form.  No counterpart in the reference.
+ *
+ * Life of a plan.  The plan's memory is the caller's; the library remembers, by the plan's address, the
+ * header it read in eppgcn_plan_status (counts and the number of the build).  Tell it with
+ * eppgcn_plan_release before that memory is freed or reused, and rebuild a plan whose bytes were
+ * overwritten.  The stream and fix-up kernels compare the header in memory with the remembered one before
+ * they index anything: on a difference they write no output and leave a mark, which
+ * eppgcn_aggregation_status reports as EPPGCN_ERR_PLAN_MISMATCH (the aggregation calls themselves are
+ * asynchronous and cannot). */
 /* 1 when a plan is expected to pay off: the [num_nodes, dim] feature table has 4 MB or more.  Large
  * tables (hundreds of MB) gain from the column-blocked order; small ones still gain from the
  * length-sorted groups, the precomputed group flags and the selective output clear; below that the
@@ -128,8 +137,9 @@ int eppgcn_build_plan(const int32_t* part_pointers, const int32_t* column_index,
                       int num_nodes, int dim, int block_shift, void* plan, size_t plan_bytes,
                       void* workspace, size_t workspace_bytes, void* stream);
 /* eppgcn_build_plan is asynchronous and contains look-back scans.  This call synchronises `stream`,
- * reads the plan's header and returns 0 or EPPGCN_ERR_SCAN_STALLED (a stalled scan leaves a corrupt
- * plan, which must not be used).  Pass the sizes the plan was built with.  *partial_rows (may be
+ * reads the plan's header and returns 0, EPPGCN_ERR_SCAN_STALLED (a stalled scan leaves a corrupt
+ * plan, which must not be used) or EPPGCN_ERR_PLAN_MISMATCH (the memory does not hold the header of a
+ * finished build of this process with these sizes).  Pass the sizes the plan was built with.  *partial_rows (may be
  * NULL) receives the number of partial sums a call through the stream form needs room for (0 when
  * the plan has no stream form).  The library remembers the header by the plan's address until the
  * next eppgcn_build_plan into that address, and the aggregation calls use the stream form only for
@@ -138,13 +148,21 @@ int eppgcn_build_plan(const int32_t* part_pointers, const int32_t* column_index,
  * called for the copy. */
 int eppgcn_plan_status(const void* plan, int num_parts, int64_t num_slots, int num_nodes,
                        int64_t* partial_rows, void* stream);
+/* Makes the library forget what it remembers about the plan at this address (NULL is ignored).  Call it
+ * before the plan's memory is freed or reused; eppgcn_build_plan into the same address does it by itself. */
+void eppgcn_plan_release(const void* plan);
+/* Synchronises `stream` and returns EPPGCN_ERR_PLAN_MISMATCH - once - when, since the last such report,
+ * the stream or fix-up kernel of an aggregation call on the current device found a plan header in memory
+ * that was not the one eppgcn_plan_status had read at that address (the plan's bytes were overwritten, or
+ * its memory was reused without eppgcn_plan_release).  That call wrote no output.  0 otherwise.  Ask once
+ * per batch of calls, next to the other status calls; planned calls through the group kernel and calls
+ * without a plan never raise it. */
+int eppgcn_aggregation_status(void* stream);
 /* Floats of the feature workspace that lets a [num_nodes, dim] aggregation over `plan` take the
  * stream form: eppgcn_feature_workspace_floats(num_nodes, dim) plus one row per partial sum (what
  * eppgcn_plan_status reported).  Equal to eppgcn_feature_workspace_floats for NULL or a plan
  * without (known) stream form. */
 size_t eppgcn_plan_workspace_floats(const void* plan, int64_t num_nodes, int dim);
-/* 0 keeps every planned call on the group kernel (for comparisons); 1 (default) allows the stream form. */
-void eppgcn_set_stream_mode(int on);
 /* 1 when the calling thread's last aggregation call ran the stream form, 0 when it ran the group kernel. */
 int eppgcn_last_call_used_stream(void);
 
@@ -219,7 +237,8 @@ size_t eppgcn_compact_workspace_bytes(int64_t length);
 size_t eppgcn_split_workspace_bytes(int64_t num_nodes);
 
 /* Status of the last scan-based call that used `workspace` (eppgcn_compact_back_edge,
- * eppgcn_mark_compact, eppgcn_split_back_part, eppgcn_build_part): synchronises `stream`, then
+ * eppgcn_mark_compact, eppgcn_split_back_part, eppgcn_build_part; NULL = the static scratch of
+ * eppgcn_compact_back_edge_static on the current device): synchronises `stream`, then
  * returns 0, EPPGCN_ERR_SCAN_STALLED (a look-back wait hit its spin limit: the outputs of that call
  * are invalid) or EPPGCN_ERR_CAPACITY (the group pointers did not fit).  The scan-based calls check
  * this themselves only when a host result (h_*) is requested; a caller that takes every count on
@@ -246,9 +265,13 @@ int eppgcn_compact_back_edge(const int32_t* edge_mask, const int32_t* column_ind
  * (cuCompactor.cu:328-465).
  *   - length may be at most eppgcn_compact_back_edge_static_max_length() = 2^30 slots; a longer
  *     input fails with EPPGCN_ERR_CAPACITY and a message, before any device work.
- *   - The array (2 MiB + 32 bytes) exists once per GPU the library runs on, for the life of the
- *     process; its address on a device is looked up on the first call there (the device that is
- *     current at the call).
+ *   - The array (512 KiB + 32 bytes: the scan state and one descriptor per 16384-slot tile) exists once
+ *     per GPU the library runs on, for the life of the process; its address on a device is looked up on
+ *     the first call there (the device that is current at the call).  A caller that captures the call
+ *     into a HIP graph makes one call - this one, or eppgcn_scan_status(NULL, stream) - on that device
+ *     outside the capture first.
+ *   - With h_valid_len == NULL nothing synchronises and a stalled look-back goes unreported by the call
+ *     itself: eppgcn_scan_status(NULL, stream) reads the status from the static scratch afterwards.
  *   - Every call on a GPU uses that GPU's one array (it is cleared at the start of each call), so
  *     calls that overlap on one GPU - on different streams or from different threads - race and
  *     must be serialised by the caller. */
@@ -395,35 +418,6 @@ void eppgcn_clear_time(void);
  * aggregation kernels alone, as the reference's timers do), 100+k backward aggregation of layer k
  * (1-based, k <= 16).  Milliseconds. */
 double eppgcn_get_time_ms(int which);
-
-/* Forces the number of lanes per neighbour group in the aggregation kernels
- * (power of two in 4..64; 0 = choose from the feature width).  For tuning runs. */
-void eppgcn_set_team_size(int lanes);
-/* Forces the number of consecutive group rounds one wave processes (0 = choose from
- * the group size so that a wave gathers about 512 rows).  For tuning runs. */
-void eppgcn_set_rounds(int rounds);
-/* The output-clear and pre-scaling kernels index with 32 bits while the matrices have fewer than 2^32
- * elements; 1 forces their 64-bit instantiations at any size.  For tests. */
-void eppgcn_set_wide_index(int on);
-/* For tests of the stall path of the look-back scans: spin_limit > 0 replaces the number of polls after
- * which a waiting tile gives up (default 2^22); mute_first_tile != 0 makes tile 0 of every scan keep its
- * result to itself, so that every later tile runs into the limit, raises the stall flag and carries on
- * with what it has - the kernels still finish, the results are invalid, and the calls that read the
- * status return EPPGCN_ERR_SCAN_STALLED.  (0, 0) restores normal operation. */
-void eppgcn_set_scan_test_mode(unsigned spin_limit, int mute_first_tile);
-/* Forces the column block size of eppgcn_build_plan to 2^shift vertices (0 = choose from the
- * feature width).  For tuning runs. */
-void eppgcn_set_plan_shift(int shift);
-/* Plan policy (tuning runs).  Rows of at most 32 * groups slots (and at most 64 groups) stay together in
- * a plan instead of being cut at column-block borders (0 = block every group).  Negative (the default) =
- * chosen per build: 2 when the launch shape (num_nodes, dim) is one the stream form runs, 8 when the
- * group kernel will run over the plan. */
-void eppgcn_set_plan_keep_rows(int groups);
-/* Within a column block, order single-group rows by length class (1-8, 9-16, 17-24, 25+ slots) so
- * that the groups of one round take the same number of gather steps.  1 on, 0 off, negative (the
- * default) = per build: off for the stream form (its gather instructions are full whatever the
- * lengths), on for the group kernel. */
-void eppgcn_set_plan_length_classes(int on);
 
 #ifdef __cplusplus
 }

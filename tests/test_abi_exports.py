@@ -6,10 +6,23 @@ import re
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_functions():
-    text = open(os.path.join(ROOT, "include", "eppgcn_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(eppgcn_[a-z0-9_]+)\s*\(", text)))
+HEADERS = ("eppgcn_hip.h", "eppgcn_hip_tuning.h")     # the drop-in surface; the process-wide tuning and test knobs
+
+
+def declared_functions(headers=HEADERS):
+    names = set()
+    for header in headers:
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(eppgcn_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
+
+
+def test_tuning_knobs_stay_out_of_the_product_header():
+    product = declared_functions(("eppgcn_hip.h",))
+    assert not [n for n in product if n.startswith("eppgcn_set_") and n != "eppgcn_set_timing"]
+    knobs = declared_functions(("eppgcn_hip_tuning.h",))
+    assert knobs and all(n.startswith("eppgcn_set_") for n in knobs)
 
 
 def test_header_declares_the_expected_surface():
@@ -26,7 +39,7 @@ def test_library_exports_every_declared_symbol():
     assert os.path.exists(capi.LIB_PATH), "build the library first: python -m eppgcn_amd.build"
     lib = ctypes.CDLL(capi.LIB_PATH)
     for name in declared_functions():
-        assert hasattr(lib, name), f"{name} is declared in include/eppgcn_hip.h but not exported"
+        assert hasattr(lib, name), f"{name} is declared under include/ but not exported"
     assert sorted(capi.EXPORTS) == declared_functions()
     assert capi.load().eppgcn_abi_version() == capi.ABI_VERSION
 
@@ -78,13 +91,15 @@ def test_argument_errors_are_reported_before_any_device_work():
         (lib.eppgcn_spmm_forward(one, p0, p0, one, one, one, one, 8, 4, 2, 1, 1, 1, p0, 0, p0, p0), "null feature"),
         (lib.eppgcn_spmm_forward(one, one, p0, one, one, one, one, 8, 0, 2, 1, 1, 1, p0, 0, p0, p0), "dim > 0"),
     ]
-    cases += [(lib.eppgcn_scan_status(p0, p0), "workspace"), (lib.eppgcn_plan_status(p0, 5, 9, 4, None, p0), "plan"),
+    cases += [(lib.eppgcn_scan_status(ctypes.c_void_p(20), p0), "workspace"), (lib.eppgcn_plan_status(p0, 5, 9, 4, None, p0), "plan"),
               (lib.eppgcn_plan_status(one, -1, 0, 4, None, p0), "negative")]
     for rc, needle in cases:
         assert rc == -1
     # the message belongs to the last failing call
     assert b"negative" in lib.eppgcn_last_error()
     assert lib.eppgcn_plan_status(p0, 0, 0, 4, None, p0) == 0
+    lib.eppgcn_plan_release(p0)           # both are no-ops for a plan the library does not know
+    lib.eppgcn_plan_release(one)
     # a plan the library has not seen is sized like the plain feature workspace
     assert lib.eppgcn_plan_workspace_floats(one, 10, 22) == lib.eppgcn_feature_workspace_floats(10, 22) == 4096 * 32
     assert [lib.eppgcn_feature_workspace_row(r) for r in (0, 31, 32, 4095, 4096, 131072 + 64)] == [0, 31, 33, 4095 ^ 127, 4096 ^ 128, (131072 + 64) ^ 2]

@@ -376,3 +376,71 @@ def test_stream_random_ragged_graphs_exact(api, seed):
     finally:
         api.set_plan_keep_rows(None)
         api.set_plan_length_classes(None)
+
+
+def test_replaced_plan_header_is_reported_not_silent(api):
+    """A plan whose header in memory is no longer the one the library read there: the stream and fix-up kernels
+    write nothing, leave a mark, and eppgcn_aggregation_status reports it once (-5); eppgcn_plan_status refuses
+    bytes that are not a finished build's header; after a rebuild everything works again.  Every kernel exits
+    normally throughout."""
+    indptr, col = GRAPHS["hub"]()
+    n = indptr.size - 1
+    dim = 16
+    s = scale_inv_sqrt(indptr)
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((n, dim)).astype(np.float32)
+    want = co.spmm_f64(x, indptr, col, s)
+    bound = cf.abs_sum_bound(indptr, col, s, x)
+    pp, p2n = co.build_part(8, indptr)
+    args = (dev(col), dev(s), dev(pp), dev(p2n))
+    lib = api.load()
+
+    def call(plan, ws):
+        out = torch.full((n, dim), -123.0, device="cuda")
+        api.spmm_forward(dev(x), *args, part_size=8, out=out, plan=plan, workspace=ws)
+        return out
+
+    plan = api.build_plan(dev(pp), dev(col), p2n.size, col.size, n, dim, part2node=dev(p2n))
+    ws = api.feature_workspace(n, dim, "cuda", plan)
+    out = call(plan, ws)
+    assert api.last_call_used_stream()
+    assert_close(out.cpu().numpy(), want, bound, "intact plan")
+    api.aggregation_status()                                     # nothing to report
+
+    header = plan.stream_view()["header"]
+    saved = header.clone()
+    for word, what in ((2, "num_partials"), (8, "generation"), (0, "valid"), (7, "magic")):
+        header[word] += 1                                        # the plan's bytes change behind the library's back
+        out = call(plan, ws)
+        assert api.last_call_used_stream()                       # the host still believes in the plan it remembers
+        assert bool((out == -123.0).all()), f"{what}: the kernels must not write through a header they do not know"
+        with pytest.raises(api.EppgcnError, match="-5.*plan"):
+            api.aggregation_status()
+        api.aggregation_status()                                 # reported once
+        header.copy_(saved)
+        assert_close(call(plan, ws).cpu().numpy(), want, bound, f"{what} restored")
+        api.aggregation_status()
+
+    # plan_status takes on only the header of a finished build with these sizes
+    status = lambda: lib.eppgcn_plan_status(plan.base_ptr, plan.num_parts, plan.num_slots, plan.num_nodes, None, None)
+    header[7] = 0
+    assert status() == -5 and b"does not hold a plan" in lib.eppgcn_last_error()
+    header.copy_(saved)
+    header[9] += 1                                               # another group count than the caller states
+    assert status() == -5
+    header.copy_(saved)
+    # the plan is forgotten after a refused status: the group kernel runs over the (intact) group arrays
+    out = call(plan, ws)
+    assert not api.last_call_used_stream()
+    assert_close(out.cpu().numpy(), want, bound, "forgotten plan")
+    assert status() == 0
+    assert_close(call(plan, ws).cpu().numpy(), want, bound, "known again")
+    assert api.last_call_used_stream()
+
+    # released: unknown to the library again; a rebuild into the same memory gets a new build number
+    plan.release()
+    plan2 = api.build_plan(dev(pp), dev(col), p2n.size, col.size, n, dim, part2node=dev(p2n))
+    assert plan2.stream_view()["header"][8].item() > int(saved[8])
+    assert_close(call(plan2, api.feature_workspace(n, dim, "cuda", plan2)).cpu().numpy(), want, bound, "rebuilt")
+    assert api.last_call_used_stream()
+    api.aggregation_status()

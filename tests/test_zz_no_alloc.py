@@ -15,6 +15,9 @@ def api():
         pytest.skip("needs the MI355X")
     from eppgcn_amd import capi
     capi.load()
+    # the documented first call on the device: looks up the static scratch's address (what it reports is the
+    # status of whichever call used the scratch last, possibly another test's forced stall: not looked at here)
+    capi.load().eppgcn_scan_status(None, None)
     return capi, torch
 
 
@@ -34,7 +37,11 @@ def _compare(capi, torch, length, density, seed, out_id, out_edge, d_count):
     out_id.fill_(-7)
     out_edge.fill_(-7)
     d_count.fill_(-7)
+    torch.cuda.synchronize()
+    free_before, held_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
     got_v = capi.compact_back_edge_static(mask, col, out_id, out_edge, d_valid_len=d_count)
+    # the call allocates nothing: neither from the device (hipMemGetInfo) nor from torch's pool
+    assert torch.cuda.mem_get_info()[0] == free_before and torch.cuda.memory_allocated() == held_before
     assert got_v == want_v == kept
     assert int(d_count.item()) == kept
     assert torch.equal(out_id[:length], want_id), "row ids differ (zero tail included)"
@@ -69,6 +76,7 @@ def test_static_scratch_compaction_without_a_host_count(api):
     d_count = torch.zeros(1, dtype=torch.int32, device=dev)
     assert capi.compact_back_edge_static(mask, col, out_id, out_edge, d_valid_len=d_count, host_count=False) is None
     want_id, want_edge, want_v = capi.compact_back_edge(mask, col)
+    capi.scan_status(None)           # the status of the static scratch: no stall, nothing raised
     assert int(d_count.item()) == kept == want_v
     assert torch.equal(out_id, want_id) and torch.equal(out_edge, want_edge)
 
