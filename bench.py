@@ -62,6 +62,8 @@ def parse():
                     help="process the groups in CSR order instead of the column-blocked execution plan")
     ap.add_argument("--no_stream", action="store_true",
                     help="keep planned launches on the group kernel instead of the plan's stream form")
+    ap.add_argument("--wide_stream", action="store_true",
+                    help="force the stream kernel's 64-bit addressing variant (it otherwise runs for tables of 4 GB and more)")
     ap.add_argument("--no_workspace", action="store_true",
                     help="aggregate without the feature workspace (per-edge scale gather, no scratch)")
     ap.add_argument("--no_cpu_baseline", action="store_true")
@@ -162,6 +164,8 @@ def main():
     log(args, "graph", g.stats(), f"{time.perf_counter() - t0:.1f}s")
     if args.no_stream:
         capi.set_stream_mode(False)      # before the plans are built: their order follows the kernel that will run
+    elif args.wide_stream:
+        capi.set_stream_mode(True, wide=True)
     if args.plan_shift:
         capi.set_plan_shift(args.plan_shift)
     if args.length_classes:

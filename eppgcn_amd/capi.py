@@ -321,9 +321,10 @@ def last_call_used_stream() -> bool:
     return bool(load().eppgcn_last_call_used_stream())
 
 
-def set_stream_mode(on: bool):
-    """False keeps planned calls on the group kernel (comparisons); True (default) allows the stream form."""
-    load().eppgcn_set_stream_mode(int(bool(on)))
+def set_stream_mode(on: bool, wide: bool = False):
+    """False keeps planned calls on the group kernel (comparisons); True (default) allows the stream form;
+    ``wide`` forces the stream kernel's 64-bit addressing variant at any table size (tests)."""
+    load().eppgcn_set_stream_mode(2 if (on and wide) else int(bool(on)))
 
 
 STREAM_WAVE = 512      # slots a wave of the stream kernel takes

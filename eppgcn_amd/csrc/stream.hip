@@ -89,13 +89,17 @@ __device__ __forceinline__ void report_mismatch(int* __restrict__ fault, int whi
     __hip_atomic_store(fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int OVW, int TS, int U>
+// kWide: the table is addressed with 64-bit global loads instead of 32-bit offsets into a buffer resource (tables of
+// 4 GB and more, wide rows of 2^24 vertices and more); the lanes a buffer load would have sent out of range load row 0
+// instead and their values are replaced by zeros when they are added.
+template <int OVW, int TS, int U, bool kWide>
 __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     float* __restrict__ out, float* __restrict__ partial, const float* __restrict__ table,
     const int* __restrict__ scol, const int* __restrict__ erow, const int* __restrict__ cev,
     const int* __restrict__ wtail, const float* __restrict__ scale, const StreamHeader* __restrict__ header,
     int* __restrict__ fault, int generation, int num_wave_chunks, int num_events,
-    int num_nodes, int num_partials, int chunks, unsigned ld_bytes, int width_out, int ld_out, unsigned table_bytes)
+    int num_nodes, int num_partials, int chunks, unsigned ld_bytes, int width_out, int ld_out, unsigned table_bytes,
+    unsigned pad_row)
 {
     constexpr int TPW = kWave / TS;
     constexpr int kParts = 8 / U;                  // batches per step
@@ -146,11 +150,17 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
             const unsigned id = swizzled_row(b.c[u] & 0x7fffffffu);      // the table's row order (common.hpp)
             // rows of a narrow team are a power of two bytes apart (row_step = log2): a shift serves any row count
             // of a table below 4 GB; wider rows use the 24-bit multiply (the host checks the row count)
-            unsigned row_off;
-            if constexpr (TS <= kStreamShiftTeams) row_off = id << row_step;
-            else row_off = __umul24(id, ld_bytes);
-            const unsigned off = lane_off == kNoRowOffset ? kNoRowOffset : row_off + lane_off;
-            b.v[u] = __builtin_amdgcn_raw_buffer_load_b128(rows, off, 0, 0);
+            if constexpr (kWide) {
+                const bool ok = lane_off != kNoRowOffset && id < pad_row;
+                const unsigned long long off = static_cast<unsigned long long>(id) * ld_bytes + lane_off;
+                b.v[u] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(table) + (ok ? off : 0ull));
+            } else {
+                unsigned row_off;
+                if constexpr (TS <= kStreamShiftTeams) row_off = id << row_step;
+                else row_off = __umul24(id, ld_bytes);
+                const unsigned off = lane_off == kNoRowOffset ? kNoRowOffset : row_off + lane_off;
+                b.v[u] = __builtin_amdgcn_raw_buffer_load_b128(rows, off, 0, 0);
+            }
         }
     };
     using P0 = std::integral_constant<int, 0>;
@@ -207,10 +217,15 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     auto consume = [&](const StreamBatch<U>& b) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            acc[0] += __uint_as_float(b.v[u].x);
-            acc[1] += __uint_as_float(b.v[u].y);
-            acc[2] += __uint_as_float(b.v[u].z);
-            acc[3] += __uint_as_float(b.v[u].w);
+            u32x4 v = b.v[u];
+            if constexpr (kWide) {          // what a buffer load would have returned as zeros
+                const bool ok = lane_off != kNoRowOffset && swizzled_row(b.c[u] & 0x7fffffffu) < pad_row;
+                if (!ok) v = u32x4{0u, 0u, 0u, 0u};
+            }
+            acc[0] += __uint_as_float(v.x);
+            acc[1] += __uint_as_float(v.y);
+            acc[2] += __uint_as_float(v.z);
+            acc[3] += __uint_as_float(v.w);
             if (static_cast<int>(b.c[u]) < 0) {            // the slot ends a piece
                 if (head_pending) {
 #pragma unroll
@@ -394,7 +409,8 @@ int plan_fault_address(int** words)
 }
 
 static int g_stream_mode = 1;
-void set_stream_mode(int on) { g_stream_mode = on ? 1 : 0; }
+static bool g_force_wide_stream = false;     // tests: the 64-bit addressing variant at any size
+void set_stream_mode(int on) { g_stream_mode = on ? 1 : 0; g_force_wide_stream = on == 2; }
 
 // Team size for rows of `chunks` 16-byte vectors, 0 when the stream kernel does not cover the shape.
 static int stream_team(int chunks)
@@ -404,18 +420,24 @@ static int stream_team(int chunks)
     return chunks <= 64 ? ts : 0;
 }
 
+// Does the shape need 64-bit addressing?  32-bit byte offsets cover tables below 4 GB; teams of up to kStreamShiftTeams
+// lanes turn a row into a byte offset with a shift (rows a power of two bytes apart: the workspace's pitch for such
+// widths), wider teams multiply 24-bit operands.
+static bool stream_needs_wide(int num_nodes, int dim, int ld_in)
+{
+    const unsigned long long bytes = static_cast<unsigned long long>(swizzle_padded_rows(num_nodes)) * ld_in * 4ull;
+    if (bytes + 16 >= (1ull << 32)) return true;
+    if (stream_team((dim + 3) / 4) <= kStreamShiftTeams) return (ld_in & (ld_in - 1)) != 0;
+    return !(swizzle_padded_rows(num_nodes) < (1 << 24) && ld_in * 4 < (1 << 24));
+}
+
 // Can a launch over a pre-scaled table with rows of ld_in floats run through the stream kernel?
 bool stream_covers(int num_nodes, int dim, int ld_in, const float* table)
 {
     if (!g_stream_mode || force_wide_index()) return false;
     if (ld_in % 4 != 0 || reinterpret_cast<uintptr_t>(table) % 16 != 0) return false;
     if (stream_team((dim + 3) / 4) == 0 || (dim + 3) / 4 * 4 > ld_in) return false;
-    const unsigned long long bytes = static_cast<unsigned long long>(swizzle_padded_rows(num_nodes)) * ld_in * 4ull;
-    if (bytes + 16 >= (1ull << 32)) return false;                      // 32-bit byte offsets into the table
-    // teams of up to kStreamShiftTeams lanes turn a row into a byte offset with a shift: rows a power of two bytes apart
-    // (the workspace's pitch for such widths), any row count; wider teams multiply 24-bit operands
-    if (stream_team((dim + 3) / 4) <= kStreamShiftTeams) return (ld_in & (ld_in - 1)) == 0;
-    return swizzle_padded_rows(num_nodes) < (1 << 24) && ld_in * 4 < (1 << 24);
+    return swizzle_padded_rows(num_nodes) < (1ll << 31);
 }
 
 // Stream kernel + fix-up kernel over a pre-scaled table in swizzled row order (stream_covers() holds).  `partial` holds
@@ -427,7 +449,9 @@ int launch_aggregate_stream(float* out, float* partial, const float* table, cons
     const int chunks = (dim + 3) / 4;
     const int ts = stream_team(chunks);
     const long long padded = stream_padded_slots(info.num_slots);
-    const unsigned long long bytes = static_cast<unsigned long long>(swizzle_padded_rows(num_nodes)) * ld_in * 4ull;
+    const bool wide = stream_needs_wide(num_nodes, dim, ld_in) || g_force_wide_stream;
+    const unsigned long long bytes = wide ? 0ull : static_cast<unsigned long long>(swizzle_padded_rows(num_nodes)) * ld_in * 4ull;
+    const unsigned pad_row = static_cast<unsigned>(swizzle_padded_rows(num_nodes));
     const int num_wave_chunks = static_cast<int>(padded / kStreamWave);
     if (num_wave_chunks == 0) return kOk;
     const dim3 grid((num_wave_chunks + kStreamWaves - 1) / kStreamWaves), block(kStreamBlock);
@@ -439,13 +463,16 @@ int launch_aggregate_stream(float* out, float* partial, const float* table, cons
     const dim3 fgrid(static_cast<unsigned>(fix_blocks < 1 ? 1 : fix_blocks));
     int* fault = nullptr;
     if (int rc = plan_fault_address(&fault)) return rc;
+#define EPPGCN_STREAM_KERNEL(OVW_, TS_, WIDE_)                                                                        \
+    hipLaunchKernelGGL((aggregate_stream_kernel<OVW_, TS_, 8, WIDE_>), grid, block, 0, stream, out, partial, table,   \
+                       scol, sv.erow, sv.cev, sv.wtail, scale, sv.header, fault, info.header.generation,              \
+                       num_wave_chunks, info.header.num_events,                                                       \
+                       num_nodes, info.header.num_partials, chunks, static_cast<unsigned>(ld_in) * 4u, dim, dim,      \
+                       static_cast<unsigned>(bytes), pad_row)
 #define EPPGCN_STREAM(OVW_, TS_)                                                                                      \
     do {                                                                                                              \
-        hipLaunchKernelGGL((aggregate_stream_kernel<OVW_, TS_, 8>), grid, block, 0, stream, out, partial, table,      \
-                           scol, sv.erow, sv.cev, sv.wtail, scale, sv.header, fault, info.header.generation,          \
-                           num_wave_chunks, info.header.num_events,                                                   \
-                           num_nodes, info.header.num_partials, chunks, static_cast<unsigned>(ld_in) * 4u, dim, dim,  \
-                           static_cast<unsigned>(bytes));                                                             \
+        if (wide) EPPGCN_STREAM_KERNEL(OVW_, TS_, true);                                                              \
+        else EPPGCN_STREAM_KERNEL(OVW_, TS_, false);                                                                  \
         if (num_fix > 0)                                                                                              \
             hipLaunchKernelGGL((stream_fixup_kernel<OVW_, TS_>), fgrid, dim3(256), 0, stream, out, partial, sv.frow,  \
                                sv.fptr, scale, sv.header, fault, info.header.generation,                              \
@@ -467,6 +494,7 @@ int launch_aggregate_stream(float* out, float* partial, const float* table, cons
     else EPPGCN_STREAM_TS(1);
 #undef EPPGCN_STREAM_TS
 #undef EPPGCN_STREAM
+#undef EPPGCN_STREAM_KERNEL
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }

@@ -112,9 +112,9 @@ int64_t eppgcn_feature_workspace_row(int64_t vertex);
  *   - eppgcn_plan_status has been called for the plan (it reads the counts the host needs),
  *   - a separate feature workspace is given (not NULL, not the input itself) that holds at least
  *     eppgcn_plan_workspace_floats(plan, num_nodes, dim) floats (the table plus the partial sums),
- *   - rows are at most 1024 bytes and the table is below 4 GB; rows of more than 128 bytes also need
- *     fewer than 2^24 vertices (narrower rows are a power of two bytes apart and are addressed with a
- *     shift, wider ones with a 24-bit multiply),
+ *   - rows are at most 1024 bytes (tables below 4 GB are addressed with 32-bit offsets - rows of up to
+ *     128 bytes with a shift, wider ones, below 2^24 vertices, with a 24-bit multiply - larger ones
+ *     with 64-bit loads),
  * and otherwise runs the group kernel over the same plan.  A plan that contains empty groups has no
  * stream form.  No counterpart in the reference.
  *

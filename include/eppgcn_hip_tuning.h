@@ -16,8 +16,10 @@
 extern "C" {
 #endif
 
-/* 0 keeps every planned call on the group kernel (for comparisons); 1 (default) allows the stream form.
- * Set it before the plans are built: the order of a plan follows the kernel that will run over it. */
+/* 0 keeps every planned call on the group kernel (for comparisons); 1 (default) allows the stream form;
+ * 2 allows it and forces its 64-bit addressing variant at any table size (for tests: it otherwise runs
+ * for tables of 4 GB and more).  Set it before the plans are built: the order of a plan follows the
+ * kernel that will run over it. */
 void eppgcn_set_stream_mode(int on);
 /* Forces the number of lanes per neighbour group in the aggregation kernels
  * (power of two in 4..64; 0 = choose from the feature width).  For tuning runs. */

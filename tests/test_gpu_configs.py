@@ -272,8 +272,8 @@ def test_headline_size_benched_numeric_path_within_tolerance(api):
 def test_stream_form_with_25_bit_vertex_ids(api):
     """R-MAT scale 25, one generated pair per vertex (33.5 M vertices, many of them isolated): vertex ids and the
     padding id need 25 bits.  At width 16 (64-byte rows, a 2 GB table) the stream form addresses rows with a
-    shift and runs; at width 22 the table passes 4 GB and the group kernel takes the same plan.  Both against
-    the float64 sparse product."""
+    shift; at width 22 the table passes 4 GB and the stream kernel addresses it with 64-bit loads.  Both against
+    the float64 sparse product, and both the same bits on a second run."""
     from eppgcn_amd import graphs
     g = graphs.make_graph("rmat:25:1", device="cuda")
     n, e = g.num_nodes, g.num_edges
@@ -282,7 +282,7 @@ def test_stream_form_with_25_bit_vertex_ids(api):
     part_ptr, part2node = api.build_part(ps, g.row_pointers, e)
     col = g.column_index.long()
     w = (g.degrees[g.row_index()] * g.degrees[col]).double()
-    for dim, streams in ((16, True), (22, False)):
+    for dim, streams in ((16, True), (22, True)):
         plan = api.build_plan(part_ptr, g.column_index, part2node.numel(), e, n, dim, part2node=part2node)
         ws = api.feature_workspace(n, dim, "cuda", plan)
         x = graphs.normal32(3, (n, dim), "cuda", dim)

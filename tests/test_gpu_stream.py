@@ -444,3 +444,32 @@ def test_replaced_plan_header_is_reported_not_silent(api):
     assert_close(call(plan2, api.feature_workspace(n, dim, "cuda", plan2)).cpu().numpy(), want, bound, "rebuilt")
     assert api.last_call_used_stream()
     api.aggregation_status()
+
+
+@pytest.mark.parametrize("dim", [3, 16, 22, 40, 64, 100, 256])
+def test_stream_kernel_with_64_bit_addressing_gives_the_same_bits(api, dim):
+    """The variant for tables of 4 GB and more (64-bit global loads; lanes that a buffer load sends out of range
+    load row 0 and count as zeros), forced at small size: the same bits as the 32-bit variant, every team size,
+    padding slots and unused lanes included; and within tolerance of the checker."""
+    indptr, col = GRAPHS["two hubs"]()
+    n = indptr.size - 1
+    s = scale_inv_sqrt(indptr)
+    rng = np.random.default_rng(dim)
+    x = rng.standard_normal((n, dim)).astype(np.float32)
+    pp, p2n = co.build_part(5, indptr)
+    args = (dev(x), dev(col), dev(s), dev(pp), dev(p2n))
+    api.set_plan_shift(11)
+    plan = api.build_plan(dev(pp), dev(col), p2n.size, col.size, n, dim, part2node=dev(p2n))
+    ws = api.feature_workspace(n, dim, "cuda", plan)
+    ws.fill_(float("nan"))                       # row 0 and everything else the masked lanes may touch
+    narrow = api.spmm_forward(*args, part_size=5, plan=plan, workspace=ws)
+    assert api.last_call_used_stream()
+    try:
+        api.set_stream_mode(True, wide=True)
+        out = torch.full((n, dim), float("nan"), device="cuda")
+        api.spmm_forward(*args, part_size=5, plan=plan, workspace=ws, out=out)
+        assert api.last_call_used_stream()
+    finally:
+        api.set_stream_mode(True)
+    assert torch.equal(out, narrow), "64-bit and 32-bit addressing must agree bit for bit"
+    assert_close(out.cpu().numpy(), co.spmm_f64(x, indptr, col, s), cf.abs_sum_bound(indptr, col, s, x), f"D={dim}")
