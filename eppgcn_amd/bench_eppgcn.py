@@ -62,10 +62,13 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--num_epoches", type=int, default=100)
     ap.add_argument("--loadFromTxt", type=str, default="True", choices=["True", "False"])
     ap.add_argument("--degree_norm", type=str, default="sqrt", choices=["sqrt", "inv_sqrt"])
+    ap.add_argument("--with_unpruned", action="store_true",
+                    help="run every combination a second time with the unpruned backward aggregation (the driver's "
+                         "--prune False) and report its times beside the pruned ones")
     return ap
 
 
-def driver_arguments(args, name, dim, classes, hidden, ratio, layers):
+def driver_arguments(args, name, dim, classes, hidden, ratio, layers, prune=True):
     """The flags of EPPGCN/bench_EPPGCN.py:54-59 for one combination."""
     back_mode, backsize = BACK_MODES[args.groupsize_model]
     folder = osp.join(args.dataRoot, name)
@@ -74,7 +77,7 @@ def driver_arguments(args, name, dim, classes, hidden, ratio, layers):
             "--manual_mode", "False", "--verbose_mode", "False", "--loadFromTxt", args.loadFromTxt,
             "--dataDir", folder if osp.isdir(folder) else args.dataRoot, "--train_ratio", str(ratio),
             "--backsize_mode", back_mode, "--backsize", str(backsize), "--num_epoches", str(args.num_epoches),
-            "--degree_norm", args.degree_norm]
+            "--degree_norm", args.degree_norm, "--prune", str(bool(prune))]
 
 
 def main(argv=None) -> int:
@@ -94,6 +97,12 @@ def main(argv=None) -> int:
                     try:
                         rc = gcn_main.main(driver_arguments(args, name, dim, classes, hidden, ratio, layers), report)
                         line.update(report, status="ok" if rc == 0 else f"driver returned {rc}")
+                        if rc == 0 and args.with_unpruned:
+                            GNNA.clear_plans()
+                            plain = {}
+                            rc = gcn_main.main(driver_arguments(args, name, dim, classes, hidden, ratio, layers, False), plain)
+                            line["unpruned"] = {k: plain.get(k) for k in ("Time", "for_time", "back_time", "back_agg_time",
+                                                                          "for_agg_time", "build_time")}
                     except FileNotFoundError as exc:
                         rc = 0
                         line.update(status="skipped", reason=str(exc))

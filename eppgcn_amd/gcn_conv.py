@@ -37,7 +37,11 @@ class GNNAFunction(torch.autograd.Function):
     ``reluInput`` (an addition, default off) makes the layer consume ``relu(X)`` without the
     activation ever being written out: the product applies it while loading X, and the backward
     returns the gradient with respect to X itself (masked where X <= 0).  dX is skipped when X
-    needs no gradient (the first layer's features)."""
+    needs no gradient (the first layer's features).
+
+    A path record with ``unpruned = True`` (an addition, for the "no pruning" ablation the reference's module
+    exports as ``backward`` but its layer never calls) makes the backward run the unpruned aggregation over the
+    forward groups instead: the same gradients, since the incoming gradient is zero outside the path."""
 
     @staticmethod
     def forward(ctx, X, weight, inputInfo, maskInfo, backInfo, isFirstIter, isBackModeNet, reluInput=False):
@@ -55,8 +59,12 @@ class GNNAFunction(torch.autograd.Function):
     def backward(ctx, d_output):
         X, weight = ctx.saved_tensors
         wants_dx = bool(ctx.needs_input_grad[0])
-        d_input, d_weight = gnnadvisor().ours_backward(d_output.contiguous(), X, weight, *_path_args(ctx.backInfo),
-                                                       need_dx=wants_dx, relu_input=ctx.reluInput)
+        if getattr(ctx.backInfo, "unpruned", False):
+            d_input, d_weight = gnnadvisor().backward(d_output.contiguous(), X, weight, *_graph_args(ctx.inputInfo),
+                                                      need_dx=wants_dx, relu_input=ctx.reluInput)
+        else:
+            d_input, d_weight = gnnadvisor().ours_backward(d_output.contiguous(), X, weight, *_path_args(ctx.backInfo),
+                                                           need_dx=wants_dx, relu_input=ctx.reluInput)
         # one gradient slot per forward argument after ctx
         return (d_input if wants_dx else None, d_weight) + (None,) * 6
 

@@ -18,6 +18,8 @@ Differences, all deliberate:
     reference loader's sqrt(deg) (EPPGCN/dataset.py:117-119).
   * ``--kernel_timers`` and ``--hip_graph`` (additions) switch the per-op device timers off and
     replay the epoch from a HIP graph.
+  * ``--prune False`` (an addition) runs every layer's backward through the unpruned aggregation
+    (the module's ``backward`` export): the ablation the pruned path is compared with.
   * ``--model gin`` is accepted by the reference's parser but never read by it; here too.
   * ``--single_spmm`` / ``--verify_spmm`` are parsed and never read by the reference; here
     ``--single_spmm True`` times the forward aggregation alone and ``--verify_spmm True``
@@ -57,6 +59,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--backsize_mode", type=str, default="constant", choices=["map", "net", "constant", "wave64"])
     ap.add_argument("--degree_norm", type=str, default="sqrt", choices=["sqrt", "inv_sqrt"],
                     help="scale vector: sqrt(deg) as the reference's loader fills it, or deg^-1/2 (symmetric GCN norm)")
+    ap.add_argument("--prune", default="True", **tf,
+                    help="False: unpruned backward aggregation in every layer (ablation; same gradients)")
     ap.add_argument("--kernel_timers", default="True", **tf,
                     help="True: per-op device timers for the print_time report, as the reference always has; "
                          "False: none (the epochs are then issued without a host wait per op)")
@@ -131,7 +135,8 @@ def main(argv=None, report: dict = None) -> int:
     tr = train.Trainer(None, hidden=args.hidden, backsize_mode=args.backsize_mode, backsize=args.backsize or 32,
                        dataset=ds, part_size=args.partSize, dim_worker=args.dimWorker,
                        warp_per_block=args.warpPerBlock, shared_mem=args.sharedMem,
-                       manual_mode=args.manual_mode == "True", verbose=verbose, weight_seed=None)
+                       manual_mode=args.manual_mode == "True", verbose=verbose, weight_seed=None,
+                       prune=args.prune == "True")
     if verbose:
         print(tr.model)
     if args.single_spmm == "True" or args.verify_spmm == "True":

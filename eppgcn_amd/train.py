@@ -78,10 +78,13 @@ class Trainer:
     def __init__(self, graph: graphs.Graph, dim=96, hidden=16, num_classes=22, num_layers=2, train_ratio=0.1,
                  train_mask=None, backsize_mode="constant", backsize=32, labels="ones", weight_seed=3, lr=0.01,
                  fuse_relu=True, dataset=None, part_size=32, dim_worker=32, warp_per_block=8, shared_mem=100,
-                 manual_mode=False, verbose=False):
+                 manual_mode=False, verbose=False, prune=True):
         """``dataset``: a loaded ``eppgcn_amd.dataset.custom_dataset`` (or any object with the same
         attributes) to train on instead of synthetic features over ``graph``.  ``part_size`` ...
-        ``manual_mode`` are the driver's forward launch flags (EPPGCN/gcn_main.py:34-40)."""
+        ``manual_mode`` are the driver's forward launch flags (EPPGCN/gcn_main.py:34-40).  ``prune=False``: the
+        backward of every layer runs the unpruned aggregation (the module's ``backward`` export) instead of the
+        pruned one over the prepared path - the ablation next to which the pruned times are read."""
+        self.prune = bool(prune)
         self.GNNA = gnnadvisor()
         self.backsize_mode, self.backsize = backsize_mode, backsize
         if dataset is not None:
@@ -109,11 +112,13 @@ class Trainer:
             self.mask_props.append(maskInputProperty(src, dst, ds.edge_masks[num_layers - 1 - i],
                                                      ds.node_degs[num_layers - 1 - i], num_layers, i + 1, width))
             self.back_props.append(backInputProperty(degrees=ds.degrees, dim=width, layer=i + 1))
+            self.back_props[-1].unpruned = not self.prune
         self.model = Net(ds, hidden, num_layers, weight_seed, fuse_relu).to(ds.x.device)
         self.optimizer = torch.optim.Adam(self.model.parameters(), lr=lr)
         self.for_time = self.loss_time = self.back_time = self.build_time = 0.0
         self.losses: List[float] = []
         self.train_idx = self.train_y = None
+        self.kept_edges = [None] * num_layers      # per conv layer, filled by build_back_part
 
     def build_back_part(self):
         """EPPGCN/gcn_main.py:151-168 ('net' mode, which needs an unpublished predictor, is not offered)."""
@@ -129,6 +134,7 @@ class Trainer:
                 part_size = max(1, self.backsize)
             part_pointer, num_parts = self.GNNA.split_back_part(ds.node_degs[i], ds.num_edges, part_size)
             self.back_props[i].fillProperty(ids, part_pointer, edge_list, part_size, int(num_parts[0].item()))
+            self.kept_edges[i] = valid_len
             ds.edge_masks[i] = None      # the marking buffer is not needed after compaction
 
     def _loss(self, out):
@@ -194,11 +200,15 @@ class Trainer:
                "loss_time": round(self.loss_time, 6), "back_time": round(self.back_time, 6),
                "build_time": round(self.build_time, 6),
                "backward_group_sizes": [b.partSize for b in self.back_props],
-               "backward_groups": [b.numParts for b in self.back_props]}
+               "backward_groups": [b.numParts for b in self.back_props],
+               "kept_edges": list(self.kept_edges), "pruned": self.prune}
         if kernel_timing:
             res["for_agg_time"] = round(self.GNNA.get_time_ms(0) / 1e3, 6)
             res["back_agg_time"] = round(self.GNNA.get_time_ms(1) / 1e3, 6)
             res["mask_time"] = round(self.GNNA.get_time_ms(2) / 1e3, 6)
+            # l{k}_back_agg_time of the reference's report (EPPGCN_kernel.cu:96-106); the unpruned ablation has no
+            # per-layer timers (its entry point has no layer argument)
+            res["layer_back_agg_time"] = [round(self.GNNA.get_time_ms(101 + k) / 1e3, 6) for k in range(self.num_layers)]
         return res
 
 

@@ -402,6 +402,33 @@ def test_deeper_models_follow_the_mask_chain(GNNA, num_layers):
         src = nxt
 
 
+@pytest.mark.parametrize("num_layers", [2, 4])
+def test_unpruned_ablation_gives_the_gradients_of_the_pruned_path(GNNA, num_layers):
+    """``Trainer(prune=False)`` (the driver's ``--prune False``): every layer's backward runs the module's unpruned
+    ``backward`` over the forward groups.  The incoming gradient is zero outside the prepared path, so the weight
+    gradients agree with the pruned run to rounding."""
+    from eppgcn_amd import graphs, train
+    indptr, col = random_symmetric_csr(700, 2100, 43)
+    n = indptr.size - 1
+    g = graphs.Graph("t", n, dev(indptr), dev(col), dev(scale_inv_sqrt(indptr)))
+    mask = torch.from_numpy(np.random.default_rng(6).random(n) < 0.15)
+    grads = []
+    for prune in (True, False):
+        tr = train.Trainer(g, dim=20, hidden=16, num_classes=9, num_layers=num_layers, train_mask=mask, backsize=4,
+                           labels="uniform", prune=prune)
+        tr.optimizer = torch.optim.SGD(tr.model.parameters(), lr=0.0)
+        tr.train_step(True)
+        tr.train_step(False)
+        grads.append([c.weights.grad.cpu().numpy().copy() for c in tr.model.convs])
+        res = tr.run(2, warmup=0, kernel_timing=True)
+        assert res["pruned"] == prune and len(res["layer_back_agg_time"]) == num_layers
+        assert all(k is not None and k > 0 for k in res["kept_edges"])
+        assert (min(res["layer_back_agg_time"]) > 0) == prune       # the unpruned entry point has no per-layer timers
+        GNNA.clear_plans()
+    for a, b in zip(*grads):
+        assert np.linalg.norm(a - b) <= 1e-5 * np.linalg.norm(a) + 1e-12
+
+
 def test_group_size_rules_on_device_degrees(GNNA):
     """get_wave64_back_part_size / get_map_back_part_size on kept degrees that live on the device: the
     wave64 rule is 16 below 24 kept edges per kept row and 32 from there on; the fitted regression

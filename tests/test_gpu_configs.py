@@ -268,6 +268,14 @@ def test_headline_size_benched_numeric_path_within_tolerance(api):
     print("worst err / limit:", {k: round(v, 4) for k, v in worst.items()})
 
 
+@pytest.mark.parametrize("ratio", [0.3, 0.8])
+def test_mask_ratios_of_the_reference_sweep_at_size(api, rmat20, ratio):
+    """The mask ratios the reference's own sweep adds to the benchmark's (EPPGCN/bench_EPPGCN.py:35: 0.1, 0.3, 0.5,
+    0.8), on the R-MAT-20 graph at the widths of the 2-layer model: the same cell checks as above."""
+    for width in (16, 22):
+        test_backward_stress_cell(api, rmat20, ratio, width, 32)
+
+
 # ----------------------------------------------------------------------------- more than 2^24 vertices
 def test_stream_form_with_25_bit_vertex_ids(api):
     """R-MAT scale 25, one generated pair per vertex (33.5 M vertices, many of them isolated): vertex ids and the
