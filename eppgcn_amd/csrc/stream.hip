@@ -44,27 +44,41 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
-// A piece of OVW floats of an output row.  16-byte pieces belong to rows of whole 16-byte units, for the benchmark's
-// widths whole 64-byte sectors, written once and never read here: non-temporal stores.  Narrower pieces belong to
-// rows that share their sectors with their neighbours, which other teams write at other times: plain stores let the
-// cache put a sector together before it goes to memory (width 22, 88-byte rows at R-MAT 22: forward call 1.589 ->
-// 1.566 ms, backward 0.266 -> 0.254 ms; plain stores for 64-byte rows: forward call 1.092 -> 1.137 ms).
-template <int OVW>
-__device__ __forceinline__ void stream_store(float* p, const float* v)
+// How a team writes the floats of an output row it owns (lane tl holds columns 4 tl .. 4 tl + 3):
+//   kStoreExact  the row is exactly the team's TS * 16 bytes and 16-byte aligned (widths 16, 32, 64, ...): every lane
+//                stores its 16 bytes, non-temporally, and a partial sum (one table row wide) is stored the same way
+//   kStoreVec4   the width is a multiple of 4 floats, rows 16-byte aligned: the lanes below the width store 16 bytes,
+//                non-temporally (whole 16-byte units written once and never read here)
+//   kStorePlain  any width and alignment: 16 bytes per lane while four columns are left, then 8 and 4.  Such rows share
+//                their 32-byte sectors with their neighbours, which other teams write at other times: plain stores let
+//                the cache put a sector together before it goes to memory (width 22, 88-byte rows at R-MAT 22: forward
+//                call 1.589 -> 1.566 ms with plain instead of non-temporal stores; for 64-byte rows the other way round:
+//                1.092 -> 1.137 ms).  The pieces are only as aligned as the rows (4 or 8 bytes), which vector memory
+//                accesses of whole dwords may be.
+enum : int { kStoreExact = 0, kStoreVec4 = 1, kStorePlain = 2 };
+typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef float f32x2u __attribute__((ext_vector_type(2), aligned(4)));
+
+template <int MODE>
+__device__ __forceinline__ void store_row_floats(float* p, const float (&v)[4], int n)
 {
-    if constexpr (OVW == 4) {
-        const f32x4 t = {v[0], v[1], v[2], v[3]};
-        __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(p));
-    } else if constexpr (OVW == 2) {
-        const f32x2 t = {v[0], v[1]};
-        *reinterpret_cast<f32x2*>(p) = t;
+    if constexpr (MODE != kStorePlain) {
+        if (MODE == kStoreExact || n > 0) {
+            const f32x4 t = {v[0], v[1], v[2], v[3]};
+            __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(p));
+        }
     } else {
-        p[0] = v[0];
+        if (n >= 4) {
+            *reinterpret_cast<f32x4u*>(p) = f32x4u{v[0], v[1], v[2], v[3]};
+        } else if (n > 0) {
+            if (n & 2) *reinterpret_cast<f32x2u*>(p) = f32x2u{v[0], v[1]};
+            if (n & 1) p[n & 2] = v[n & 2];
+        }
     }
 }
 
 // table rows: pitch ld_bytes (a multiple of 16), `chunks` 16-byte vectors of a row are read (chunks <= TS);
-// out rows: pitch ld_out floats, columns < width_out written in pieces of OVW floats;
+// out rows: pitch ld_out floats, columns < width_out written as the store mode says;
 // partial rows: pitch ld_bytes, written whole (unscaled sums).
 // U: row gathers per batch (4 or 8); two batches are in flight.
 template <int U> struct StreamBatch {
@@ -92,7 +106,7 @@ __device__ __forceinline__ void report_mismatch(int* __restrict__ fault, int whi
 // kWide: the table is addressed with 64-bit global loads instead of 32-bit offsets into a buffer resource (tables of
 // 4 GB and more, wide rows of 2^24 vertices and more); the lanes a buffer load would have sent out of range load row 0
 // instead and their values are replaced by zeros when they are added.
-template <int OVW, int TS, int U, bool kWide>
+template <int MODE, int TS, int U, bool kWide>
 __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     float* __restrict__ out, float* __restrict__ partial, const float* __restrict__ table,
     const int* __restrict__ scol, const int* __restrict__ erow, const int* __restrict__ cev,
@@ -104,8 +118,10 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     constexpr int TPW = kWave / TS;
     constexpr int kParts = 8 / U;                  // batches per step
     constexpr int kCevPerTeam = TS / 4;            // cev counts chunks of 32 slots; a team owns 8 * TS slots
-    __shared__ int ev_row[kStreamWaves][kStreamEvents + 3];
-    __shared__ float ev_scale[kStreamWaves][kStreamEvents + 3];
+    // per wave: where the sum of every piece that ends in its slots goes.  x, y: address of the target row's first
+    // float (0: nowhere), z: the factor (the row's scale; 1 for a partial sum), w: floats the target row takes
+    // (a partial sum is one table row wide) | bit 16 for a partial sum
+    __shared__ u32x4 ev_list[kStreamWaves][kStreamEvents + 1];
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -120,8 +136,25 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
         if (w == 0 && lane == 0) report_mismatch(fault, 1, generation, header->generation);
         return;
     }
-    int* my_row = ev_row[wave];
-    float* my_scale = ev_scale[wave];
+    u32x4* my_list = ev_list[wave];
+    constexpr unsigned kPartialTarget = 0x10000u;
+    const unsigned ld_floats = ld_bytes / 4u;
+    auto target_of = [&](int r) {
+        unsigned long long a;
+        unsigned factor, floats;
+        if (r < 0) {                                    // never out of range with a well-formed stream
+            const unsigned at = static_cast<unsigned>(r) & 0x7fffffffu;
+            a = at < static_cast<unsigned>(num_partials)
+                    ? reinterpret_cast<unsigned long long>(partial) + static_cast<unsigned long long>(at) * ld_bytes : 0ull;
+            factor = __float_as_uint(1.f);
+            floats = ld_floats | kPartialTarget;
+        } else {
+            a = r < num_nodes ? reinterpret_cast<unsigned long long>(out) + static_cast<unsigned long long>(r) * ld_out * 4ull : 0ull;
+            factor = __float_as_uint(scale[min(r, num_nodes - 1)]);
+            floats = static_cast<unsigned>(width_out);
+        }
+        return u32x4{static_cast<unsigned>(a), static_cast<unsigned>(a >> 32), factor, floats};
+    };
 
     // the wave's 512 slot ids, 8 per lane (streamed once: non-temporal)
     const u32x4* idp = reinterpret_cast<const u32x4*>(scol + static_cast<size_t>(w) * kStreamWave) + lane * 2;
@@ -174,33 +207,27 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     const int ev1 = ce_last & 0x7fffffff;
     {
         const int staged = min(min(ev1, num_events) - ev0, kStreamEvents);
-        for (int j = lane; j < staged; j += kWave) {
-            const int r = erow[ev0 + j];
-            my_row[j] = r;
-            my_scale[j] = r < 0 ? 1.f : scale[min(r, num_nodes - 1)];
-        }
+        for (int j = lane; j < staged; j += kWave) my_list[j] = target_of(erow[ev0 + j]);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
 
-    // a complete piece goes to its row, scaled; anything else to its place among the partial sums
-    auto flush = [&](const float (&a)[4], int target, float s) {
-        if (target < 0) {
-            const int at = target & 0x7fffffff;
-            // the whole pitch is written (lanes past the row's vectors hold zeros): a partial sum then fills its
-            // 64- or 128-byte line and goes to memory without a read-modify-write
-            if (at >= num_partials || tl * 16u >= ld_bytes) return;   // the first never happens with a well-formed stream
-            float* dst = reinterpret_cast<float*>(reinterpret_cast<char*>(partial) + static_cast<size_t>(at) * ld_bytes) + tl * 4;
-            const f32x4 t = {a[0], a[1], a[2], a[3]};
-            __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(dst));
+    // a complete piece goes to its row, scaled; anything else, unscaled (factor 1), to its place among the partial
+    // sums, where the whole pitch is written (lanes past the row's vectors hold zeros): a partial sum then fills its
+    // 64- or 128-byte line and goes to memory without a read-modify-write
+    auto flush = [&](const float (&a)[4], const u32x4& e) {
+        const unsigned long long addr = static_cast<unsigned long long>(e.x) | (static_cast<unsigned long long>(e.y) << 32);
+        if (addr == 0ull) return;
+        float* dst = reinterpret_cast<float*>(addr) + tl * 4;
+        const float f = __uint_as_float(e.z);
+        const float v[4] = {a[0] * f, a[1] * f, a[2] * f, a[3] * f};
+        if constexpr (MODE == kStoreExact) {
+            store_row_floats<kStoreExact>(dst, v, 4);
         } else {
-            if (target >= num_nodes) return;
-            float* dst = out + static_cast<size_t>(target) * ld_out + tl * 4;
-            const float v[4] = {a[0] * s, a[1] * s, a[2] * s, a[3] * s};
-#pragma unroll
-            for (int piece = 0; piece < 4 / OVW; ++piece)
-                if (tl * 4 + piece * OVW < width_out) stream_store<OVW>(dst + piece * OVW, v + piece * OVW);
+            const int n = static_cast<int>(e.w & 0xffffu) - tl * 4;
+            if (e.w & kPartialTarget) store_row_floats<kStoreVec4>(dst, v, n);
+            else store_row_floats<MODE>(dst, v, n);
         }
     };
 
@@ -209,10 +236,8 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     bool had_event = false;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     float head[4] = {0.f, 0.f, 0.f, 0.f};
-    int head_row = 0;
-    float head_scale = 0.f;
-    int next_row = my_row[ev];
-    float next_scale = my_scale[ev];
+    u32x4 head_to = {0u, 0u, 0u, 0u};
+    u32x4 next_to = my_list[ev];
 
     auto consume = [&](const StreamBatch<U>& b) {
 #pragma unroll
@@ -230,18 +255,16 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
                 if (head_pending) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) head[j] = acc[j];
-                    head_row = next_row;
-                    head_scale = next_scale;
+                    head_to = next_to;
                     head_pending = false;
                 } else {
-                    flush(acc, next_row, next_scale);
+                    flush(acc, next_to);
                 }
                 had_event = true;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[j] = 0.f;
                 ev = min(ev + 1, kStreamEvents);
-                next_row = my_row[ev];
-                next_scale = my_scale[ev];
+                next_to = my_list[ev];
             }
         }
     };
@@ -296,10 +319,10 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
     if (ce_team < 0 && had_event) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) head[j] += carry[j];
-        flush(head, head_row, head_scale);
+        flush(head, head_to);
     }
     // the wave's last tail belongs to a piece that ends in a later wave: one more partial sum
-    if (team == TPW - 1 && tail_at >= 0) flush(run, tail_at | static_cast<int>(kStreamFlag), 1.f);
+    if (team == TPW - 1 && tail_at >= 0) flush(run, target_of(tail_at | static_cast<int>(kStreamFlag)));
 }
 
 // Rows with partial sums: out[frow[i], :] = s[frow[i]] * (sum of the partial rows fptr[i] .. fptr[i+1]), summed in
@@ -308,7 +331,7 @@ __global__ __launch_bounds__(kStreamBlock) void aggregate_stream_kernel(
 // partial sums (hub rows cut into column blocks and waves) are then taken one at a time by the whole wave: team t
 // adds the partial sums t, t + TPW, ..., and the teams are summed with cross-lane operations.
 constexpr int kFixTeamMax = 32;
-template <int OVW, int TS>
+template <int MODE, int TS>
 __global__ __launch_bounds__(256) void stream_fixup_kernel(float* __restrict__ out, const float* __restrict__ partial,
                                                            const int* __restrict__ frow, const int* __restrict__ fptr,
                                                            const float* __restrict__ scale, const StreamHeader* header,
@@ -349,10 +372,7 @@ __global__ __launch_bounds__(256) void stream_fixup_kernel(float* __restrict__ o
     };
     auto write_row = [&](const float (&acc)[4], int r, float s) {
         const float v[4] = {acc[0] * s, acc[1] * s, acc[2] * s, acc[3] * s};
-        float* dst = out + static_cast<size_t>(r) * ld_out + tl * 4;
-#pragma unroll
-        for (int piece = 0; piece < 4 / OVW; ++piece)
-            if (tl * 4 + piece * OVW < width_out) stream_store<OVW>(dst + piece * OVW, v + piece * OVW);
+        store_row_floats<MODE>(out + static_cast<size_t>(r) * ld_out + tl * 4, v, width_out - tl * 4);
     };
     for (long long wv = wave0; wv * TPW < num_fix; wv += waves) {
         const long long i = wv * TPW + team;
@@ -456,42 +476,42 @@ int launch_aggregate_stream(float* out, float* partial, const float* table, cons
     if (num_wave_chunks == 0) return kOk;
     const dim3 grid((num_wave_chunks + kStreamWaves - 1) / kStreamWaves), block(kStreamBlock);
     const uintptr_t a = reinterpret_cast<uintptr_t>(out);
-    const int ovw = (dim % 4 == 0 && a % 16 == 0) ? 4 : (dim % 2 == 0 && a % 8 == 0) ? 2 : 1;
+    const int mode = (dim % 4 == 0 && a % 16 == 0) ? ((dim == ts * 4 && ld_in == ts * 4) ? kStoreExact : kStoreVec4) : kStorePlain;
     const int num_fix = info.header.num_fix;
     long long fix_blocks = (static_cast<long long>(num_fix) * ts + 255) / 256;
     if (fix_blocks > 256 * 64) fix_blocks = 256 * 64;
     const dim3 fgrid(static_cast<unsigned>(fix_blocks < 1 ? 1 : fix_blocks));
     int* fault = nullptr;
     if (int rc = plan_fault_address(&fault)) return rc;
-#define EPPGCN_STREAM_KERNEL(OVW_, TS_, WIDE_)                                                                        \
-    hipLaunchKernelGGL((aggregate_stream_kernel<OVW_, TS_, 8, WIDE_>), grid, block, 0, stream, out, partial, table,   \
+#define EPPGCN_STREAM_KERNEL(MODE_, TS_, WIDE_)                                                                        \
+    hipLaunchKernelGGL((aggregate_stream_kernel<MODE_, TS_, 8, WIDE_>), grid, block, 0, stream, out, partial, table,   \
                        scol, sv.erow, sv.cev, sv.wtail, scale, sv.header, fault, info.header.generation,              \
                        num_wave_chunks, info.header.num_events,                                                       \
                        num_nodes, info.header.num_partials, chunks, static_cast<unsigned>(ld_in) * 4u, dim, dim,      \
                        static_cast<unsigned>(bytes), pad_row)
-#define EPPGCN_STREAM(OVW_, TS_)                                                                                      \
+#define EPPGCN_STREAM(MODE_, TS_)                                                                                      \
     do {                                                                                                              \
-        if (wide) EPPGCN_STREAM_KERNEL(OVW_, TS_, true);                                                              \
-        else EPPGCN_STREAM_KERNEL(OVW_, TS_, false);                                                                  \
+        if (wide) EPPGCN_STREAM_KERNEL(MODE_, TS_, true);                                                              \
+        else EPPGCN_STREAM_KERNEL(MODE_, TS_, false);                                                                  \
         if (num_fix > 0)                                                                                              \
-            hipLaunchKernelGGL((stream_fixup_kernel<OVW_, TS_>), fgrid, dim3(256), 0, stream, out, partial, sv.frow,  \
+            hipLaunchKernelGGL((stream_fixup_kernel<MODE_, TS_>), fgrid, dim3(256), 0, stream, out, partial, sv.frow,  \
                                sv.fptr, scale, sv.header, fault, info.header.generation,                              \
                                info.header.num_partials, chunks,                                                      \
                                static_cast<unsigned>(ld_in) * 4u, dim, dim);                                          \
     } while (0)
-#define EPPGCN_STREAM_TS(OVW_)                                                                                        \
+#define EPPGCN_STREAM_TS(MODE_)                                                                                        \
     do {                                                                                                              \
         switch (ts) {                                                                                                 \
-            case 4: EPPGCN_STREAM(OVW_, 4); break;                                                                    \
-            case 8: EPPGCN_STREAM(OVW_, 8); break;                                                                    \
-            case 16: EPPGCN_STREAM(OVW_, 16); break;                                                                  \
-            case 32: EPPGCN_STREAM(OVW_, 32); break;                                                                  \
-            default: EPPGCN_STREAM(OVW_, 64); break;                                                                  \
+            case 4: EPPGCN_STREAM(MODE_, 4); break;                                                                    \
+            case 8: EPPGCN_STREAM(MODE_, 8); break;                                                                    \
+            case 16: EPPGCN_STREAM(MODE_, 16); break;                                                                  \
+            case 32: EPPGCN_STREAM(MODE_, 32); break;                                                                  \
+            default: EPPGCN_STREAM(MODE_, 64); break;                                                                  \
         }                                                                                                             \
     } while (0)
-    if (ovw == 4) EPPGCN_STREAM_TS(4);
-    else if (ovw == 2) EPPGCN_STREAM_TS(2);
-    else EPPGCN_STREAM_TS(1);
+    if (mode == kStoreExact) EPPGCN_STREAM_TS(kStoreExact);
+    else if (mode == kStoreVec4) EPPGCN_STREAM_TS(kStoreVec4);
+    else EPPGCN_STREAM_TS(kStorePlain);
 #undef EPPGCN_STREAM_TS
 #undef EPPGCN_STREAM
 #undef EPPGCN_STREAM_KERNEL
