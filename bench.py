@@ -66,6 +66,10 @@ def parse():
                     help="process the groups in CSR order instead of the column-blocked execution plan")
     ap.add_argument("--no_stream", action="store_true",
                     help="keep planned launches on the group kernel instead of the plan's stream form")
+    ap.add_argument("--degree_order", action="store_true",
+                    help="renumber the vertices of the synthetic graph by descending degree inside blocks of 2^17 ids "
+                         "before anything else (graphs.degree_order: what a caller who may choose its numbering gains; "
+                         "NOT the benchmark's graph numbering, so not a headline figure - config.degree_order says so)")
     ap.add_argument("--wide_stream", action="store_true",
                     help="force the stream kernel's 64-bit addressing variant (it otherwise runs for tables of 4 GB and more)")
     ap.add_argument("--no_workspace", action="store_true",
@@ -167,6 +171,8 @@ def main():
 
     t0 = time.perf_counter()
     g = graphs.make_graph(args.config, device=dev)
+    if args.degree_order:
+        g = graphs.renumber(g, graphs.degree_order(g))
     torch.cuda.synchronize()
     log(args, "graph", g.stats(), f"{time.perf_counter() - t0:.1f}s")
     if args.no_stream:
@@ -347,7 +353,7 @@ def main():
                    "backward_group_size": [p.part_size for p in wl.paths],
                    "kept_edges": [p.valid_len for p in wl.paths],
                    "backward_groups": [p.num_parts for p in wl.paths], "max_degree": g.stats()["max_degree"],
-                   "feature_workspace": not args.no_workspace,
+                   "feature_workspace": not args.no_workspace, "degree_order": bool(args.degree_order),
                    "column_blocked_plan": bool(wl.plans),
                    "stream_form": all(k["stream_form"] for k in per_kernel.values()),
                    "partial_sum_rows": {"fwd_agg_d16": getattr(wl.plans.get(16), "partial_rows", 0),

@@ -36,6 +36,7 @@
 // use float atomics, once per wave instead of once per group.
 // Precondition: the groups of one row are consecutive (build_part and the path
 // splitter produce them that way).
+#include <atomic>
 #include <type_traits>
 
 #include "common.hpp"
@@ -538,13 +539,13 @@ __global__ __launch_bounds__(kAggBlock) void aggregate_kernel(
 }
 
 // ---------------------------------------------------------------- dispatch
-struct AggTuning {
-    int force_team = 0;      // 0 = automatic; otherwise lanes per team (power of two, 4..64)
-    int force_rounds = 0;    // 0 = automatic; otherwise rounds per wave
+struct AggTuning {            // process-wide knobs (tuning header)
+    std::atomic<int> force_team{0};      // 0 = automatic; otherwise lanes per team (power of two, 4..64)
+    std::atomic<int> force_rounds{0};    // 0 = automatic; otherwise rounds per wave
 };
 static AggTuning g_tuning;
-void set_agg_force_team(int ts) { g_tuning.force_team = ts; }
-void set_agg_force_rounds(int r) { g_tuning.force_rounds = r; }
+void set_agg_force_team(int ts) { g_tuning.force_team.store(ts); }
+void set_agg_force_rounds(int r) { g_tuning.force_rounds.store(r); }
 constexpr int kEdgesPerWave = 800;
 constexpr int kGroupsPerWave = 64;
 constexpr int kMinWaves = 256 * 24 * 4;
@@ -569,7 +570,7 @@ static hipError_t launch_one(float* out, const float* in, const int* col, const 
     // when a round holds fewer than 16 (measured at R-MAT scale 22 with execution plans: width 16, 16
     // groups a round, 1 / 2 / 4 / 8 rounds -> 1.36 / 1.32 / 1.35 / 1.45 ms; width 22, 8 groups a round, gains 9 % from 8 rounds
     // because a long row is then flushed once per 64 groups instead of once per 8)
-    int rounds = g_tuning.force_rounds;
+    int rounds = g_tuning.force_rounds.load();
     if (rounds <= 0) {
         const int per_round = TPW * (sh.group_size > 0 ? sh.group_size : 1);
         rounds = (kEdgesPerWave + per_round - 1) / per_round;
@@ -597,7 +598,7 @@ static hipError_t launch_slab(float* out, const float* in, const int* col, const
     const int chunks = sh.chunks;
     int ts = 4;
     while (ts < 64 && ts < chunks) ts <<= 1;
-    const int ft = g_tuning.force_team;
+    const int ft = g_tuning.force_team.load();
     if (ft >= 4 && ft <= 64 && (ft & (ft - 1)) == 0 && chunks <= ft) ts = ft;   // only wider teams can be forced
     const int cpl = (chunks + ts - 1) / ts;
 #define EPPGCN_LAUNCH(TS_, CPL_, U_) \

@@ -2,6 +2,7 @@
 // host halves (count read-back, heuristics) of the aggregation path.
 #include "../../include/eppgcn_hip_tuning.h"
 
+#include <atomic>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -63,13 +64,13 @@ int hip_fail(hipError_t e, const char* what)
 
 // ---- timers (milliseconds)
 constexpr int kMaxTimedLayers = 16;
-static bool g_timing = false;
+static std::atomic<bool> g_timing{false};
 static double g_for_agg_ms = 0.0, g_back_agg_ms = 0.0, g_mask_ms = 0.0;
 static double g_layer_back_ms[kMaxTimedLayers] = {0};
 
 static double g_phase_ms[2] = {0.0, 0.0};       // output clears, pre-scaling passes of the aggregation calls
 
-bool timing_enabled() { return g_timing; }
+bool timing_enabled() { return g_timing.load(); }
 double* phase_sink(int which) { return &g_phase_ms[which & 1]; }
 
 static int read_state(void* workspace, hipStream_t stream, ScanState* host)
@@ -490,7 +491,7 @@ int eppgcn_get_ginfo(const int32_t* node_deg, int64_t num_nodes, int64_t valid_l
     return kOk;
 }
 
-void eppgcn_set_timing(int enabled) { g_timing = enabled != 0; }
+void eppgcn_set_timing(int enabled) { g_timing.store(enabled != 0); }
 
 void eppgcn_print_time(void)
 {

@@ -13,6 +13,7 @@
 // per step, until it meets a tile whose inclusive prefix is known.  Lane ranks
 // inside a wave come from a 64-bit ballot and mbcnt; no block-wide bit-sliced
 // counting and no second pass over the input.
+#include <atomic>
 #include <mutex>
 
 #include "common.hpp"
@@ -44,11 +45,11 @@ __global__ void scan_init_kernel(ScanState* st, uint64_t* desc, int num_tiles)
 
 // Test knob for the stall path: with tile 0 muted every look-back runs into its (then tiny) spin limit,
 // raises the error flag and carries on, so the kernels still drain and the host sees EPPGCN_ERR_SCAN_STALLED.
-static unsigned g_scan_mode = 0;
-unsigned scan_mode() { return g_scan_mode; }
+static std::atomic<unsigned> g_scan_mode{0};     // process-wide test knob (tuning header)
+unsigned scan_mode() { return g_scan_mode.load(); }
 void set_scan_test_mode(unsigned spin_limit, int mute_first_tile)
 {
-    g_scan_mode = (spin_limit & 0x7fffffffu) | (mute_first_tile ? 0x80000000u : 0u);
+    g_scan_mode.store((spin_limit & 0x7fffffffu) | (mute_first_tile ? 0x80000000u : 0u));
 }
 
 // ================================================================ path marking
@@ -655,9 +656,9 @@ __global__ __launch_bounds__(256) void zero_listed_rows_kernel(float* __restrict
     }
 }
 
-static bool g_force_wide_index = false;
-bool force_wide_index() { return g_force_wide_index; }
-void set_force_wide_index(bool on) { g_force_wide_index = on; }
+static std::atomic<bool> g_force_wide_index{false};
+bool force_wide_index() { return g_force_wide_index.load(); }
+void set_force_wide_index(bool on) { g_force_wide_index.store(on); }
 
 int launch_zero_rows_unless(float* out, const uint32_t* skip, long long num_rows, int dim, hipStream_t stream)
 {

@@ -478,7 +478,7 @@ static size_t plan_sort_state_offset(long long num_parts, long long num_slots)
 
 int workspace_pitch(int dim);   // aggregate.hip
 
-static int g_force_shift = 0;
+static std::atomic<int> g_force_shift{0};     // process-wide knobs (tuning header), atomics like the ones below
 // Plan policy.  Rows of up to 32 * keep slots are kept together instead of being cut at column-block borders, and
 // single-group rows may be ordered by length class inside a block.  Negative = chosen per build from the kernel that
 // will run over the plan:
@@ -489,22 +489,23 @@ static int g_force_shift = 0;
 //  * group kernel (runs over a plan when the shape is outside the stream kernel's: table of 4 GB or more, rows beyond
 //    1024 bytes, stream mode off): equal gather steps per round matter, 256 slots with classes is its optimum and the
 //    stream policy costs it 10 % (5.11 against 4.66 ms at R-MAT 22; 22.6 against 20.6 ms at R-MAT 24): keep 8, classes.
-static int g_keep_rows = -1;         // in units of 32 slots
-static int g_length_classes = -1;
-void set_plan_length_classes(int on) { g_length_classes = on < 0 ? -1 : on ? 1 : 0; }
-void set_plan_keep_rows(int keep) { g_keep_rows = keep < 0 ? -1 : keep; }
+static std::atomic<int> g_keep_rows{-1};         // in units of 32 slots
+static std::atomic<int> g_length_classes{-1};
+void set_plan_length_classes(int on) { g_length_classes.store(on < 0 ? -1 : on ? 1 : 0); }
+void set_plan_keep_rows(int keep) { g_keep_rows.store(keep < 0 ? -1 : keep); }
 bool stream_covers(int num_nodes, int dim, int ld_in, const float* table);   // stream.hip
 static void plan_policy(int num_nodes, int dim, int* keep_rows, int* length_classes)
 {
     const bool stream = stream_covers(num_nodes, dim, workspace_pitch(dim), nullptr);
-    *keep_rows = g_keep_rows >= 0 ? g_keep_rows : stream ? 2 : 8;
-    *length_classes = g_length_classes >= 0 ? g_length_classes : stream ? 0 : 1;
+    const int keep = g_keep_rows.load(), classes = g_length_classes.load();
+    *keep_rows = keep >= 0 ? keep : stream ? 2 : 8;
+    *length_classes = classes >= 0 ? classes : stream ? 0 : 1;
 }
-void set_schedule_shift(int shift) { g_force_shift = shift; }
+void set_schedule_shift(int shift) { g_force_shift.store(shift); }
 
 int schedule_shift(int dim)
 {
-    if (g_force_shift > 0) return g_force_shift;
+    if (const int forced = g_force_shift.load(); forced > 0) return forced;
     // column blocks of at most 128K rows and 16 MB of feature rows.  Measured at R-MAT scale 22
     // (ms per epoch, 64- and 128-byte rows): 2^14 5.95, 2^15 5.74, 2^16 5.63, 2^17 5.60, 2^18 5.65,
     // 2^19 5.83 - the window all waves gather from has to stay resident in the memory-side cache,

@@ -406,6 +406,7 @@ __global__ __launch_bounds__(256) void stream_fixup_kernel(float* __restrict__ o
 static __device__ __align__(16) int plan_fault_words[kPlanFaultWords];
 }  // namespace eppgcn
 
+#include <atomic>
 #include <map>
 #include <mutex>
 
@@ -428,9 +429,10 @@ int plan_fault_address(int** words)
     return kOk;
 }
 
-static int g_stream_mode = 1;
-static bool g_force_wide_stream = false;     // tests: the 64-bit addressing variant at any size
-void set_stream_mode(int on) { g_stream_mode = on ? 1 : 0; g_force_wide_stream = on == 2; }
+// process-wide knobs (tuning header): atomics, so that a setter racing with a call is at least not a data race
+static std::atomic<int> g_stream_mode{1};
+static std::atomic<bool> g_force_wide_stream{false};     // tests: the 64-bit addressing variant at any size
+void set_stream_mode(int on) { g_stream_mode.store(on ? 1 : 0); g_force_wide_stream.store(on == 2); }
 
 // Team size for rows of `chunks` 16-byte vectors, 0 when the stream kernel does not cover the shape.
 static int stream_team(int chunks)
@@ -454,7 +456,7 @@ static bool stream_needs_wide(int num_nodes, int dim, int ld_in)
 // Can a launch over a pre-scaled table with rows of ld_in floats run through the stream kernel?
 bool stream_covers(int num_nodes, int dim, int ld_in, const float* table)
 {
-    if (!g_stream_mode || force_wide_index()) return false;
+    if (!g_stream_mode.load() || force_wide_index()) return false;
     if (ld_in % 4 != 0 || reinterpret_cast<uintptr_t>(table) % 16 != 0) return false;
     if (stream_team((dim + 3) / 4) == 0 || (dim + 3) / 4 * 4 > ld_in) return false;
     return swizzle_padded_rows(num_nodes) < (1ll << 31);
@@ -469,7 +471,7 @@ int launch_aggregate_stream(float* out, float* partial, const float* table, cons
     const int chunks = (dim + 3) / 4;
     const int ts = stream_team(chunks);
     const long long padded = stream_padded_slots(info.num_slots);
-    const bool wide = stream_needs_wide(num_nodes, dim, ld_in) || g_force_wide_stream;
+    const bool wide = stream_needs_wide(num_nodes, dim, ld_in) || g_force_wide_stream.load();
     const unsigned long long bytes = wide ? 0ull : static_cast<unsigned long long>(swizzle_padded_rows(num_nodes)) * ld_in * 4ull;
     const unsigned pad_row = static_cast<unsigned>(swizzle_padded_rows(num_nodes));
     const int num_wave_chunks = static_cast<int>(padded / kStreamWave);

@@ -78,11 +78,16 @@ def write_train_mask(data_path: str, ratio: float, mask) -> str:
 
 class custom_dataset(torch.nn.Module):
     """Same constructor arguments and attributes as the reference's class; ``device``,
-    ``scale_mode``, ``feature_seed`` and ``train_mask`` are additions (a mask tensor given here
-    replaces the mask file)."""
+    ``scale_mode``, ``feature_seed``, ``train_mask`` and ``degree_order`` are additions (a mask tensor
+    given here replaces the mask file).
+
+    ``degree_order=True`` renumbers the vertices after loading (``graphs.degree_order``: descending degree
+    inside blocks of 2^17 ids, which the aggregation kernels reward with a few per cent); ``new_id`` then
+    holds the new id of every vertex of the files, and the mask, the features and the labels are stored
+    under the new ids.  Results for vertex v of the files are at row ``new_id[v]``."""
 
     def __init__(self, path, dataPath, ratio, dim, num_class, num_layer, load_from_txt=True, verbose=False,
-                 device="cuda", scale_mode="sqrt", feature_seed=None, train_mask=None):
+                 device="cuda", scale_mode="sqrt", feature_seed=None, train_mask=None, degree_order=False):
         super().__init__()
         if not load_from_txt and not path.endswith(".npz"):
             raise ValueError("graph file must be a .npz file")
@@ -111,6 +116,17 @@ class custom_dataset(torch.nn.Module):
         self.train_mask = train_mask.to(device=device, dtype=torch.bool)
         if self.train_mask.numel() != n:
             raise ValueError("train_mask must have one entry per vertex")
+        self.new_id = None
+        if degree_order:
+            g = self.graph()
+            self.new_id = graphs.degree_order(g)
+            g = graphs.renumber(g, self.new_id)
+            self.row_pointers, self.column_index, self.degrees = g.row_pointers, g.column_index, g.degrees
+            for name in ("x", "y", "train_mask"):
+                old = getattr(self, name)
+                moved = torch.empty_like(old)
+                moved[self.new_id] = old
+                setattr(self, name, moved)
         self._init_masks(device)
 
     def _init_masks(self, device):

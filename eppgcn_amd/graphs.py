@@ -146,6 +146,46 @@ def csr_from_pairs(name: str, src: torch.Tensor, dst: torch.Tensor, num_nodes: i
     return Graph(name, n, indptr, cols, scale_vector(indptr, scale_mode))
 
 
+def degree_order(graph: Graph, block_shift: int = 17) -> torch.Tensor:
+    """new_id int64[N]: a renumbering of the vertices in which, inside every aligned block of
+    2^block_shift ids, the vertices come in order of descending degree (ties: old order).  Vertices stay
+    in their block, so anything that depends on the coarse position of an id is unchanged.
+
+    Why a caller may want it: the aggregation kernels gather feature rows by vertex id; with the rows of
+    one block ordered by degree the hot 64-byte rows share 128-byte lines and the rows are processed and
+    written in an order that follows their length (forward aggregation of an R-MAT scale-22 graph on an
+    MI355X: -3.7 % at width 16, -3.1 % at width 22).  The numbering of the vertices is the caller's, so
+    this is offered to the caller and never applied behind its back."""
+    n = graph.num_nodes
+    dev = graph.row_pointers.device
+    deg = (graph.row_pointers[1:] - graph.row_pointers[:-1]).to(torch.int64)
+    ident = torch.arange(n, dtype=torch.int64, device=dev)
+    order = torch.argsort((ident >> block_shift) * (1 << 32) + ((1 << 31) - deg), stable=True)
+    new_id = torch.empty(n, dtype=torch.int64, device=dev)
+    new_id[order] = ident
+    return new_id
+
+
+def renumber(graph: Graph, new_id: torch.Tensor) -> Graph:
+    """The same graph with vertex v called new_id[v] (a permutation of 0..N-1): row new_id[r] holds the
+    columns new_id[c] of the old row r, ascending; the scale vector moves with the vertices.  Per-vertex
+    data of the caller moves the same way: ``x_new[new_id] = x_old``."""
+    n = graph.num_nodes
+    new_id = new_id.to(torch.int64)
+    deg = (graph.row_pointers[1:] - graph.row_pointers[:-1]).to(torch.int64)
+    rows = torch.repeat_interleave(torch.arange(n, device=new_id.device), deg)
+    keys = torch.sort(new_id[rows] * n + new_id[graph.column_index.long()]).values
+    del rows
+    r = keys // n
+    cols = (keys - r * n).to(torch.int32)
+    del keys
+    indptr = torch.zeros(n + 1, dtype=torch.int64, device=new_id.device)
+    torch.cumsum(torch.bincount(r, minlength=n), 0, out=indptr[1:])
+    degrees = torch.empty_like(graph.degrees)
+    degrees[new_id] = graph.degrees
+    return Graph(graph.name + "_renumbered", n, indptr.to(torch.int32), cols, degrees)
+
+
 def _first_distinct_pairs(seed: int, n: int, want: int, draw, device) -> tuple:
     """First ``want`` distinct unordered non-loop pairs in draw order."""
     total = 0

@@ -2,9 +2,9 @@
  * Tuning and test knobs of libeppgcn_hip.so.  Not part of the drop-in surface: nothing in the
  * reference corresponds to them, and a product build never needs to call any of them.
  *
- * Every setter here writes a PROCESS-WIDE value without synchronisation: it changes the launches of
- * every thread of the process from the next call on, and it must not run concurrently with a call
- * into the library.  They exist for benchmark sweeps and for tests that have to reach code paths a
+ * Every setter here writes a PROCESS-WIDE value (an atomic word, so a setter that races with a call is
+ * not a data race - but the call may see either value): it changes the launches of every thread of the
+ * process from the next call on, so set them before the calls they are meant for, from one place.  They exist for benchmark sweeps and for tests that have to reach code paths a
  * small input would not (64-bit indexing, a stalled look-back, the group kernel over a plan).
  */
 #ifndef EPPGCN_HIP_TUNING_H_

@@ -73,3 +73,34 @@ def test_inv_sqrt_scale_mode(tmp_path):
     assert np.allclose(d.degrees.numpy(), [2 ** -0.5, 2 ** -0.5, 1.0])
     assert torch.equal(d.x, ds.custom_dataset(str(tmp_path / "e.txt"), str(tmp_path), 0.5, 4, 2, 2, device="cpu",
                                                train_mask=torch.tensor([True, False, True]), feature_seed=7).x)
+
+
+def test_degree_order_is_a_block_preserving_permutation_and_renumbering_keeps_the_graph():
+    """``graphs.degree_order`` / ``graphs.renumber`` (CPU tensors): a permutation that keeps every vertex in
+    its block of ids and orders the block by descending degree; the renumbered CSR is the same edge set under
+    the new names, rows ascending, and the scale vector moves with the vertices."""
+    import numpy as np
+    import torch
+    from eppgcn_amd import graphs
+    g = graphs.chung_lu_graph(3000, 9000, 2.1, 5)
+    new_id = graphs.degree_order(g, block_shift=9)
+    n = g.num_nodes
+    assert sorted(new_id.tolist()) == list(range(n))
+    ident = torch.arange(n)
+    assert torch.equal(new_id >> 9, ident >> 9)
+    deg = (g.row_pointers[1:] - g.row_pointers[:-1]).long()
+    by_new = torch.empty(n, dtype=torch.long)
+    by_new[new_id] = deg
+    for lo in range(0, n, 512):
+        block = by_new[lo:lo + 512]
+        assert bool((block[:-1] >= block[1:]).all())
+    h = graphs.renumber(g, new_id)
+    assert h.num_edges == g.num_edges and h.num_nodes == n
+    rows = torch.repeat_interleave(ident, deg)
+    old_pairs = set(zip(new_id[rows].tolist(), new_id[g.column_index.long()].tolist()))
+    hrows = torch.repeat_interleave(ident, (h.row_pointers[1:] - h.row_pointers[:-1]).long())
+    assert set(zip(hrows.tolist(), h.column_index.tolist())) == old_pairs
+    cols = h.column_index.numpy()
+    ptr = h.row_pointers.numpy()
+    assert all(np.all(np.diff(cols[ptr[r]:ptr[r + 1]]) > 0) for r in range(n))
+    assert torch.equal(h.degrees[new_id], g.degrees)

@@ -317,6 +317,35 @@ def test_training_from_a_dataset_file(GNNA, tmp_path):
     assert np.linalg.norm(tr.model.convs[1].weights.grad.cpu().numpy() - want_g1) / np.linalg.norm(want_g1) < 1e-4
 
 
+def test_dataset_in_degree_order_trains_the_same_model(GNNA, tmp_path):
+    """``custom_dataset(degree_order=True)``: the vertices are renumbered after loading (features, labels and mask
+    move with them), so the loss and the weight gradients are those of the files' numbering up to rounding, and
+    the output rows are the old ones at ``new_id``."""
+    from eppgcn_amd import dataset as dsmod, train
+    indptr, col = random_symmetric_csr(900, 4000, 33)
+    n = indptr.size - 1
+    rows = np.repeat(np.arange(n), np.diff(indptr))
+    np.savez(str(tmp_path / "g.npz"), src_li=rows, dst_li=col, num_nodes=n)
+    mask = np.random.default_rng(10).random(n) < 0.2
+    dsmod.write_train_mask(str(tmp_path), 0.2, mask)
+    runs = []
+    for order in (False, True):
+        d = dsmod.custom_dataset(str(tmp_path / "g.npz"), str(tmp_path), 0.2, 12, 7, 2, load_from_txt=False,
+                                 scale_mode="inv_sqrt", feature_seed=5, degree_order=order)
+        tr = train.Trainer(None, hidden=16, dataset=d, backsize=4, weight_seed=3)
+        tr.optimizer = torch.optim.SGD(tr.model.parameters(), lr=0.0)
+        loss = float(tr.train_step(True))
+        out = tr.model(d.x, tr.inputInfo, tr.mask_props, tr.back_props, False, False).detach()
+        runs.append((d, loss, [c.weights.grad.cpu().numpy().copy() for c in tr.model.convs], out))
+        GNNA.clear_plans()
+    (d0, l0, g0, o0), (d1, l1, g1, o1) = runs
+    assert d0.new_id is None and sorted(d1.new_id.tolist()) == list(range(n))
+    assert abs(l0 - l1) <= 1e-5 * max(1.0, abs(l0))
+    for a, b in zip(g0, g1):
+        assert np.linalg.norm(a - b) <= 1e-4 * np.linalg.norm(a) + 1e-12
+    assert torch.allclose(o1[d1.new_id], o0, rtol=1e-4, atol=1e-5)
+
+
 def test_driver_command_line_end_to_end(GNNA, tmp_path, capsys):
     """`python -m eppgcn_amd.gcn_main` with the reference's flags on reference-format files: the
     report carries the reference's lines (EPPGCN/gcn_main.py:286-291), --verify_spmm passes, a
