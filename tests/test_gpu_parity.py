@@ -745,6 +745,61 @@ def test_rmat20_linearity_and_tolerance(api, rmat20):
         assert worst <= 1.0, f"D={dim}: max err/limit {worst:.3f}"
 
 
+def test_rmat20_against_the_reference_order_restatement(api, rmat20):
+    """R-MAT 20 at its own size against the checker's fp32 restatement of the reference's loops (one group after the
+    other, `w = fl(s_r s_c)`, the reference's roundings per term; EPPGCN_kernel.cu:263-293, :642-668), not only
+    against a float64 sum: forward at both widths through the path without workspace (the reference's rounding
+    model, groups in CSR order) and through the benchmark's path (plan, pre-scaled table, stream form); pruned
+    backward over a 10 % mask both ways.  What remains is the order in which the groups of a row are combined and,
+    on the pre-scaled path, one rounding more per term and one less per row: 2e-5 of the absolute sum."""
+    from eppgcn_amd import graphs
+    g = rmat20
+    n, e = g.num_nodes, g.num_edges
+    ps = max(16, int(g.avg_degree))
+    pp, p2n = api.build_part(ps, g.row_pointers, e)
+    col_h, s_h = g.column_index.cpu().numpy(), g.degrees.cpu().numpy()
+    pp_h, p2n_h = pp.cpu().numpy(), p2n.cpu().numpy()
+    row = g.row_index()
+    w_abs = (g.degrees[row] * g.degrees[g.column_index.long()]).abs()
+
+    def bound_of(x):
+        return torch.zeros(n, x.shape[1], device="cuda").index_add_(0, row, w_abs[:, None] * x[g.column_index.long()].abs())
+
+    def check(got, want_h, bound, what):
+        worst = ((got - torch.from_numpy(want_h).cuda()).abs() / (2e-5 * bound + 1e-30)).max().item()
+        assert worst <= 1.0, f"{what}: max err/limit {worst:.3f}"
+
+    plan = api.build_plan(pp, g.column_index, p2n.numel(), e, n, 22, part2node=p2n)
+    for dim in (16, 22):
+        x = graphs.normal32(1, (n, dim), "cuda", dim)
+        want = co.spmm_groups(x.cpu().numpy(), col_h, s_h, pp_h, p2n_h, n, threads=True)
+        bound = bound_of(x)
+        check(api.spmm_forward(x, g.column_index, g.degrees, pp, p2n, part_size=ps, workspace=None), want, bound,
+              f"forward D={dim}, reference rounding model")
+        ws = api.feature_workspace(n, dim, "cuda", plan)
+        check(api.spmm_forward(x, g.column_index, g.degrees, pp, p2n, part_size=ps, workspace=ws, plan=plan), want, bound,
+              f"forward D={dim}, benchmark path")
+        assert api.last_call_used_stream()
+    # pruned backward over the last layer's path of a 10 % mask
+    mask = graphs.bernoulli_mask(n, 0.1, 2, "cuda")
+    bem = torch.full((e,), -1, dtype=torch.int32, device="cuda")
+    degs = torch.zeros(n, dtype=torch.int32, device="cuda")
+    api.mask_forward(p2n, pp, g.column_index, mask, None, bem, degs, True)
+    ids, edge_list, v = api.compact_back_edge(bem, g.column_index)
+    part_pointer, num_parts, _ = api.split_back_part(degs, e, 32)
+    dy = graphs.normal32(5, (n, 22), "cuda") * mask[:, None]
+    want = co.ours_backward(dy.cpu().numpy(), ids.cpu().numpy(), part_pointer.cpu().numpy(), edge_list.cpu().numpy(), s_h,
+                            num_parts, threads=True)
+    bound = bound_of(dy)
+    check(api.ours_backward(dy, ids, part_pointer, edge_list, g.degrees, num_parts, 32, workspace=None), want, bound,
+          "pruned backward, reference rounding model")
+    path_plan = api.build_plan(part_pointer, edge_list, num_parts, v, n, 22, ids=ids, block_shift=31)
+    ws = api.feature_workspace(n, 22, "cuda", path_plan)
+    check(api.ours_backward(dy, ids, part_pointer, edge_list, g.degrees, num_parts, 32, 1, 4, 16, None, ws, plan=path_plan),
+          want, bound, "pruned backward, benchmark path")
+    assert api.last_call_used_stream()
+
+
 # ----------------------------------------------------------------------------- fused marking + compaction
 @pytest.mark.parametrize("name", list(GRAPHS))
 @pytest.mark.parametrize("ratio", [0.0, 0.1, 0.6, 1.0])
