@@ -30,9 +30,10 @@ EXPORTS = [
     "eppgcn_auto_back_part_size", "eppgcn_scan_status", "eppgcn_plan_status", "eppgcn_set_scan_test_mode",
     "eppgcn_plan_workspace_floats", "eppgcn_set_stream_mode", "eppgcn_last_call_used_stream",
     "eppgcn_update_forward_table", "eppgcn_feature_workspace_row", "eppgcn_plan_release", "eppgcn_aggregation_status",
+    "eppgcn_ours_backward_rows", "eppgcn_update_backward_rows",
 ]
 
-ABI_VERSION = 15      # what eppgcn_abi_version() of a matching library returns
+ABI_VERSION = 16      # what eppgcn_abi_version() of a matching library returns
 
 _lib = None
 
@@ -141,8 +142,12 @@ def load():
     lib.eppgcn_update_workspace_bytes.restype = sz
     lib.eppgcn_update_backward_weight.argtypes = [p, p, p, i, i64, i, i, p, sz, p]
     lib.eppgcn_update_backward.argtypes = [p, p, p, p, p, i, i64, i, i, p, sz, p]
+    lib.eppgcn_update_backward_rows.argtypes = [p, p, p, p, p, i, p, i64, i, i, p, sz, p]
+    lib.eppgcn_ours_backward_rows.argtypes = [p, p, p, p, p, p, i, i, i, i, i, i, i, p, sz, p, p,
+                                              C.POINTER(C.c_void_p), C.POINTER(i64), p]
+    lib.eppgcn_ours_backward_rows.restype = i
     for name in ("eppgcn_update_forward", "eppgcn_update_backward_input", "eppgcn_update_backward_weight",
-                 "eppgcn_update_backward"):
+                 "eppgcn_update_backward", "eppgcn_update_backward_rows"):
         getattr(lib, name).restype = i
     for name in ("eppgcn_spmm_forward", "eppgcn_spmm_backward", "eppgcn_ours_backward", "eppgcn_mask_forward",
                  "eppgcn_compact_back_edge", "eppgcn_count_nonzero", "eppgcn_map_back_part_size",
@@ -290,6 +295,37 @@ def update_backward(x, w, g, relu_input=False):
     ws = torch.empty(max(1, (nbytes + 3) // 4), dtype=torch.float32, device=x.device)
     _check(lib.eppgcn_update_backward(_ptr(d_x), _ptr(d_w), _ptr(x), _ptr(g), _ptr(w), int(bool(relu_input)), n, k, m,
                                       _ptr(ws), nbytes, _stream()))
+    return d_x, d_w
+
+
+def update_backward_rows(x, w, g, rows, relu_input=False, need_dx=True):
+    """``update_backward`` for a gradient ``g`` of which only the rows with a set bit in ``rows`` are defined (a
+    device int32 bitmap, bit r of word r // 32, or the device address ``ours_backward_rows`` returns, or None for
+    all rows): the other rows count as zeros and are not read, nor are their rows of ``x``.
+    -> (d_x [N, in_dim] or None when ``need_dx`` is false, d_w [in_dim, out_dim])."""
+    lib = load()
+    _dev(x, torch.float32, "x"); _dev(g, torch.float32, "g")
+    n, k = x.shape
+    m = g.shape[1]
+    if g.shape[0] != n:
+        raise EppgcnError("x and g must have the same number of rows")
+    if need_dx:
+        _dev(w, torch.float32, "w")
+        if tuple(w.shape) != (k, m):
+            raise EppgcnError("w must be [in_dim, out_dim]")
+    if isinstance(rows, torch.Tensor):
+        _dev(rows, torch.int32, "rows")
+        if rows.numel() < (n + 31) // 32:
+            raise EppgcnError("the row bitmap needs (N + 31) // 32 words")
+        rows_ptr = _ptr(rows)
+    else:
+        rows_ptr = C.c_void_p(rows) if rows else None
+    d_x = torch.empty((n, k), dtype=torch.float32, device=x.device) if need_dx else None
+    d_w = torch.empty((k, m), dtype=torch.float32, device=x.device)
+    nbytes = lib.eppgcn_update_workspace_bytes(n, k, m)
+    ws = torch.empty(max(1, (nbytes + 3) // 4), dtype=torch.float32, device=x.device)
+    _check(lib.eppgcn_update_backward_rows(_ptr(d_x), _ptr(d_w), _ptr(x), _ptr(g), _ptr(w) if need_dx else None,
+                                           int(bool(relu_input)), rows_ptr, n, k, m, _ptr(ws), nbytes, _stream()))
     return d_x, d_w
 
 
@@ -510,6 +546,30 @@ def ours_backward(d_output, ids, part_pointer, edge_list, degrees, num_parts, pa
                                     _ptr(ws), 0 if ws is None else ws.numel(),
                                     _plan_ptr(plan, int(num_parts), n), _ptr(gathered_rows), _stream()))
     return out
+
+
+def ours_backward_rows(d_output, ids, part_pointer, edge_list, degrees, num_parts, part_size=32, layer=1,
+                       blockx=4, blocky=16, out=None, workspace=True, plan=None, gathered_rows=None):
+    """``ours_backward`` that leaves the rows without groups as they are when it runs a plan's stream form.
+    -> (out, rows, num_written): ``rows`` is the device address of the bitmap of the written rows (inside the
+    plan; pass it to ``update_backward_rows``), or None when every row of ``out`` is defined."""
+    lib = load()
+    _dev(d_output, torch.float32, "d_output"); _dev(ids, torch.int32, "ids")
+    _dev(part_pointer, torch.int32, "part_pointer"); _dev(edge_list, torch.int32, "edge_list")
+    _dev(degrees, torch.float32, "degrees")
+    n, dim = d_output.shape
+    if part_pointer.numel() < num_parts + 1:
+        raise EppgcnError("part_pointer needs num_parts + 1 entries")
+    if out is None:
+        out = torch.empty_like(d_output)
+    ws = _feature_workspace(workspace, d_output, plan)
+    rows, count = C.c_void_p(), C.c_int64()
+    _check(lib.eppgcn_ours_backward_rows(_ptr(out), _ptr(d_output), _ptr(ids), _ptr(part_pointer), _ptr(edge_list),
+                                         _ptr(degrees), n, dim, int(num_parts), part_size, layer, blockx, blocky,
+                                         _ptr(ws), 0 if ws is None else ws.numel(),
+                                         _plan_ptr(plan, int(num_parts), n), _ptr(gathered_rows),
+                                         C.byref(rows), C.byref(count), _stream()))
+    return out, rows.value, count.value
 
 
 # --------------------------------------------------------------------------- preparation

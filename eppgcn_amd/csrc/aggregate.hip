@@ -780,15 +780,22 @@ static bool stream_usable(const StreamInfo* info, const float* in, const float* 
 static thread_local int g_last_used_stream = 0;
 int last_call_used_stream() { return g_last_used_stream; }
 
+// written: nullptr, or where the caller wants the bitmap of the rows this call writes (one bit per vertex, inside the
+// plan); the rows without any slot are then left as they are instead of being cleared, and *count is their complement.
 static int aggregate_stream_call(float* out, const float* in, const int* scol, const float* scale, const StreamInfo& info,
                                  const void* plan, int num_nodes, int dim, float* workspace, hipStream_t stream,
-                                 double* sink, double* sink2, const uint32_t* gathered_rows)
+                                 double* sink, double* sink2, const uint32_t* gathered_rows,
+                                 const uint32_t** written = nullptr, long long* count = nullptr)
 {
     const StreamView sv = stream_view(const_cast<void*>(plan), info.num_parts, info.num_slots, info.num_nodes);
     const int ld = workspace_pitch(dim);
     g_last_used_stream = 1;
+    if (written) {
+        *written = sv.touched;
+        if (count) *count = static_cast<long long>(num_nodes) - info.header.empty_rows;
+    }
     // only rows without any slot are left to a clear: every other row is written by the stream kernel or the fix-up
-    if (info.header.empty_rows > 0) {
+    if (info.header.empty_rows > 0 && !written) {
         KernelTimer timer(stream, phase_sink(0));
         if (2ll * info.header.empty_rows <= num_nodes) {
             if (int rc = launch_zero_rows_unless(out, sv.touched, num_nodes, dim, stream)) return rc;
@@ -897,14 +904,16 @@ int aggregate_forward_groups(float* out, const float* in, const int* col, const 
 int aggregate_compacted_groups(float* out, const float* in, const int* ids, const int* part_ptr,
                                const int* edge_list, const float* scale, const void* plan, int num_nodes, int dim,
                                int num_parts, int group_size, float* workspace, size_t workspace_floats,
-                               const uint32_t* gathered_rows, hipStream_t stream, double* sink, double* sink2)
+                               const uint32_t* gathered_rows, hipStream_t stream, double* sink, double* sink2,
+                               const uint32_t** written, long long* num_written)
 {
+    if (written) *written = nullptr;        // unless the stream form runs, every row of `out` is defined
     if (plan && num_parts > 0) {
         const PlanView v = plan_view(const_cast<void*>(plan), num_parts, num_nodes);
         StreamInfo info;
         if (stream_usable(find_stream_info(plan, &info), in, workspace, workspace_floats, num_nodes, dim, num_parts))
             return aggregate_stream_call(out, in, v.col, scale, info, plan, num_nodes, dim, workspace, stream, sink, sink2,
-                                         gathered_rows);
+                                         gathered_rows, written, num_written);
         return aggregate_dispatch(out, in, v.col, scale, PlanGroups{v.ptr, v.row, v.flags}, num_nodes, dim, num_parts,
                                   group_size, workspace, stream, sink, sink2, v.single, gathered_rows);
     }

@@ -15,7 +15,8 @@ namespace eppgcn {
 int aggregate_forward_groups(float*, const float*, const int*, const float*, const int*, const int*, const void*, int,
                              int, int, int, float*, size_t, hipStream_t, double*, double*);
 int aggregate_compacted_groups(float*, const float*, const int*, const int*, const int*, const float*, const void*,
-                               int, int, int, int, float*, size_t, const uint32_t*, hipStream_t, double*, double*);
+                               int, int, int, int, float*, size_t, const uint32_t*, hipStream_t, double*, double*,
+                               const uint32_t** written = nullptr, long long* num_written = nullptr);
 size_t plan_workspace_bytes(long long, long long);
 int read_plan_status(const void*, long long, long long, long long, long long*, hipStream_t);
 void set_stream_mode(int);
@@ -31,12 +32,13 @@ void set_agg_force_rounds(int);
 size_t feature_workspace_floats(long long, int);
 int workspace_pitch(int);
 int launch_dense_rows(float*, int, int, const float*, int, const float*, long long, long long, const float*,
-                      const float*, int, int, long long, int, int, hipStream_t, unsigned);
+                      const float*, int, int, long long, int, int, hipStream_t, unsigned, const uint32_t* rows = nullptr);
 size_t update_workspace_bytes(long long, int, int);
-int launch_dense_weight(float*, const float*, int, const float*, int, int, long long, int, int, void*, hipStream_t);
+int launch_dense_weight(float*, const float*, int, const float*, int, int, long long, int, int, void*, hipStream_t,
+                        const uint32_t* rows = nullptr);
 bool dense_backward_fused_covers(int, int, const float*, const float*);
 int launch_dense_backward(float*, float*, const float*, const float*, const float*, int, long long, int, int, void*,
-                          hipStream_t);
+                          hipStream_t, const uint32_t* rows = nullptr);
 size_t compact_workspace_bytes(long long);
 size_t split_workspace_bytes(long long);
 int launch_mask_forward(const int*, const int*, const int*, const uint8_t*, uint8_t*, int*, int*, int, long long, int,
@@ -93,7 +95,7 @@ using namespace eppgcn;
 extern "C" {
 
 const char* eppgcn_last_error(void) { return g_last_error.c_str(); }
-int eppgcn_abi_version(void) { return 15; }
+int eppgcn_abi_version(void) { return 16; }
 
 int eppgcn_spmm_forward(float* out, const float* in, const int32_t* row_pointers, const int32_t* column_index,
                         const float* degrees, const int32_t* part_pointers, const int32_t* part2node, int num_nodes,
@@ -161,6 +163,37 @@ int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* i
                                       dim, num_parts, part_size > 0 ? part_size : 1, workspace, workspace_floats, gathered_rows,
                                       static_cast<hipStream_t>(stream), &g_back_agg_ms,
                                       layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr);
+}
+
+int eppgcn_ours_backward_rows(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
+                              const int32_t* edge_list, const float* degrees, int num_nodes, int dim, int num_parts,
+                              int part_size, int layer, int blockx, int blocky, float* workspace,
+                              size_t workspace_floats, const void* plan, const uint32_t* gathered_rows,
+                              const uint32_t** written_rows, int64_t* num_written, void* stream)
+{
+    EPPGCN_REQUIRE(written_rows, "written_rows must not be NULL (eppgcn_ours_backward is the call without it)");
+    *written_rows = nullptr;
+    if (num_written) *num_written = num_nodes > 0 ? num_nodes : 0;
+    EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
+    EPPGCN_REQUIRE(blockx > 0 && blocky > 0, "launch hints must be positive");
+    EPPGCN_REQUIRE(layer >= 1, "layer is 1-based");
+    if (num_nodes == 0) return kOk;
+    EPPGCN_REQUIRE(d_input && (d_output || workspace) && degrees, "null feature or scale pointer");
+    EPPGCN_REQUIRE(num_parts == 0 || (ids && part_pointer && edge_list), "null index pointer");
+    EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
+    EPPGCN_REQUIRE(!plan || aligned(plan, 256), "plan must be 256-byte aligned");
+    EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != d_input),
+                   "workspace must be 16-byte aligned and distinct from the output");
+    EPPGCN_REQUIRE(!workspace || workspace == d_output || workspace_floats >= feature_workspace_floats(num_nodes, dim),
+                   "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
+    long long count = num_nodes;
+    const int rc = aggregate_compacted_groups(d_input, d_output, ids, part_pointer, edge_list, degrees, plan, num_nodes,
+                                              dim, num_parts, part_size > 0 ? part_size : 1, workspace, workspace_floats,
+                                              gathered_rows, static_cast<hipStream_t>(stream), &g_back_agg_ms,
+                                              layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr,
+                                              written_rows, &count);
+    if (num_written) *num_written = *written_rows ? count : num_nodes;
+    return rc;
 }
 
 int eppgcn_mask_forward(const int32_t* part2node, const int32_t* part_pointers, const int32_t* column_index,
@@ -635,6 +668,30 @@ int eppgcn_update_backward(float* d_x, float* d_w, const float* x, const float* 
     if (num_nodes == 0) return kOk;
     return launch_dense_rows(d_x, in_dim, in_dim, g, out_dim, w, 1, out_dim, nullptr, relu_input ? x : nullptr, in_dim,
                              0, num_nodes, out_dim, in_dim, s, 0u);
+}
+
+int eppgcn_update_backward_rows(float* d_x, float* d_w, const float* x, const float* g, const float* w, int relu_input,
+                                const uint32_t* rows, int64_t num_nodes, int in_dim, int out_dim, void* workspace,
+                                size_t workspace_bytes, void* stream)
+{
+    EPPGCN_REQUIRE(num_nodes >= 0 && in_dim > 0 && out_dim > 0, "num_nodes >= 0, in_dim > 0, out_dim > 0 required");
+    EPPGCN_REQUIRE(d_w, "null output pointer");
+    EPPGCN_REQUIRE(num_nodes == 0 || (x && g && (w || !d_x)), "null matrix pointer");
+    EPPGCN_REQUIRE(aligned(d_x, 4) && aligned(d_w, 4) && aligned(x, 4) && aligned(g, 4) && aligned(w, 4) && aligned(rows, 4),
+                   "matrix pointers and the row bitmap must be 4-byte aligned");
+    EPPGCN_REQUIRE(!d_x || (d_x != g && d_x != x), "the input gradient cannot be written over an input");
+    EPPGCN_REQUIRE(num_nodes == 0 || (workspace && aligned(workspace, 4) &&
+                                      workspace_bytes >= update_workspace_bytes(num_nodes, in_dim, out_dim)),
+                   "workspace smaller than eppgcn_update_workspace_bytes(num_nodes, in_dim, out_dim)");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (d_x && (num_nodes == 0 || dense_backward_fused_covers(in_dim, out_dim, x, g)))
+        return launch_dense_backward(d_x, d_w, x, g, w, relu_input ? 1 : 0, num_nodes, in_dim, out_dim, workspace, s, rows);
+    if (int rc = launch_dense_weight(d_w, x, in_dim, g, out_dim, relu_input ? 1 : 0, num_nodes, in_dim, out_dim,
+                                     workspace, s, rows))
+        return rc;
+    if (num_nodes == 0 || !d_x) return kOk;
+    return launch_dense_rows(d_x, in_dim, in_dim, g, out_dim, w, 1, out_dim, nullptr, relu_input ? x : nullptr, in_dim,
+                             0, num_nodes, out_dim, in_dim, s, 0u, rows);
 }
 
 }  // extern "C"

@@ -244,13 +244,31 @@ Tensor scaled_product(const Tensor& X, const Tensor& W, const Tensor& degrees, b
     return scaled;
 }
 
-// {dX or an empty tensor, dW} from the aggregated gradient G
-std::vector<Tensor> dense_backward(const Tensor& G, const Tensor& X, const Tensor& W, bool need_dx, bool relu_input)
+// g_masked_update: 1 (default) lets the pruned backward hand the bitmap of the rows it wrote to the dense products
+// (rows outside the path are then neither cleared nor read); 0 clears and reads every row.
+int g_masked_update = 1;
+
+// {dX or an empty tensor, dW} from the aggregated gradient G; `rows`: nullptr, or the bitmap of the rows of G that
+// are defined (the others count as zeros and are not read)
+std::vector<Tensor> dense_backward(const Tensor& G, const Tensor& X, const Tensor& W, bool need_dx, bool relu_input,
+                                   const uint32_t* rows = nullptr)
 {
     const int64_t n = X.size(0);
     const int in_dim = static_cast<int>(X.size(1)), out_dim = static_cast<int>(W.size(1));
     const int sup = dense_support(X, W);
     Tensor d_weight, d_input;
+    if (rows) {
+        // only reached when the shapes fit the library's kernels (the caller checked dense_support)
+        d_weight = torch::empty({in_dim, out_dim}, X.options());
+        d_input = need_dx ? torch::empty({n, in_dim}, X.options()) : torch::empty({0}, X.options());
+        const size_t nbytes = eppgcn_update_workspace_bytes(n, in_dim, out_dim);
+        auto ws = torch::empty({static_cast<int64_t>((nbytes + 3) / 4) + 1}, X.options());
+        check(eppgcn_update_backward_rows(need_dx ? d_input.data_ptr<float>() : nullptr, d_weight.data_ptr<float>(), f32(X),
+                                          f32(G), f32(W), relu_input ? 1 : 0, rows, n, in_dim, out_dim,
+                                          ws.data_ptr<float>(), nbytes, stream_of(X)),
+              "update_backward_rows");
+        return {d_input, d_weight};
+    }
     if (need_dx && (sup & 6) == 6) {
         // both gradients from one call: narrow layers read X and G once for the two products
         d_weight = torch::empty({in_dim, out_dim}, X.options());
@@ -399,13 +417,29 @@ std::vector<Tensor> ours_backward(Tensor d_output, Tensor X, Tensor W, Tensor id
                         static_cast<int>(d_output.size(1)), choice.use_plan ? 0 : 31);
     }
     auto scaled = feature_scratch(d_output, plan);     // d_output belongs to autograd: scale into scratch
-    check(eppgcn_ours_backward(d_input_prime.data_ptr<float>(), f32(d_output), i32(id), i32(partPointer),
-                               i32(edgeList), f32(degrees), static_cast<int>(d_output.size(0)),
-                               static_cast<int>(d_output.size(1)), numParts, partSize > 0 ? partSize : 1, layer, blockx,
-                               blocky, scaled.numel() ? scaled.data_ptr<float>() : nullptr,
-                               static_cast<size_t>(scaled.numel()), plan, gathered, stream_of(d_output)),
-          "ours_backward");
-    return dense_backward(d_input_prime, X, W, need_dx, relu_input);
+    // The aggregated gradient is only read by the two dense products below.  When they run in the library's kernels
+    // (which take the bitmap of the rows the aggregation wrote), the rows outside the path are neither cleared
+    // nor read - the row-masked products the reference sketches in its comments (EPPGCN_kernel.cu:607,616).
+    const int sup = dense_support(X, W);
+    const bool masked = g_masked_update > 0 && plan && (sup & 4) && (!need_dx || (sup & 2));
+    const uint32_t* written = nullptr;
+    if (masked) {
+        check(eppgcn_ours_backward_rows(d_input_prime.data_ptr<float>(), f32(d_output), i32(id), i32(partPointer),
+                                        i32(edgeList), f32(degrees), static_cast<int>(d_output.size(0)),
+                                        static_cast<int>(d_output.size(1)), numParts, partSize > 0 ? partSize : 1, layer,
+                                        blockx, blocky, scaled.numel() ? scaled.data_ptr<float>() : nullptr,
+                                        static_cast<size_t>(scaled.numel()), plan, gathered, &written, nullptr,
+                                        stream_of(d_output)),
+              "ours_backward_rows");
+    } else {
+        check(eppgcn_ours_backward(d_input_prime.data_ptr<float>(), f32(d_output), i32(id), i32(partPointer),
+                                   i32(edgeList), f32(degrees), static_cast<int>(d_output.size(0)),
+                                   static_cast<int>(d_output.size(1)), numParts, partSize > 0 ? partSize : 1, layer, blockx,
+                                   blocky, scaled.numel() ? scaled.data_ptr<float>() : nullptr,
+                                   static_cast<size_t>(scaled.numel()), plan, gathered, stream_of(d_output)),
+              "ours_backward");
+    }
+    return dense_backward(d_input_prime, X, W, need_dx, relu_input, written);
 }
 
 // ---------------------------------------------------------------- path preparation
@@ -595,6 +629,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
           py::arg("blocky"), py::arg("need_dx") = true, py::arg("relu_input") = false);
     m.def("set_dense_policy", [](int policy) { g_dense_policy = policy; },
           "dense products: 0 = library kernels where the shapes fit (default), -1 = always torch::mm");
+    m.def("set_masked_update", [](bool on) { g_masked_update = on ? 1 : 0; },
+          "pruned backward: true (default) = the dense products take the bitmap of the rows the aggregation wrote and the "
+          "other rows are neither cleared nor read; false = clear and read every row");
     m.def("print_time", &eppgcn_print_time, "print accumulated kernel times");
     m.def("clear_time", &eppgcn_clear_time, "reset accumulated kernel times");
     m.def("set_timing", [](bool on) { eppgcn_set_timing(on ? 1 : 0); }, "enable per-call kernel timing");

@@ -21,11 +21,22 @@
 //   backward kernel  both gradients of a narrow layer (<= 16 inputs, <= 32 gradient columns) in one pass:
 //                  the 16 rows of a step are copied to LDS with full 16-byte loads and both products take
 //                  their operands from there, accumulated exactly as the two kernels above do it.
+//
+// Row bitmap (the backward products of a pruned layer; the reference sketches the same with an index,
+// `torch::mm(X.index({mask}).transpose(0,1), d_input_prime.index({mask}))`, EPPGCN_kernel.cu:607,616): with `rows`
+// given, a row of the tall operands whose bit is clear is taken as zero and never read - neither the gradient
+// row, which then need not hold defined values, nor the layer-input row that would be multiplied with it.
 #include "common.hpp"
 
 namespace eppgcn {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// bits of the 16 rows from r0 on (r0 a multiple of 16); all set without a bitmap
+__device__ __forceinline__ unsigned tile_row_bits(const uint32_t* __restrict__ rows, long long r0)
+{
+    return rows ? (rows[r0 >> 5] >> (r0 & 31)) & 0xffffu : 0xffffu;
+}
 
 constexpr int kUpdateThreads = 256;
 constexpr int kUpdateWaves = kUpdateThreads / kWave;
@@ -81,6 +92,7 @@ struct RowsArgs {
     int tile_store;          // the 16 rows of a tile are 16 * out_cols contiguous floats (ld_out == out_cols == 32,
                              // 16-byte aligned): they go through LDS and out as two 1 KB stores per wave
     unsigned swz_mask;       // row r of out lives at swizzled_row(r, swz_mask): 0 = vertex order (common.hpp)
+    const uint32_t* rows;    // nullptr, or one bit per row of x: clear = the row counts as zeros and is not read
 };
 
 template <int VW, int MT, int CU>
@@ -108,6 +120,7 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_rows_kernel(RowsArgs a)
          tile += static_cast<long long>(gridDim.x) * kUpdateWaves) {
         const long long r = tile * kTileRows + i;
         const bool row_ok = r < a.n;
+        const bool live = row_ok && (!a.rows || ((a.rows[r >> 5] >> (r & 31)) & 1u));
         const long long rc = row_ok ? r : a.n - 1;      // rows past the end read the last row, store nothing
         const float* __restrict__ xrow = a.x + rc * a.ld_x;
         floatx4 acc[MT];
@@ -117,7 +130,14 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_rows_kernel(RowsArgs a)
         for (int t0 = 0; t0 < chunks_p; t0 += CU) {
             float x[CU][VW];
 #pragma unroll
-            for (int u = 0; u < CU; ++u) load_row_piece<VW>(x[u], xrow, (4 * (t0 + u) + j) * VW, a.K, a.relu_in != 0);
+            for (int u = 0; u < CU; ++u) {
+                if (live || !a.rows) {
+                    load_row_piece<VW>(x[u], xrow, (4 * (t0 + u) + j) * VW, a.K, a.relu_in != 0);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < VW; ++v) x[u][v] = 0.f;
+                }
+            }
 #pragma unroll
             for (int u = 0; u < CU; ++u) {
 #pragma unroll
@@ -155,7 +175,7 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_rows_kernel(RowsArgs a)
                 for (int mt = 0; mt < 2; ++mt) {
                     const int m0 = mt * 16 + 4 * j;
                     float y[4] = {acc[mt][0] * s, acc[mt][1] * s, acc[mt][2] * s, acc[mt][3] * s};
-                    if (a.relu_ref && row_ok) {
+                    if (a.relu_ref && live) {
                         const float* __restrict__ ref = a.relu_ref + r * a.ld_ref;
 #pragma unroll
                         for (int v = 0; v < 4; ++v)
@@ -190,7 +210,7 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_rows_kernel(RowsArgs a)
             const int m0 = mt * 16 + 4 * j;
             if (m0 >= a.out_cols) continue;
             float y[4] = {acc[mt][0] * s, acc[mt][1] * s, acc[mt][2] * s, acc[mt][3] * s};
-            if (a.relu_ref) {
+            if (a.relu_ref && live) {
                 const float* __restrict__ ref = a.relu_ref + r * a.ld_ref;
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
@@ -240,7 +260,7 @@ static hipError_t launch_rows_mt(const RowsArgs& a, int mt, int cu, unsigned blo
 // operand to fit the LDS (the caller then has to use a general GEMM).
 int launch_dense_rows(float* out, int ld_out, int out_cols, const float* x, int ld_x, const float* w, long long sk,
                       long long sm, const float* scale, const float* relu_ref, int ld_ref, int relu_in,
-                      long long n, int K, int M, hipStream_t stream, unsigned swz_mask)
+                      long long n, int K, int M, hipStream_t stream, unsigned swz_mask, const uint32_t* rows)
 {
     if (n == 0 || out_cols == 0) return kOk;
     const uintptr_t xa = reinterpret_cast<uintptr_t>(x);
@@ -279,6 +299,7 @@ int launch_dense_rows(float* out, int ld_out, int out_cols, const float* x, int 
         a.M = M - c0 > 0 ? (M - c0 < cols ? M - c0 : cols) : 0;
         a.relu_in = relu_in;
         a.swz_mask = swz_mask;
+        a.rows = rows;
         a.vec_store = (ld_out % 4 == 0 && reinterpret_cast<uintptr_t>(a.out) % 16 == 0) ? 1 : 0;
         // measured at 4.2 M rows: a [N, 96] result 0.63 -> 0.47 ms with non-temporal stores, [N, 16] and
         // [N, 32] results unchanged or slower
@@ -301,7 +322,8 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_weight_kernel(float* __r
                                                                       const float* __restrict__ x, int ld_x,
                                                                       const float* __restrict__ g, int ld_g,
                                                                       int relu_in, long long n, int K, int D,
-                                                                      long long rows_per_wave)
+                                                                      long long rows_per_wave,
+                                                                      const uint32_t* __restrict__ rows)
 {
     __shared__ float red[kUpdateWaves][KTB * DT * 4 * kWave];
     const int lane = lane_id();
@@ -319,11 +341,13 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_weight_kernel(float* __r
     long long r_end = r_begin + rows_per_wave;
     if (r_end > n) r_end = n;
     for (long long r0 = r_begin; r0 < r_end; r0 += 16) {
+        const unsigned bits = tile_row_bits(rows, r0);
+        if (bits == 0u) continue;                       // wave-uniform: none of the 16 rows contributes
         float av[4][KTB], bv[4][DT];
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             const long long row = r0 + 4 * s + j;
-            const bool ok = row < r_end;
+            const bool ok = row < r_end && ((bits >> (4 * s + j)) & 1u);
             const float* __restrict__ xr = x + (ok ? row : r_begin) * ld_x;
             const float* __restrict__ gr = g + (ok ? row : r_begin) * ld_g;
 #pragma unroll
@@ -407,17 +431,18 @@ size_t update_workspace_bytes(long long n, int K, int D)
 
 template <int KTB, int DT>
 static hipError_t launch_weight(float* partial, const float* x, int ld_x, const float* g, int ld_g, int relu_in,
-                                long long n, int K, int D, long long rows_per_wave, int blocks, hipStream_t stream)
+                                long long n, int K, int D, long long rows_per_wave, int blocks, hipStream_t stream,
+                                const uint32_t* rows)
 {
     const int ktiles = (K + 15) / 16;
     hipLaunchKernelGGL((dense_weight_kernel<KTB, DT>), dim3(blocks, (ktiles + KTB - 1) / KTB), dim3(kUpdateThreads), 0,
-                       stream, partial, x, ld_x, g, ld_g, relu_in, n, K, D, rows_per_wave);
+                       stream, partial, x, ld_x, g, ld_g, relu_in, n, K, D, rows_per_wave, rows);
     return hipGetLastError();
 }
 
 // dw[K, D] = act(X[N, K])^T * G[N, D]; D <= 64.
 int launch_dense_weight(float* dw, const float* x, int ld_x, const float* g, int ld_g, int relu_in, long long n,
-                        int K, int D, void* workspace, hipStream_t stream)
+                        int K, int D, void* workspace, hipStream_t stream, const uint32_t* rows)
 {
     if (K == 0 || D == 0) return kOk;
     if (n == 0) {
@@ -436,7 +461,7 @@ int launch_dense_weight(float* dw, const float* x, int ld_x, const float* g, int
     int ktb = 8 / dt;
     while (ktb > 1 && ktb / 2 >= ktiles) ktb /= 2;
     hipError_t e;
-#define EPPGCN_W(KTB_, DT_) launch_weight<KTB_, DT_>(partial, x, ld_x, g, ld_g, relu_in, n, K, D, rows_per_wave, blocks, stream)
+#define EPPGCN_W(KTB_, DT_) launch_weight<KTB_, DT_>(partial, x, ld_x, g, ld_g, relu_in, n, K, D, rows_per_wave, blocks, stream, rows)
     if (dt == 1) e = ktb == 8 ? EPPGCN_W(8, 1) : ktb == 4 ? EPPGCN_W(4, 1) : ktb == 2 ? EPPGCN_W(2, 1) : EPPGCN_W(1, 1);
     else if (dt == 2) e = ktb == 4 ? EPPGCN_W(4, 2) : ktb == 2 ? EPPGCN_W(2, 2) : EPPGCN_W(1, 2);
     else e = ktb == 2 ? EPPGCN_W(2, 4) : EPPGCN_W(1, 4);
@@ -468,6 +493,7 @@ struct BackwardArgs {
     int K, D;
     int relu_in;             // the layer applied max(x, 0) to its input
     int vec_store;           // rows of dx are 16-byte aligned
+    const uint32_t* rows;    // nullptr, or one bit per row: clear = the row of g counts as zeros, it and its row of x are not read
 };
 
 constexpr int kBackMaxK = 16, kBackMaxD = 32;
@@ -507,8 +533,18 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_backward_kernel(Backward
 
     // 16 rows from row r0 on (fewer at the end of the matrix; what lies past the wave's own range is loaded but
     // never used): G as kGVecs vectors per lane, X as one
+    // which of the tile's 16 rows a lane's vectors touch (a 16-byte vector can lie across two rows): the same
+    // for every tile, so worked out once.  A vector is fetched when one of its rows has its bit set.
     floatx4 gv[kGVecs], xv;
-    auto request = [&](long long r0) {
+    unsigned gneed[kGVecs], xneed;
+    auto rows_of = [](int off, int width) {
+        const int ra = off / width, rb = (off + 3) / width;
+        return (ra < 16 ? 1u << ra : 0u) | (rb < 16 ? 1u << rb : 0u);
+    };
+#pragma unroll
+    for (int q = 0; q < kGVecs; ++q) gneed[q] = rows_of((q * kWave + lane) * 4, a.D);
+    xneed = rows_of(lane * 4, a.K);
+    auto request = [&](long long r0, unsigned bits) {
         const long long rows = a.n - r0 < 16 ? a.n - r0 : 16;
         const float* __restrict__ gsrc = a.g + r0 * a.D;
         const float* __restrict__ xsrc = a.x + r0 * a.K;
@@ -516,20 +552,46 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_backward_kernel(Backward
 #pragma unroll
         for (int q = 0; q < kGVecs; ++q) {
             const int off = (q * kWave + lane) * 4;
-            if (off + 4 <= gcount) gv[q] = *reinterpret_cast<const floatx4*>(gsrc + off);
+            if (!(gneed[q] & bits)) gv[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+            else if (off + 4 <= gcount) gv[q] = *reinterpret_cast<const floatx4*>(gsrc + off);
             else
 #pragma unroll
                 for (int c = 0; c < 4; ++c) gv[q][c] = off + c < gcount ? gsrc[off + c] : 0.f;
         }
         const int off = lane * 4;
-        if (off + 4 <= xcount) xv = *reinterpret_cast<const floatx4*>(xsrc + off);
+        if (!(xneed & bits)) xv = floatx4{0.f, 0.f, 0.f, 0.f};
+        else if (off + 4 <= xcount) xv = *reinterpret_cast<const floatx4*>(xsrc + off);
         else
 #pragma unroll
             for (int c = 0; c < 4; ++c) xv[c] = off + c < xcount ? xsrc[off + c] : 0.f;
     };
-    if (r_begin < r_end) request(r_begin);
+    unsigned bits = 0u, bits_next = 0u;
+    if (r_begin < r_end) {
+        bits = tile_row_bits(a.rows, r_begin);
+        request(r_begin, bits);
+    }
 
-    for (long long r0 = r_begin; r0 < r_end; r0 += 16) {
+    for (long long r0 = r_begin; r0 < r_end; r0 += 16, bits = bits_next) {
+        const long long r = r0 + i;
+        const bool row_ok = r < r_end;
+        const int m0 = 4 * j;
+        if (bits == 0u) {            // wave-uniform: no row of the tile carries a gradient; its rows of dX are zeros
+            if (r0 + 16 < r_end) {
+                bits_next = tile_row_bits(a.rows, r0 + 16);
+                request(r0 + 16, bits_next);
+            }
+            if (row_ok && m0 < a.K) {
+                float* __restrict__ orow = a.dx + r * a.K;
+                if (a.vec_store && m0 + 4 <= a.K) {
+                    *reinterpret_cast<float4*>(orow + m0) = make_float4(0.f, 0.f, 0.f, 0.f);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (m0 + v < a.K) orow[m0 + v] = 0.f;
+                }
+            }
+            continue;
+        }
         // the wave's LDS area is its own: its LDS operations execute in order, so the stores below come after the
         // previous step's reads without a barrier
 #pragma unroll
@@ -538,11 +600,14 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_backward_kernel(Backward
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        if (r0 + 16 < r_end) request(r0 + 16);               // under way during this step's products
+        if (r0 + 16 < r_end) {                               // under way during this step's products
+            bits_next = tile_row_bits(a.rows, r0 + 16);
+            request(r0 + 16, bits_next);
+        }
 
         // ---- dX for rows r0 .. r0 + 15: lane (i, j) takes VW consecutive gradient columns of row r0 + i per step
-        const long long r = r0 + i;
-        const bool row_ok = r < r_end;
+        // (a row whose bit is clear may share a fetched vector with a neighbour: its values are not used)
+        const bool row_live = (bits >> i) & 1u;
         floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int t = 0; t < CH; ++t) {
@@ -550,10 +615,9 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_backward_kernel(Backward
 #pragma unroll
             for (int v = 0; v < VW; ++v) {
                 const int d = (4 * t + j) * VW + v;
-                acc = mfma16(wp[v], d < a.D ? gt[i * a.D + d] : 0.f, acc);
+                acc = mfma16(wp[v], (d < a.D && row_live) ? gt[i * a.D + d] : 0.f, acc);
             }
         }
-        const int m0 = 4 * j;
         if (row_ok && m0 < a.K) {
             float y[4] = {acc[0], acc[1], acc[2], acc[3]};
             if (a.relu_in) {
@@ -574,7 +638,7 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_backward_kernel(Backward
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             const int lr = 4 * s + j;
-            const bool ok = r0 + lr < r_end;
+            const bool ok = r0 + lr < r_end && ((bits >> lr) & 1u);
             const float t = (ok && i < a.K) ? xt[lr * a.K + i] : 0.f;
             const float av = a.relu_in ? fmaxf(t, 0.f) : t;
 #pragma unroll
@@ -614,7 +678,7 @@ bool dense_backward_fused_covers(int K, int D, const float* x, const float* g)
 // dx[N, K] and dw[K, D] of a layer out = act(X) * W from the gradient G[N, D] of the product, in one pass over X
 // and G (dense_backward_fused_covers(K, D) holds; `workspace` as for launch_dense_weight).
 int launch_dense_backward(float* dx, float* dw, const float* x, const float* g, const float* w, int relu_in,
-                          long long n, int K, int D, void* workspace, hipStream_t stream)
+                          long long n, int K, int D, void* workspace, hipStream_t stream, const uint32_t* rows)
 {
     if (n == 0) return launch_zero_words(dw, static_cast<size_t>(K) * D, stream);
     const int blocks = weight_blocks(n);
@@ -631,6 +695,7 @@ int launch_dense_backward(float* dx, float* dw, const float* x, const float* g, 
     a.D = D;
     a.relu_in = relu_in;
     a.vec_store = (K % 4 == 0 && reinterpret_cast<uintptr_t>(dx) % 16 == 0) ? 1 : 0;
+    a.rows = rows;
     const int vw = D % 4 == 0 ? 4 : D % 2 == 0 ? 2 : 1;        // the order of additions of dense_rows_kernel for aligned g
     const int dt = D <= 16 ? 1 : 2;
 #define EPPGCN_B(VW_, DT_) hipLaunchKernelGGL((dense_backward_kernel<VW_, DT_>), dim3(blocks), dim3(kUpdateThreads), 0, stream, a)

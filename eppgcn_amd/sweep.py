@@ -2,7 +2,9 @@
 aggregation widths x backward group sizes.  For every cell, what a caller sees: the time of the
 whole pruned backward *call* (output clear + pre-scaling pass + aggregation kernels; two HIP events
 around back-to-back calls) next to the whole unpruned call, algorithmic GB/s and the speed-up on the
-calls, the aggregation kernels alone as sub-fields, and what the pruned path costs to prepare
+calls, the same pruned call for a consumer that takes the bitmap of the written rows instead of a
+cleared output (``eppgcn_ours_backward_rows``: what the extension module's backward runs), the
+aggregation kernels alone as sub-fields, and what the pruned path costs to prepare
 (marking, compaction, split, gathered-rows bitmap, execution plan) with the number of backward
 calls after which the preparation has paid for itself.
 
@@ -101,6 +103,11 @@ def main():
                     capi.ours_backward(dy, ids, part_pointer, edge_list, g.degrees, num_parts, gs, 1, 4, 16, out, ws,
                                        plan=plan, gathered_rows=gathered)
 
+                def pruned_rows_call():
+                    # for a consumer that takes the bitmap of the written rows (the layer's dense products): no clear
+                    capi.ours_backward_rows(dy, ids, part_pointer, edge_list, g.degrees, num_parts, gs, 1, 4, 16, out, ws,
+                                            plan=plan, gathered_rows=gathered)
+
                 def unpruned_call():
                     capi.spmm_forward(dy, g.column_index, g.degrees, part_ptr, part2node, ps, 32, 8, None, out, True, ws,
                                       plan=forward_plan(width))
@@ -122,6 +129,7 @@ def main():
                 pruned_ms = _events_ms(pruned_call, args.reps)
                 streamed = capi.last_call_used_stream()
                 unpruned_ms = _events_ms(unpruned_call, args.reps)
+                pruned_rows_ms = _events_ms(pruned_rows_call, args.reps)
                 pruned_kernel_ms, pruned_clear_ms, pruned_scale_ms = parts_ms(pruned_call)
                 unpruned_kernel_ms, unpruned_clear_ms, unpruned_scale_ms = parts_ms(unpruned_call)
                 unpruned_call()                   # `out` holds the unpruned result for the check below
@@ -146,6 +154,8 @@ def main():
                         "mark_ms": round(mark_ms, 4), "compact_ms": round(compact_ms, 4), "split_ms": round(split_ms, 4),
                         "bitmap_ms": round(bitmap_ms, 4), "plan_ms": round(plan_ms, 4), "prep_ms": round(prep_ms, 4),
                         "pruned_call_ms": round(pruned_ms, 4), "unpruned_call_ms": round(unpruned_ms, 4),
+                        "pruned_rows_call_ms": round(pruned_rows_ms, 4),
+                        "speedup_rows_call": round(unpruned_ms / pruned_rows_ms, 2),
                         "pruned_GBps": round(nbytes / pruned_ms / 1e6, 1),
                         "unpruned_GBps": round(workload.bytes_forward(n, e, width) / unpruned_ms / 1e6, 1),
                         "speedup": round(unpruned_ms / pruned_ms, 2),

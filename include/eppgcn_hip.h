@@ -208,6 +208,22 @@ int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* i
                          int num_nodes, int dim, int num_parts, int part_size, int layer,
                          int blockx, int blocky, float* workspace, size_t workspace_floats, const void* plan,
                          const uint32_t* gathered_rows, void* stream);
+/* eppgcn_ours_backward for a caller that reads d_input only in the rows the path writes (the dense products
+ * of the layer's backward step, eppgcn_update_backward_rows): the same call, same results in those rows, but
+ * when it runs a plan's stream form the rows without any group are LEFT AS THEY ARE instead of being cleared
+ * (with a 10 % train mask two thirds of the rows of the last layer's gradient: the clear was most of a heavily
+ * pruned call), and *written_rows receives the device address of the bitmap of the rows that were written
+ * (bit r of word r / 32; it lies inside the plan and lives as long as the plan), *num_written (may be NULL)
+ * their number.  When the call cannot skip the clear (no plan, no stream form for the shape or workspace),
+ * it clears as eppgcn_ours_backward does and sets *written_rows = NULL: every row of d_input is defined.
+ * The reference sketches the consumer side of this in the comments of ours_backward_cuda
+ * (`X.index({mask})`, EPPGCN_kernel.cu:607,616); it has no such call itself. */
+int eppgcn_ours_backward_rows(float* d_input, const float* d_output, const int32_t* ids,
+                              const int32_t* part_pointer, const int32_t* edge_list, const float* degrees,
+                              int num_nodes, int dim, int num_parts, int part_size, int layer,
+                              int blockx, int blocky, float* workspace, size_t workspace_floats, const void* plan,
+                              const uint32_t* gathered_rows, const uint32_t** written_rows, int64_t* num_written,
+                              void* stream);
 
 /* bitmap[(num_nodes + 31) / 32]: bit c is set for every vertex c that occurs in
  * edge_list[0 .. valid_len) (the rows a pruned backward over this path gathers); *d_count (device)
@@ -403,6 +419,17 @@ int eppgcn_update_backward_weight(float* d_w, const float* x, const float* g, in
 int eppgcn_update_backward(float* d_x, float* d_w, const float* x, const float* g, const float* w, int relu_input,
                            int64_t num_nodes, int in_dim, int out_dim, void* workspace, size_t workspace_bytes,
                            void* stream);
+/* eppgcn_update_backward for a gradient of which only some rows are defined: `rows` holds one bit per row of g
+ * (bit r of word r / 32, (num_nodes + 31) / 32 words; NULL = every row, i.e. eppgcn_update_backward).  A row whose
+ * bit is clear counts as zeros and is not read - neither that row of g, which may hold anything, nor the row of x
+ * it would be multiplied with; its row of d_x is written as zeros.  Where the rows with clear bits do hold zeros the
+ * results equal those of eppgcn_update_backward bit for bit.  d_x may be NULL (and then w): only d_w is formed (a
+ * first layer whose input needs no gradient).  This is the row-masked product the reference sketches in
+ * `d_weight = torch::mm(X.index({mask}).transpose(0,1), d_input_prime.index({mask}))`, EPPGCN_kernel.cu:616, taken
+ * over the bitmap eppgcn_ours_backward_rows hands out instead of an index list. */
+int eppgcn_update_backward_rows(float* d_x, float* d_w, const float* x, const float* g, const float* w, int relu_input,
+                                const uint32_t* rows, int64_t num_nodes, int in_dim, int out_dim, void* workspace,
+                                size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Timers (print_time / clear_time, EPPGCN_kernel.cu:89-116; EPPGCN.cpp:394-395).

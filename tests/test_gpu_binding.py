@@ -458,6 +458,37 @@ def test_unpruned_ablation_gives_the_gradients_of_the_pruned_path(GNNA, num_laye
         assert np.linalg.norm(a - b) <= 1e-5 * np.linalg.norm(a) + 1e-12
 
 
+@pytest.mark.parametrize("num_layers", [2, 3])
+def test_row_masked_dense_products_give_the_same_gradients(GNNA, num_layers):
+    """With execution plans the pruned backward leaves the rows outside the path uncleared and its two dense products
+    read only the rows the aggregation wrote (``set_masked_update``, on by default; the reference sketches the masked
+    weight gradient at EPPGCN_kernel.cu:607,616).  The weight gradients of every layer are the bits of the run that
+    clears and reads every row."""
+    from eppgcn_amd import graphs, train
+    indptr, col = random_symmetric_csr(3000, 9000, 47)
+    n = indptr.size - 1
+    g = graphs.Graph("t", n, dev(indptr), dev(col), dev(scale_inv_sqrt(indptr)))
+    mask = torch.from_numpy(np.random.default_rng(7).random(n) < 0.1)
+    grads = []
+    GNNA.set_plan_policy(1)
+    try:
+        for masked in (True, False):
+            GNNA.set_masked_update(masked)
+            tr = train.Trainer(g, dim=20, hidden=16, num_classes=9, num_layers=num_layers, train_mask=mask, backsize=4,
+                               labels="uniform")
+            tr.optimizer = torch.optim.SGD(tr.model.parameters(), lr=0.0)
+            tr.train_step(True)
+            tr.train_step(False)
+            grads.append([c.weights.grad.clone() for c in tr.model.convs])
+            GNNA.clear_plans()
+    finally:
+        GNNA.set_masked_update(True)
+        GNNA.set_plan_policy(0)
+    assert all(a.abs().sum() > 0 for a in grads[0])
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
+
+
 def test_group_size_rules_on_device_degrees(GNNA):
     """get_wave64_back_part_size / get_map_back_part_size on kept degrees that live on the device: the
     wave64 rule is 16 below 24 kept edges per kept row and 32 from there on; the fitted regression

@@ -290,6 +290,49 @@ def test_stream_pruned_backward_with_gathered_rows(api, name, ratio):
             assert_close(out.cpu().numpy(), want, bound, f"{name} D={dim} shift={shift}")
 
 
+@pytest.mark.parametrize("name,ratio", [("hub", 0.5), ("medium", 0.05), ("isolated", 0.3)])
+def test_pruned_backward_that_leaves_unwritten_rows_alone(api, name, ratio):
+    """eppgcn_ours_backward_rows (no counterpart in the reference): through a plan's stream form the rows without
+    groups keep what they held (NaN here), the written rows hold the bits eppgcn_ours_backward writes, the bitmap it
+    hands out marks exactly the rows with kept slots and is the one inside the plan; the dense products over that
+    bitmap equal the products over the cleared gradient bit for bit.  Without a plan the call clears like
+    eppgcn_ours_backward and hands out no bitmap."""
+    indptr, col = GRAPHS[name]()
+    n = indptr.size - 1
+    s = scale_inv_sqrt(indptr)
+    rng = np.random.default_rng(3)
+    src = rng.random(n) < ratio
+    fpp, fp2n = co.build_part(8, indptr)
+    mask = torch.full((col.size,), -1, dtype=torch.int32, device="cuda")
+    degs = torch.zeros(n, dtype=torch.int32, device="cuda")
+    api.mask_forward(dev(fp2n), dev(fpp), dev(col), dev(src), None, mask, degs, True)
+    oid, oedge, v = api.compact_back_edge(mask, dev(col))
+    has_slots = degs.cpu().numpy() > 0
+    for dim, ps, k in ((16, 32, 96), (22, 4, 16)):
+        bpp, p, _ = api.split_back_part(degs, col.size, ps)
+        dy = dev((rng.standard_normal((n, dim)) * src[:, None]).astype(np.float32))
+        plan = api.build_plan(bpp, oedge, p, v, n, dim, ids=oid)
+        want = api.ours_backward(dy, oid, bpp, oedge, dev(s), p, part_size=ps, plan=plan)
+        assert api.last_call_used_stream()
+        out = torch.full((n, dim), float("nan"), device="cuda")
+        got, rows, count = api.ours_backward_rows(dy, oid, bpp, oedge, dev(s), p, part_size=ps, plan=plan, out=out)
+        assert api.last_call_used_stream() and rows is not None and count == int(has_slots.sum())
+        assert rows == plan.stream_view()["touched"].data_ptr()
+        g = got.cpu().numpy()
+        assert np.array_equal(g[has_slots], want.cpu().numpy()[has_slots]) and np.isnan(g[~has_slots]).all()
+        # the layer's two dense products over the bitmap, from the uncleared gradient
+        x = dev(rng.standard_normal((n, k)).astype(np.float32))
+        w = dev(rng.uniform(-0.5, 0.5, (k, dim)).astype(np.float32))
+        want_dx, want_dw = api.update_backward(x, w, want, relu_input=True)
+        dx, dw = api.update_backward_rows(x, w, got, rows, relu_input=True)
+        assert torch.equal(dx, want_dx) and torch.equal(dw, want_dw)
+        # no plan: the group kernel clears, every row is defined
+        out.fill_(float("nan"))
+        got, rows, count = api.ours_backward_rows(dy, oid, bpp, oedge, dev(s), p, part_size=ps, out=out)
+        assert rows is None and count == n and not api.last_call_used_stream()
+        assert not torch.isnan(got).any() and not got.cpu().numpy()[~has_slots].any()
+
+
 def test_stream_from_a_table_written_by_the_dense_update(api):
     """eppgcn_update_forward_table leaves the table in the workspace's row order with room for the partial sums;
     the aggregation with a NULL input then runs the stream form on it."""

@@ -111,6 +111,49 @@ def test_update_backward_pair_equals_the_two_products(api, n, k, m, relu):
         assert not dx.cpu().numpy()[x <= 0].any()
 
 
+def pack_rows(live):
+    """bool[n] -> the int32 bitmap the masked products take (bit r of word r // 32)."""
+    n = live.size
+    padded = np.zeros((n + 31) // 32 * 32, bool)
+    padded[:n] = live
+    words = np.packbits(padded.reshape(-1, 32), axis=1, bitorder="little").view(np.uint32).reshape(-1)
+    return dev(words.view(np.int32))
+
+
+# the shapes of the pair test (one-pass kernel, the two separate kernels), a first layer (only d_w), and densities of
+# the bitmap from "no row" over whole dead tiles to "every row"
+@pytest.mark.parametrize("n,k,m", [(1, 1, 1), (5, 3, 2), (16, 16, 16), (17, 16, 22), (1000, 16, 22), (4097, 16, 16),
+                                   (300, 13, 17), (999, 8, 7), (65536, 16, 22), (300007, 16, 22), (1000, 96, 16),
+                                   (500, 16, 40), (200, 33, 33)])
+@pytest.mark.parametrize("density", [0.0, 0.03, 0.4, 1.0])
+def test_update_backward_rows_reads_only_the_marked_rows(api, n, k, m, density):
+    """eppgcn_update_backward_rows (no counterpart in the reference beyond the sketch in its comments,
+    EPPGCN_kernel.cu:607,616): with the gradient zero outside the marked rows the results are those of
+    eppgcn_update_backward bit for bit; with NaN in the unmarked rows of the gradient AND of the layer input they
+    still are - those rows are not read - and the unmarked rows of d_x are zeros.  Also without d_x."""
+    x, w, g, _ = data(n, k, m, 8)
+    rng = np.random.default_rng(n + k + m)
+    live = rng.random(n) < density
+    if density == 0.03 and n > 64:
+        live[: n // 2] = False                          # whole tiles and whole wave ranges without a marked row
+    g[~live] = 0.0
+    rows = pack_rows(live)
+    for relu in (False, True):
+        want_dx, want_dw = api.update_backward(dev(x), dev(w), dev(g), relu_input=relu)
+        dx, dw = api.update_backward_rows(dev(x), dev(w), dev(g), rows, relu_input=relu)
+        assert torch.equal(dx, want_dx) and torch.equal(dw, want_dw), "zeros outside the marked rows"
+        gp, xp = g.copy(), x.copy()
+        gp[~live] = np.nan
+        xp[~live] = np.nan
+        dx, dw = api.update_backward_rows(dev(xp), dev(w), dev(gp), rows, relu_input=relu)
+        assert torch.equal(dx, want_dx) and torch.equal(dw, want_dw), "NaN outside the marked rows"
+        assert not dx.cpu().numpy()[~live].any()
+        none, dw = api.update_backward_rows(dev(xp), None, dev(gp), rows, relu_input=relu, need_dx=False)
+        assert none is None and torch.equal(dw, want_dw), "weight gradient alone"
+        dx, dw = api.update_backward_rows(dev(x), dev(w), dev(g), None, relu_input=relu)
+        assert torch.equal(dx, want_dx) and torch.equal(dw, want_dw), "no bitmap: every row"
+
+
 def test_update_backward_pair_on_unaligned_views(api):
     """Gradient and input that start 4 or 8 bytes into an allocation: the one-pass kernel's narrower loads and
     scalar stores."""
