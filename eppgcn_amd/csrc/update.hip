@@ -95,7 +95,7 @@ struct RowsArgs {
     const uint32_t* rows;    // nullptr, or one bit per row of x: clear = the row counts as zeros and is not read
 };
 
-template <int VW, int MT, int CU>
+template <int VW, int MT, int CU, bool kRows>
 __global__ __launch_bounds__(kUpdateThreads) void dense_rows_kernel(RowsArgs a)
 {
     extern __shared__ __align__(16) float w_lds[];   // [MT][chunks_p][64 lanes][VW]
@@ -120,8 +120,12 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_rows_kernel(RowsArgs a)
          tile += static_cast<long long>(gridDim.x) * kUpdateWaves) {
         const long long r = tile * kTileRows + i;
         const bool row_ok = r < a.n;
-        const bool live = row_ok && (!a.rows || ((a.rows[r >> 5] >> (r & 31)) & 1u));
-        const long long rc = row_ok ? r : a.n - 1;      // rows past the end read the last row, store nothing
+        bool live = row_ok;
+        if constexpr (kRows) live = row_ok && ((a.rows[r >> 5] >> (r & 31)) & 1u);
+        const bool dead = row_ok && !live;               // a row the bitmap leaves out: counts as zeros
+        // rows past the end read the last row and store nothing; a row the bitmap leaves out reads row 0 instead of its
+        // own (every load stays unconditional) and its values are replaced by zeros
+        const long long rc = live ? r : (row_ok ? 0 : a.n - 1);
         const float* __restrict__ xrow = a.x + rc * a.ld_x;
         floatx4 acc[MT];
 #pragma unroll
@@ -130,13 +134,12 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_rows_kernel(RowsArgs a)
         for (int t0 = 0; t0 < chunks_p; t0 += CU) {
             float x[CU][VW];
 #pragma unroll
-            for (int u = 0; u < CU; ++u) {
-                if (live || !a.rows) {
-                    load_row_piece<VW>(x[u], xrow, (4 * (t0 + u) + j) * VW, a.K, a.relu_in != 0);
-                } else {
+            for (int u = 0; u < CU; ++u) load_row_piece<VW>(x[u], xrow, (4 * (t0 + u) + j) * VW, a.K, a.relu_in != 0);
+            if constexpr (kRows) {
 #pragma unroll
-                    for (int v = 0; v < VW; ++v) x[u][v] = 0.f;
-                }
+                for (int u = 0; u < CU; ++u)
+#pragma unroll
+                    for (int v = 0; v < VW; ++v) x[u][v] = dead ? 0.f : x[u][v];
             }
 #pragma unroll
             for (int u = 0; u < CU; ++u) {
@@ -238,9 +241,15 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_rows_kernel(RowsArgs a)
 template <int VW, int MT>
 static hipError_t launch_rows_cu(const RowsArgs& a, int cu, unsigned blocks, size_t lds, hipStream_t stream)
 {
-    if (cu == 4) hipLaunchKernelGGL((dense_rows_kernel<VW, MT, 4>), dim3(blocks), dim3(kUpdateThreads), lds, stream, a);
-    else if (cu == 2) hipLaunchKernelGGL((dense_rows_kernel<VW, MT, 2>), dim3(blocks), dim3(kUpdateThreads), lds, stream, a);
-    else hipLaunchKernelGGL((dense_rows_kernel<VW, MT, 1>), dim3(blocks), dim3(kUpdateThreads), lds, stream, a);
+#define EPPGCN_ROWS(CU_)                                                                                                \
+    do {                                                                                                               \
+        if (a.rows) hipLaunchKernelGGL((dense_rows_kernel<VW, MT, CU_, true>), dim3(blocks), dim3(kUpdateThreads), lds, stream, a); \
+        else hipLaunchKernelGGL((dense_rows_kernel<VW, MT, CU_, false>), dim3(blocks), dim3(kUpdateThreads), lds, stream, a);       \
+    } while (0)
+    if (cu == 4) EPPGCN_ROWS(4);
+    else if (cu == 2) EPPGCN_ROWS(2);
+    else EPPGCN_ROWS(1);
+#undef EPPGCN_ROWS
     return hipGetLastError();
 }
 
