@@ -422,8 +422,8 @@ int eppgcn_update_backward(float* d_x, float* d_w, const float* x, const float* 
 /* eppgcn_update_backward for a gradient of which only some rows are defined: `rows` holds one bit per row of g
  * (bit r of word r / 32, (num_nodes + 31) / 32 words; NULL = every row, i.e. eppgcn_update_backward).  A row whose
  * bit is clear counts as zeros and is not read - neither that row of g, which may hold anything, nor the row of x
- * it would be multiplied with; its row of d_x is written as zeros.  Where the rows with clear bits do hold zeros the
- * results equal those of eppgcn_update_backward bit for bit.  d_x may be NULL (and then w): only d_w is formed (a
+ * it would be multiplied with; its row of d_x is written as zeros.  Where the rows with clear bits do hold zeros (and
+ * finite values in x) the results equal those of eppgcn_update_backward bit for bit.  d_x may be NULL (and then w): only d_w is formed (a
  * first layer whose input needs no gradient).  This is the row-masked product the reference sketches in
  * `d_weight = torch::mm(X.index({mask}).transpose(0,1), d_input_prime.index({mask}))`, EPPGCN_kernel.cu:616, taken
  * over the bitmap eppgcn_ours_backward_rows hands out instead of an index list. */
