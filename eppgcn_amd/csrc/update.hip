@@ -401,28 +401,36 @@ __global__ __launch_bounds__(kUpdateThreads) void dense_weight_kernel(float* __r
     }
 }
 
-// dw[e] = sum over blocks of partial[b][e], added in a fixed order
-__global__ __launch_bounds__(256) void reduce_partials_kernel(float* __restrict__ dw,
-                                                              const float* __restrict__ partial, int num_blocks,
-                                                              int count)
+// dw[e] = sum over blocks of partial[b][e], added in a fixed order: 16 slices of a workgroup take every 16th block
+// each (four running sums per slice), then the 16 slice sums are added as a tree
+constexpr int kReduceSlices = 16;
+__global__ __launch_bounds__(64 * kReduceSlices) void reduce_partials_kernel(float* __restrict__ dw,
+                                                                             const float* __restrict__ partial,
+                                                                             int num_blocks, int count)
 {
-    __shared__ float red[4][64];
-    const int e = blockIdx.x * 64 + threadIdx.x % 64;
+    __shared__ float red[kReduceSlices][64];
+    const int col = threadIdx.x % 64;
+    const int e = blockIdx.x * 64 + col;
     const int slice = threadIdx.x / 64;
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     if (e < count) {
         int b = slice;
-        for (; b + 12 < num_blocks; b += 16) {
+        for (; b + 3 * kReduceSlices < num_blocks; b += 4 * kReduceSlices) {
             s0 += partial[static_cast<size_t>(b) * count + e];
-            s1 += partial[static_cast<size_t>(b + 4) * count + e];
-            s2 += partial[static_cast<size_t>(b + 8) * count + e];
-            s3 += partial[static_cast<size_t>(b + 12) * count + e];
+            s1 += partial[static_cast<size_t>(b + kReduceSlices) * count + e];
+            s2 += partial[static_cast<size_t>(b + 2 * kReduceSlices) * count + e];
+            s3 += partial[static_cast<size_t>(b + 3 * kReduceSlices) * count + e];
         }
-        for (; b < num_blocks; b += 4) s0 += partial[static_cast<size_t>(b) * count + e];
+        for (; b < num_blocks; b += kReduceSlices) s0 += partial[static_cast<size_t>(b) * count + e];
     }
-    red[slice][threadIdx.x % 64] = (s0 + s1) + (s2 + s3);
+    red[slice][col] = (s0 + s1) + (s2 + s3);
     __syncthreads();
-    if (slice == 0 && e < count) dw[e] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+#pragma unroll
+    for (int half = kReduceSlices / 2; half >= 1; half /= 2) {
+        if (slice < half) red[slice][col] += red[slice + half][col];
+        __syncthreads();
+    }
+    if (slice == 0 && e < count) dw[e] = red[0][col];
 }
 
 static int weight_blocks(long long n)
@@ -477,7 +485,7 @@ int launch_dense_weight(float* dw, const float* x, int ld_x, const float* g, int
 #undef EPPGCN_W
     if (e != hipSuccess) return hip_fail(e, "dense weight kernel launch");
     const int count = K * D;
-    hipLaunchKernelGGL(reduce_partials_kernel, dim3((count + 63) / 64), dim3(256), 0, stream, dw, partial, blocks, count);
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3((count + 63) / 64), dim3(64 * kReduceSlices), 0, stream, dw, partial, blocks, count);
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }
@@ -714,7 +722,7 @@ int launch_dense_backward(float* dx, float* dw, const float* x, const float* g, 
 #undef EPPGCN_B
     EPPGCN_HIP(hipGetLastError());
     const int count = K * D;
-    hipLaunchKernelGGL(reduce_partials_kernel, dim3((count + 63) / 64), dim3(256), 0, stream, dw, a.partial, blocks, count);
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3((count + 63) / 64), dim3(64 * kReduceSlices), 0, stream, dw, a.partial, blocks, count);
     EPPGCN_HIP(hipGetLastError());
     return kOk;
 }
