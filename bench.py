@@ -20,8 +20,12 @@ can pass 1.0 (`frac_basis` says so).  The physical, bounded figure is `hbm_frac`
 (fabric-side) traffic of the same call - TCC->EA read and write requests times their sizes, from the
 committed rocprofv3 summary under profiles/, no fitted factor, used only while the kernel sources still
 hash to what was profiled - over the same time; those counters sit between L2 and the fabric and cannot
-tell the memory-side cache from HBM.  `kernel_only_frac` is the aggregation kernels alone,
-`compulsory_frac` the lower bound with perfect reuse.
+tell the memory-side cache from HBM.  By default the same counters are also read live, before anything else
+touches the GPU: two `rocprofv3 --pmc` child runs of this script's `--traffic_probe` mode (the four calls of a step,
+three times each; about 20 s per run); where that works `roofline.traffic` is the live figure and the committed
+summary is the cross-check (`traffic_committed`), where it does not (no rocprofv3, a time-out, this process itself
+running under a profiler) the committed figure is used and `traffic_source` says so.  `kernel_only_frac` is the
+aggregation kernels alone, `compulsory_frac` the lower bound with perfect reuse.
 Before anything is timed every launch is checked against the same operator without plan and
 workspace (different kernel instantiation, different summation order).
 """
@@ -87,6 +91,12 @@ def parse():
     ap.add_argument("--hip_graph", action="store_true",
                     help="also time the step replayed from a HIP graph of its four calls (removes the launch gaps that "
                          "matter on small graphs; reported as graph_ms_per_step, the headline value stays the eager step)")
+    ap.add_argument("--no_live_traffic", action="store_true",
+                    help="do not start the two rocprofv3 --pmc child runs that measure the calls' L2-miss traffic; "
+                         "roofline.traffic then comes from the committed summary under profiles/")
+    ap.add_argument("--traffic_probe", action="store_true",
+                    help="(what the rocprofv3 child runs execute) set the workload up, issue the four calls of a step "
+                         "three times each in a fixed order, print nothing, time nothing")
     ap.add_argument("--verbose", action="store_true")
     return ap.parse_args()
 
@@ -153,12 +163,110 @@ def pipeline_figures(g, wl, kernels, x16, x22, out16, out22, args):
     return fig
 
 
+# ---------------------------------------------------------------- live L2-miss traffic of the calls
+CALL_ORDER = ("fwd_agg_d16", "fwd_agg_d22", "bwd_agg_d22_last", "bwd_agg_d16_first")
+PROBE_REPS = 3
+PMC_PASSES = (("TCC_EA0_RDREQ_sum", "TCC_EA0_RDREQ_32B_sum", "TCC_EA0_RDREQ_64B_sum", "TCC_EA0_RDREQ_128B_sum"),
+              ("TCC_EA0_WRREQ_sum", "TCC_EA0_WRREQ_64B_sum"))
+# kernels of a call before its stream kernel: output clear for rows without slots, pre-scaling pass
+CALL_PROLOGUE = ("zero_words_kernel", "zero_listed_rows_kernel", "zero_rows_unless_kernel", "scale_rows", "scale_listed_rows_kernel")
+
+
+def _short_kernel_name(name):
+    return name.replace("void ", "").replace("eppgcn::", "").split("(")[0]
+
+
+def call_bytes_from_counters(csv_path, bytes_of):
+    """{call name: average of bytes_of(counters) per call} from one rocprofv3 counter_collection CSV of a
+    `--traffic_probe` run.  The probe issues the four calls in CALL_ORDER, PROBE_REPS times, and nothing else runs
+    a stream kernel, so the k-th stream-kernel dispatch belongs to call k mod 4; a call is that dispatch, the (at
+    most two) clear / pre-scaling dispatches right before it and the fix-up dispatch right after it."""
+    import csv
+    disp = {}
+    with open(csv_path, newline="") as f:
+        for r in csv.DictReader(f):
+            d = disp.setdefault(int(r["Dispatch_Id"]), [_short_kernel_name(r["Kernel_Name"]), {}])
+            d[1][r["Counter_Name"]] = d[1].get(r["Counter_Name"], 0.0) + float(r["Counter_Value"])
+    seq = [disp[k] for k in sorted(disp)]
+    at = [i for i, (name, _) in enumerate(seq) if name.startswith("aggregate_stream_kernel")]
+    if len(at) != len(CALL_ORDER) * PROBE_REPS:
+        raise RuntimeError(f"{len(at)} stream-kernel dispatches in the probe run, expected {len(CALL_ORDER) * PROBE_REPS}")
+    total = {name: 0.0 for name in CALL_ORDER}
+    for k, i in enumerate(at):
+        members = [i]
+        j = i - 1
+        while j >= 0 and i - j <= 2 and seq[j][0].startswith(CALL_PROLOGUE):
+            members.append(j)
+            j -= 1
+        if i + 1 < len(seq) and seq[i + 1][0].startswith("stream_fixup_kernel"):
+            members.append(i + 1)
+        total[CALL_ORDER[k % len(CALL_ORDER)]] += sum(bytes_of(seq[m][1]) for m in members)
+    return {name: v / PROBE_REPS for name, v in total.items()}
+
+
+def live_traffic(timeout_s=180):
+    """({call name: L2-miss bytes per call}, note) measured now: two child runs of `rocprofv3 --pmc <counters> --
+    python3 bench.py <same flags> --traffic_probe`, read requests in one, write requests in the other (one run
+    holds at most four TCC counters).  Must be called before this process touches the GPU.  (None, reason) when
+    it cannot be done; never raises."""
+    import glob
+    import shutil
+    import signal
+    import subprocess
+    import tempfile
+    if any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ) or "rocprof" in os.environ.get("LD_PRELOAD", ""):
+        return None, "this process runs under a profiler itself: no nested counter runs"
+    tool = shutil.which("rocprofv3") or os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "bin", "rocprofv3")
+    if not os.path.exists(tool):
+        return None, "rocprofv3 not found"
+    flags = [a for a in sys.argv[1:]]
+    read_b = lambda c: 32.0 * c.get("TCC_EA0_RDREQ_32B_sum", 0.0) + 64.0 * c.get("TCC_EA0_RDREQ_64B_sum", 0.0) + \
+        128.0 * c.get("TCC_EA0_RDREQ_128B_sum", 0.0)
+    write_b = lambda c: 64.0 * c.get("TCC_EA0_WRREQ_64B_sum", 0.0) + \
+        32.0 * (c.get("TCC_EA0_WRREQ_sum", 0.0) - c.get("TCC_EA0_WRREQ_64B_sum", 0.0))
+    parts = []
+    work = tempfile.mkdtemp(prefix="eppgcn_traffic_", dir="/tmp")
+    try:
+        for counters, bytes_of in zip(PMC_PASSES, (read_b, write_b)):
+            out_dir = os.path.join(work, counters[0])
+            cmd = [tool, "--pmc", *counters, "--output-format", "csv", "-d", out_dir, "-o", "run", "--",
+                   sys.executable, os.path.join(ROOT, "bench.py"), *flags, "--traffic_probe"]
+            env = dict(os.environ, TMPDIR="/tmp")
+            proc = subprocess.Popen(cmd, cwd="/tmp", env=env, stdout=subprocess.DEVNULL, stderr=subprocess.PIPE,
+                                    start_new_session=True)
+            try:
+                _, err = proc.communicate(timeout=timeout_s)
+            except subprocess.TimeoutExpired:
+                os.killpg(proc.pid, signal.SIGKILL)      # the process group this call started, nothing else
+                proc.communicate()
+                return None, f"counter run ({counters[0]} ...) exceeded {timeout_s} s and was stopped"
+            if proc.returncode != 0:
+                tail = err.decode(errors="replace").strip().splitlines()[-1:] or [""]
+                return None, f"counter run ({counters[0]} ...) ended with code {proc.returncode}: {tail[0][:200]}"
+            found = glob.glob(os.path.join(out_dir, "**", "*counter_collection.csv"), recursive=True)
+            if not found:
+                return None, "the counter run left no counter_collection.csv"
+            parts.append(call_bytes_from_counters(found[0], bytes_of))
+    except Exception as exc:               # a measurement aid must never take the benchmark down
+        return None, f"live counters failed: {exc!r}"
+    finally:
+        shutil.rmtree(work, ignore_errors=True)
+    return {name: float(round(parts[0][name] + parts[1][name])) for name in CALL_ORDER}, \
+        "measured in this run: rocprofv3 --pmc " + " ".join(PMC_PASSES[0]) + " / " + " ".join(PMC_PASSES[1]) + \
+        f" over `bench.py --traffic_probe` ({PROBE_REPS} calls each)"
+
+
 def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus must be 1 (no multi-GPU path exists).",
               file=sys.stderr)
         sys.exit(2)
+
+    # the counter runs are child processes of their own and come first: nothing in this process has touched the GPU yet
+    live, live_note = (None, "switched off (--no_live_traffic)") if (args.no_live_traffic or args.traffic_probe) \
+        else live_traffic()
+    log(args, "live traffic:", live, live_note)
 
     import torch
     from eppgcn_amd import capi, graphs, workload
@@ -242,6 +350,13 @@ def main():
         for _, fn, _ in kernels:
             fn()
 
+    if args.traffic_probe:
+        assert tuple(k[0] for k in kernels) == CALL_ORDER
+        for _ in range(PROBE_REPS):
+            step()
+        torch.cuda.synchronize()
+        return
+
     checked = None if args.no_check else check_launches(g, wl, kernels, (x16, x22, dy22, dy16), (out16, out22))
 
     for _ in range(args.warmup):
@@ -320,7 +435,12 @@ def main():
     dk = per_kernel[dominant]
     dim = 22 if "d22" in dominant else 16
     compulsory = workload.bytes_compulsory(n, e, dim)
-    traffic, traffic_note = measured_traffic(args.config, dominant)
+    committed, committed_note = measured_traffic(args.config, dominant)
+    if live is not None and all(per_kernel[k]["stream_form"] for k in per_kernel):
+        traffic, traffic_note = live[dominant], live_note
+    else:
+        traffic, traffic_note = committed, committed_note + ("" if live_note.startswith("switched off") else
+                                                              f" (live counters: {live_note})")
     sec = dk["call_ms"] * 1e-3
     roofline = {"bound": "hbm", "kernel": dominant,
                 "launch": "whole call: output clear + pre-scaling pass + stream kernel + fix-up kernel "
@@ -332,6 +452,7 @@ def main():
                               "any work being skipped (the result check covers the timed launches); the bounded "
                               "figure is hbm_frac",
                 "traffic": traffic, "traffic_source": traffic_note,
+                "traffic_committed": committed, "traffic_committed_source": committed_note,
                 "traffic_is": "L2-miss (fabric-side) bytes of the call: TCC->EA read requests x their sizes (32 / 64 / "
                               "128 B) + write requests x their sizes (32 / 64 B), rocprofv3 --pmc, no fitted factor; "
                               "the counters sit between L2 and the fabric, so a hit in the 256 MB memory-side cache "
@@ -369,9 +490,10 @@ def main():
         "result_check": checked,
         "roofline": roofline,
     }
-    traffic_epoch = [measured_traffic(args.config, k)[0] for k in per_kernel]
+    traffic_epoch = [live[k] for k in per_kernel] if traffic_note == live_note and live is not None else \
+        [measured_traffic(args.config, k)[0] for k in per_kernel]
     if all(t is not None for t in traffic_epoch):
-        # L2-miss (fabric-side) traffic of the four calls, from the same counter summary as roofline.traffic
+        # L2-miss (fabric-side) traffic of the four calls, from the same source as roofline.traffic
         result["l2_miss_traffic_bytes_per_epoch"] = sum(traffic_epoch)
         result["l2_miss_traffic_GBps"] = round(sum(traffic_epoch) / (ms_per_step * 1e-3) / 1e9, 1)
         result["l2_miss_traffic_pct_of_peak"] = round(result["l2_miss_traffic_GBps"] / PEAK_HBM_GBS * 100, 2)

@@ -165,3 +165,55 @@ def test_counter_summary_is_only_used_for_the_sources_it_was_taken_from(tmp_path
     assert value is None and "other kernel sources" in why
     (prof / "a.md").write_text("    traffic_bytes cfgX fwd = 1.5e+09\n")
     assert bench.measured_traffic("cfgX", "fwd")[0] is None
+
+
+def test_live_counter_attribution_and_guards(tmp_path, monkeypatch):
+    """bench.py's live traffic figure: the k-th stream-kernel dispatch of a `--traffic_probe` run belongs to call
+    k mod 4, together with the clear / pre-scaling dispatches right before it and the fix-up right after it; a run
+    with another number of stream-kernel dispatches is refused; no counter runs are started from a process that is
+    itself under a profiler."""
+    import csv
+    import bench
+    rows, did = [], 0
+
+    def dispatch(name, **counters):
+        nonlocal did
+        did += 1
+        for k, v in counters.items():
+            for half in (0.25, 0.75):                      # rocprofv3 writes one row per counter instance
+                rows.append({"Dispatch_Id": did, "Kernel_Name": name, "Counter_Name": k, "Counter_Value": v * half})
+
+    rd = lambda n: {"TCC_EA0_RDREQ_sum": 3 * n, "TCC_EA0_RDREQ_32B_sum": n, "TCC_EA0_RDREQ_64B_sum": n, "TCC_EA0_RDREQ_128B_sum": n}
+    dispatch("void eppgcn::plan_keys_kernel(int*)", **rd(1000))            # set-up: belongs to no call
+    dispatch("eppgcn::zero_words_kernel(unsigned int*, unsigned long)", **rd(1000))
+    dispatch("void at::native::something<float>(float*)", **rd(1000))
+    for rep in range(bench.PROBE_REPS):
+        dispatch("void eppgcn::scale_rows_flat4_kernel<unsigned int>(float*)", **rd(1))
+        dispatch("void eppgcn::aggregate_stream_kernel<0, 4, 8, false>(float*, float*)", **rd(10))
+        dispatch("void eppgcn::stream_fixup_kernel<0, 4>(float*)", **rd(100))
+        dispatch("void eppgcn::scale_rows_kernel<unsigned int>(float*)", **rd(2))
+        dispatch("void eppgcn::aggregate_stream_kernel<2, 8, 8, false>(float*, float*)", **rd(20))       # no fix-up
+        dispatch("eppgcn::zero_words_kernel(unsigned int*, unsigned long)", **rd(3))
+        dispatch("eppgcn::scale_listed_rows_kernel(float*)", **rd(3))
+        dispatch("void eppgcn::aggregate_stream_kernel<2, 8, 8, false>(float*, float*)", **rd(30))
+        dispatch("void eppgcn::stream_fixup_kernel<2, 8>(float*)", **rd(300))
+        dispatch("void eppgcn::zero_listed_rows_kernel<4>(float*)", **rd(4))
+        dispatch("eppgcn::scale_listed_rows_kernel(float*)", **rd(4))
+        dispatch("void eppgcn::aggregate_stream_kernel<0, 4, 8, false>(float*, float*)", **rd(40))
+        dispatch("void eppgcn::stream_fixup_kernel<0, 4>(float*)", **rd(400))
+    path = tmp_path / "run_counter_collection.csv"
+    with open(path, "w", newline="") as f:
+        w = csv.DictWriter(f, fieldnames=["Dispatch_Id", "Kernel_Name", "Counter_Name", "Counter_Value"])
+        w.writeheader()
+        w.writerows(rows)
+    read_b = lambda c: 32 * c["TCC_EA0_RDREQ_32B_sum"] + 64 * c["TCC_EA0_RDREQ_64B_sum"] + 128 * c["TCC_EA0_RDREQ_128B_sum"]
+    got = bench.call_bytes_from_counters(str(path), read_b)
+    assert got == {"fwd_agg_d16": 224.0 * 111, "fwd_agg_d22": 224.0 * 22, "bwd_agg_d22_last": 224.0 * 336,
+                   "bwd_agg_d16_first": 224.0 * 448}
+    with open(path, "a", newline="") as f:               # a thirteenth stream-kernel dispatch: not the probe's sequence
+        csv.writer(f).writerow([did + 1, "void eppgcn::aggregate_stream_kernel<0, 4, 8, false>(float*)", "TCC_EA0_RDREQ_sum", 1])
+    with pytest.raises(RuntimeError, match="13 stream-kernel dispatches"):
+        bench.call_bytes_from_counters(str(path), read_b)
+    monkeypatch.setenv("ROCPROFILER_LIBRARY_CTOR", "1")
+    value, why = bench.live_traffic()
+    assert value is None and "under a profiler" in why
