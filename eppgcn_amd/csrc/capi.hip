@@ -141,10 +141,12 @@ int eppgcn_spmm_backward(float* d_input, const float* d_output, const int32_t* r
                                     static_cast<hipStream_t>(stream), &g_back_agg_ms, nullptr);
 }
 
-int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
-                         const int32_t* edge_list, const float* degrees, int num_nodes, int dim, int num_parts,
-                         int part_size, int layer, int blockx, int blocky, float* workspace,
-                         size_t workspace_floats, const void* plan, const uint32_t* gathered_rows, void* stream)
+// shared by the two pruned-backward entry points; written == nullptr: the plain call (every row of d_input defined)
+static int ours_backward_call(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
+                              const int32_t* edge_list, const float* degrees, int num_nodes, int dim, int num_parts,
+                              int part_size, int layer, int blockx, int blocky, float* workspace,
+                              size_t workspace_floats, const void* plan, const uint32_t* gathered_rows,
+                              const uint32_t** written, long long* num_written, void* stream)
 {
     // part_size only sizes the work per wave (the reference's kernel ignores it, EPPGCN_kernel.cu:636)
     EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
@@ -162,7 +164,16 @@ int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* i
     return aggregate_compacted_groups(d_input, d_output, ids, part_pointer, edge_list, degrees, plan, num_nodes,
                                       dim, num_parts, part_size > 0 ? part_size : 1, workspace, workspace_floats, gathered_rows,
                                       static_cast<hipStream_t>(stream), &g_back_agg_ms,
-                                      layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr);
+                                      layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr, written, num_written);
+}
+
+int eppgcn_ours_backward(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
+                         const int32_t* edge_list, const float* degrees, int num_nodes, int dim, int num_parts,
+                         int part_size, int layer, int blockx, int blocky, float* workspace,
+                         size_t workspace_floats, const void* plan, const uint32_t* gathered_rows, void* stream)
+{
+    return ours_backward_call(d_input, d_output, ids, part_pointer, edge_list, degrees, num_nodes, dim, num_parts, part_size,
+                              layer, blockx, blocky, workspace, workspace_floats, plan, gathered_rows, nullptr, nullptr, stream);
 }
 
 int eppgcn_ours_backward_rows(float* d_input, const float* d_output, const int32_t* ids, const int32_t* part_pointer,
@@ -174,25 +185,11 @@ int eppgcn_ours_backward_rows(float* d_input, const float* d_output, const int32
     EPPGCN_REQUIRE(written_rows, "written_rows must not be NULL (eppgcn_ours_backward is the call without it)");
     *written_rows = nullptr;
     if (num_written) *num_written = num_nodes > 0 ? num_nodes : 0;
-    EPPGCN_REQUIRE(num_nodes >= 0 && dim > 0 && num_parts >= 0, "num_nodes >= 0, dim > 0, num_parts >= 0 required");
-    EPPGCN_REQUIRE(blockx > 0 && blocky > 0, "launch hints must be positive");
-    EPPGCN_REQUIRE(layer >= 1, "layer is 1-based");
-    if (num_nodes == 0) return kOk;
-    EPPGCN_REQUIRE(d_input && (d_output || workspace) && degrees, "null feature or scale pointer");
-    EPPGCN_REQUIRE(num_parts == 0 || (ids && part_pointer && edge_list), "null index pointer");
-    EPPGCN_REQUIRE(aligned(d_input, 4) && aligned(d_output, 4), "feature pointers must be 4-byte aligned");
-    EPPGCN_REQUIRE(!plan || aligned(plan, 256), "plan must be 256-byte aligned");
-    EPPGCN_REQUIRE(!workspace || (aligned(workspace, 16) && workspace != d_input),
-                   "workspace must be 16-byte aligned and distinct from the output");
-    EPPGCN_REQUIRE(!workspace || workspace == d_output || workspace_floats >= feature_workspace_floats(num_nodes, dim),
-                   "workspace smaller than eppgcn_feature_workspace_floats(num_nodes, dim)");
     long long count = num_nodes;
-    const int rc = aggregate_compacted_groups(d_input, d_output, ids, part_pointer, edge_list, degrees, plan, num_nodes,
-                                              dim, num_parts, part_size > 0 ? part_size : 1, workspace, workspace_floats,
-                                              gathered_rows, static_cast<hipStream_t>(stream), &g_back_agg_ms,
-                                              layer <= kMaxTimedLayers ? &g_layer_back_ms[layer - 1] : nullptr,
-                                              written_rows, &count);
-    if (num_written) *num_written = *written_rows ? count : num_nodes;
+    const int rc = ours_backward_call(d_input, d_output, ids, part_pointer, edge_list, degrees, num_nodes, dim, num_parts,
+                                      part_size, layer, blockx, blocky, workspace, workspace_floats, plan, gathered_rows,
+                                      written_rows, &count, stream);
+    if (rc == kOk && num_written && *written_rows) *num_written = count;
     return rc;
 }
 
