@@ -204,7 +204,7 @@ def call_bytes_from_counters(csv_path, bytes_of):
     return {name: v / PROBE_REPS for name, v in total.items()}
 
 
-def live_traffic(timeout_s=180):
+def live_traffic(timeout_s=240):
     """({call name: L2-miss bytes per call}, note) measured now: two child runs of `rocprofv3 --pmc <counters> --
     python3 bench.py <same flags> --traffic_probe`, read requests in one, write requests in the other (one run
     holds at most four TCC counters).  Must be called before this process touches the GPU.  (None, reason) when
